@@ -1,0 +1,37 @@
+"""Engine options in one place.
+
+Names and meanings follow the reference where it has them: ``block_size``
+and ``num_gpu_blocks`` (pico_vllm/blockmanager.py:21-28; run_single.py:17-22
+uses 500 blocks of 16), ``max_seq_len`` (engine.py:41), ``max_num_seqs``
+(scheduler.py:84), ``use_cuda_graph`` and ``max_batch_size`` (engine.py:21-22;
+the graph here is a HIP graph), ``manual_seed`` (engine.py:30).
+``max_num_batched_tokens`` (the token budget of a step; the reference prefills
+whole prompts, engine.py:305-306) and ``dtype`` have no counterpart there.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+
+@dataclass
+class EngineArgs:
+    model: str = ""                      # folder with config.json and model.safetensors
+    dtype: str = "bfloat16"              # "bfloat16" or "float32" (true 32-bit everywhere)
+    block_size: int = 16                 # tokens per cache page
+    num_gpu_blocks: Optional[int] = None  # pages per layer group; None: from max_num_seqs * max_seq_len
+    max_seq_len: int = 4096              # longest request (prompt + generated)
+    max_num_seqs: int = 4                # requests running at once
+    max_num_batched_tokens: int = 2048   # token budget of one step
+    use_cuda_graph: bool = True          # replay pure-decode steps from a captured HIP graph
+    max_batch_size: int = 8              # largest decode batch that has a graph
+    manual_seed: int = 42
+    device: str = "cuda:0"
+
+    def validate(self) -> None:
+        if self.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
+        if self.block_size < 8 or self.block_size % 8:
+            raise ValueError(f"block_size must be a positive multiple of 8, got {self.block_size}")
+        if self.max_num_seqs < 1 or self.max_num_batched_tokens < 1 or self.max_seq_len < 1:
+            raise ValueError("max_num_seqs, max_num_batched_tokens and max_seq_len must be positive")

@@ -1,0 +1,229 @@
+// Row-wise and element-wise kernels: embedding gather, RMSNorm with optional fused
+// residual add, SwiGLU, and rotate-half position encoding fused with the store of
+// keys and values into the paged cache.  All arithmetic is float32; T is the storage
+// type of activations (float or raw bfloat16 bits).  The residual stream is float32
+// in both engine dtypes.
+#include "common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+extern "C" const char* pico_last_error() { return g_error; }
+void pico_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+// ---------------------------------------------------------------------------
+// embedding: out[t, :] = table[ids[t], :] as float32.  An id outside [0, V) gives a
+// row of zeros (the host checks ids before a step; this only keeps the kernel in bounds).
+// Reference: nn.Embedding lookup, pico_vllm/model.py:427.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embedding_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                 float* __restrict__ out, int H, int V) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const bool ok = id >= 0 && id < V;
+  const T* row = table + (size_t)(ok ? id : 0) * H;
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ok ? load_f32(row + i) : 0.f;
+}
+
+extern "C" int pico_embedding(const void* table, int table_dtype, const int* ids, float* out, int T, int H,
+                              int V, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0 && V > 0, "pico_embedding: bad sizes T=%d H=%d V=%d", T, H, V);
+  if (T == 0) return 0;
+  if (table_dtype == PICO_DTYPE_F32)
+    embedding_kernel<float><<<T, 256, 0, stream>>>((const float*)table, ids, out, H, V);
+  else if (table_dtype == PICO_DTYPE_BF16)
+    embedding_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V);
+  else
+    PICO_REQUIRE(false, "pico_embedding: unknown dtype %d", table_dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm: y = x / sqrt(mean(x^2) + eps) * w   (pico_vllm/RMSNorm.py:22-31)
+// with the residual sum fused in front (the reference has such a kernel,
+// kernels/fused_add_norm.py:21-36, but does not call it):
+//   rows == nullptr:  resid[t] += delta[t] (if delta);  out[t] = norm(resid[t])
+//   rows != nullptr:  out[i] = norm(resid[rows[i]] + delta[rows[i]]);  resid unchanged
+// One workgroup per row.  The sum of squares is taken over the float32 sum.
+// ---------------------------------------------------------------------------
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                   const float* __restrict__ w, TO* __restrict__ out,
+                                   const int* __restrict__ rows, int H, float eps) {
+  __shared__ float scratch[16];
+  const int src = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)src * H;
+  const TD* dl = delta ? delta + (size_t)src * H : nullptr;
+  TO* o = out + (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (dl) {
+      v += load_f32(dl + i);
+      if (!rows) x[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (dl && rows) v += load_f32(dl + i);
+    store_f32(o + i, v * r * w[i]);
+  }
+}
+
+extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype, const float* w, void* out,
+                                int out_dtype, const int* rows, int T, int H, float eps, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0, "pico_add_rmsnorm: bad sizes T=%d H=%d", T, H);
+  PICO_REQUIRE(eps > 0.f, "pico_add_rmsnorm: eps must be positive");
+  if (T == 0) return 0;
+  const int threads = H >= 2048 ? 512 : 256;
+#define LAUNCH(TD, TO) \
+  add_rmsnorm_kernel<TD, TO><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H, eps)
+  if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_F32) LAUNCH(float, float);
+  else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_F32) LAUNCH(bf16_t, float);
+  else PICO_REQUIRE(false, "pico_add_rmsnorm: unknown dtypes %d %d", delta_dtype, out_dtype);
+#undef LAUNCH
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// resid[t] += delta[t] without a norm (for an arrangement that ends on an add)
+template <typename TD>
+__global__ void residual_add_kernel(float* __restrict__ resid, const TD* __restrict__ delta, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) resid[i] += load_f32(delta + i);
+}
+
+extern "C" int pico_residual_add(float* resid, const void* delta, int delta_dtype, long long n, hipStream_t stream) {
+  PICO_REQUIRE(n >= 0, "pico_residual_add: bad size");
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (delta_dtype == PICO_DTYPE_F32)
+    residual_add_kernel<float><<<blocks, 256, 0, stream>>>(resid, (const float*)delta, (size_t)n);
+  else if (delta_dtype == PICO_DTYPE_BF16)
+    residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(resid, (const bf16_t*)delta, (size_t)n);
+  else
+    PICO_REQUIRE(false, "pico_residual_add: unknown dtype %d", delta_dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU: out[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g * sigmoid(g)
+// (pico_vllm/kernels/swiglu.py:22-41: gate is the first half of the last dim).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t row = idx / I, col = idx % I;
+  const float g = load_f32(gu + row * 2 * (size_t)I + col);
+  const float u = load_f32(gu + row * 2 * (size_t)I + I + col);
+  const float s = g / (1.0f + expf(-g));
+  store_f32(out + idx, s * u);
+}
+
+extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && I > 0, "pico_swiglu: bad sizes T=%d I=%d", T, I);
+  if (T == 0) return 0;
+  const size_t total = (size_t)T * I;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == PICO_DTYPE_F32)
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+  else if (dtype == PICO_DTYPE_BF16)
+    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+  else
+    PICO_REQUIRE(false, "pico_swiglu: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Rotate-half position encoding of q and k, fused with the store of k and v into the
+// paged cache (pico_vllm/kernels/fused_rope_kvcache_store.py:51-101 does this for decode
+// only; prefill there uses eager RoPE, model.py:99-124, plus kernels/store_kvcache.py).
+//   pair (j, j + rot/2), angle = position * inv_freq[j] in float32:
+//     out[j]         = x[j] * cos - x[j + rot/2] * sin
+//     out[j + rot/2] = x[j + rot/2] * cos + x[j] * sin
+//   entries at index >= rot pass through unrotated.
+// qkv: [T, (nq + 2 nkv) * d], rows [q heads | k heads | v heads]; q is rotated in place.
+// Cache of one layer: K pages [page][kv head][slot in page][d],
+//                     V pages [page][kv head][d][slot in page]  (slot contiguous).
+// A token at position p of sequence s goes to page block_table[s][p / P], slot p % P.
+// Grid (T, nq + nkv); block 64.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                  const int* __restrict__ token_seq, const int* __restrict__ block_table,
+                                  int max_pages, const float* __restrict__ inv_freq, T* __restrict__ k_cache,
+                                  T* __restrict__ v_cache, int nq, int nkv, int d, int rot, int P,
+                                  int num_pages) {
+  const int t = blockIdx.x, head = blockIdx.y;
+  const int pos = positions[t];
+  T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
+  const int half = rot >> 1;
+  if (head < nq) {
+    T* x = row + (size_t)head * d;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      const float ang = (float)pos * inv_freq[j];
+      const float c = cosf(ang), s = sinf(ang);
+      const float a = load_f32(x + j), b = load_f32(x + j + half);
+      store_f32(x + j, a * c - b * s);
+      store_f32(x + j + half, b * c + a * s);
+    }
+    return;
+  }
+  const int g = head - nq;
+  const int page = block_table[(size_t)token_seq[t] * max_pages + pos / P];
+  if (page < 0 || page >= num_pages) return;  // the host has checked; stay in bounds regardless
+  const int off = pos % P;
+  const T* k = row + (size_t)(nq + g) * d;
+  const T* v = row + (size_t)(nq + nkv + g) * d;
+  T* kc = k_cache + (((size_t)page * nkv + g) * P + off) * d;
+  T* vc = v_cache + ((size_t)page * nkv + g) * d * P + off;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const float ang = (float)pos * inv_freq[j];
+    const float c = cosf(ang), s = sinf(ang);
+    const float a = load_f32(k + j), b = load_f32(k + j + half);
+    store_f32(kc + j, a * c - b * s);
+    store_f32(kc + j + half, b * c + a * s);
+  }
+  for (int j = rot + threadIdx.x; j < d; j += blockDim.x) kc[j] = k[j];
+  for (int j = threadIdx.x; j < d; j += blockDim.x) vc[(size_t)j * P] = v[j];
+}
+
+extern "C" int pico_rope_kv_store(void* qkv, int dtype, const int* positions, const int* token_seq,
+                                  const int* block_table, int max_pages, const float* inv_freq, void* k_cache,
+                                  void* v_cache, int T, int nq, int nkv, int d, int rot, int P, int num_pages,
+                                  hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && d > 0 && P > 0 && max_pages > 0 && num_pages > 0,
+               "pico_rope_kv_store: bad sizes");
+  PICO_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "pico_rope_kv_store: rotary size %d does not fit head size %d", rot, d);
+  if (T == 0) return 0;
+  dim3 grid(T, nq + nkv);
+  if (dtype == PICO_DTYPE_F32)
+    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, positions, token_seq, block_table, max_pages,
+                                                      inv_freq, (float*)k_cache, (float*)v_cache, nq, nkv, d, rot,
+                                                      P, num_pages);
+  else if (dtype == PICO_DTYPE_BF16)
+    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, positions, token_seq, block_table, max_pages,
+                                                       inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, nq, nkv, d,
+                                                       rot, P, num_pages);
+  else
+    PICO_REQUIRE(false, "pico_rope_kv_store: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,130 @@
+// Sampling from float32 logits, one workgroup per row, with per-row parameters:
+//   temperature == 0        argmax, lowest index on a tie            (pico_vllm/sampler.py:8)
+//   top_p >= 1              draw from softmax(logits / T)             (sampler.py:16-17)
+//   top_p <  1              keep the tokens whose preceding cumulative mass, in descending
+//                           order of probability, is < top_p (the token that crosses stays),
+//                           renormalise, draw                          (sampler.py:25-36)
+// The draw is the inverse CDF in vocabulary order at the uniform number u[row] that the
+// host supplies (the reference calls torch.multinomial; only the distribution is shared).
+// The kept set of top-p is found without sorting: with e_i = exp((x_i - max) / T) and
+// f(t) = sum of e_i > t, the kept tokens are those with e_i >= t*, t* being the smallest
+// float with f(t*) < top_p * sum(e); t* comes from bisection over the float's bit pattern.
+// All sums run in a fixed order, so a row's result depends on its inputs only.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+__device__ __forceinline__ float masked_sum(const float* __restrict__ x, int V, float mx, float inv_t, float thr,
+                                            bool inclusive, float* scratch) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < V; i += SAMPLE_THREADS) {
+    const float e = expf((x[i] - mx) * inv_t);
+    if (inclusive ? (e >= thr) : (e > thr)) s += e;
+  }
+  return block_sum(s, scratch);
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, int ld, int V,
+                                                                const float* __restrict__ temperature,
+                                                                const float* __restrict__ top_p,
+                                                                const float* __restrict__ u, int* __restrict__ out) {
+  __shared__ float scratch[16];
+  __shared__ float part[SAMPLE_THREADS];
+  __shared__ int idx_scratch[16];
+  __shared__ int chosen_chunk;
+  __shared__ float chosen_before;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * ld;
+  const float temp = temperature[row];
+
+  // max and its first index
+  float mx = -INFINITY;
+  int mi = 0x7fffffff;
+  for (int i = tid; i < V; i += SAMPLE_THREADS) {
+    const float v = x[i];
+    if (v > mx || (v == mx && i < mi)) { mx = v; mi = i; }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(mx, off, 64);
+    const int oi = __shfl_xor(mi, off, 64);
+    if (ov > mx || (ov == mx && oi < mi)) { mx = ov; mi = oi; }
+  }
+  if ((tid & 63) == 0) { scratch[tid >> 6] = mx; idx_scratch[tid >> 6] = mi; }
+  __syncthreads();
+  mx = scratch[0]; mi = idx_scratch[0];
+  for (int w = 1; w < SAMPLE_THREADS / 64; w++) {
+    const float ov = scratch[w]; const int oi = idx_scratch[w];
+    if (ov > mx || (ov == mx && oi < mi)) { mx = ov; mi = oi; }
+  }
+  __syncthreads();
+  if (!(temp > 0.f)) {
+    if (tid == 0) out[row] = mi;
+    return;
+  }
+  const float inv_t = 1.0f / temp;
+  const float tp = top_p[row];
+  float thr = 0.f;  // keep e >= thr
+  if (tp < 1.0f) {
+    const float total = masked_sum(x, V, mx, inv_t, -1.f, false, scratch);
+    const float target = tp * total;
+    uint32_t lo = 0u, hi = 0x3f800000u;  // f(lo) >= target, f(hi) = 0 < target
+    while (hi - lo > 1u) {
+      const uint32_t mid = lo + (hi - lo) / 2u;
+      const float f = masked_sum(x, V, mx, inv_t, __uint_as_float(mid), false, scratch);
+      if (f < target) hi = mid; else lo = mid;
+    }
+    thr = __uint_as_float(hi);
+  }
+  // inverse CDF over the kept tokens in vocabulary order; thread i owns a contiguous chunk
+  const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int b = min(tid * chunk, V), e_ = min(b + chunk, V);
+  float s = 0.f;
+  for (int i = b; i < e_; i++) {
+    const float e = expf((x[i] - mx) * inv_t);
+    if (e >= thr) s += e;
+  }
+  part[tid] = s;
+  __syncthreads();
+  if (tid == 0) {
+    float kept = 0.f;
+    for (int i = 0; i < SAMPLE_THREADS; i++) kept += part[i];
+    const float target = u[row] * kept;
+    float run = 0.f;
+    int c = -1, last_nonzero = 0;
+    float before_last = 0.f;
+    for (int i = 0; i < SAMPLE_THREADS; i++) {
+      if (part[i] > 0.f) { last_nonzero = i; before_last = run; }
+      if (run + part[i] > target) { c = i; break; }
+      run += part[i];
+    }
+    if (c < 0) { c = last_nonzero; run = before_last; }
+    chosen_chunk = c;
+    chosen_before = run;
+    scratch[0] = target;
+  }
+  __syncthreads();
+  if (tid == chosen_chunk) {
+    const float target = scratch[0];
+    float run = chosen_before;
+    int pick = -1, last_kept = mi;
+    for (int i = b; i < e_; i++) {
+      const float e = expf((x[i] - mx) * inv_t);
+      if (e >= thr) {
+        last_kept = i;
+        run += e;
+        if (run > target) { pick = i; break; }
+      }
+    }
+    out[row] = pick >= 0 ? pick : last_kept;
+  }
+}
+
+extern "C" int pico_sample(const float* logits, int ld, int R, int V, const float* temperature, const float* top_p,
+                           const float* u, int* out, hipStream_t stream) {
+  PICO_REQUIRE(R >= 0 && V > 0 && ld >= V, "pico_sample: bad sizes R=%d V=%d ld=%d", R, V, ld);
+  if (R == 0) return 0;
+  sample_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, top_p, u, out);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,143 @@
+"""One step's batch: from (request, its next tokens, wanted places) on the host
+to the flat arrays on the device that the parts read.
+
+All integer arrays of a step travel in one pinned buffer and one copy.  The
+reference builds five tensors per decode step from Python lists and refills a
+[B, 8192] block table (pico_vllm/engine.py:146-181,198-220).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..parts.base import StepContext
+
+
+@dataclass
+class SeqStep:
+    """One request's share of a step: its next ``tokens`` (they follow the
+    ``num_cached`` tokens already in the cache) and ``want``, the places among
+    these tokens whose logits are asked for."""
+    req: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class BatchError(ValueError):
+    pass
+
+
+class BatchBuffers:
+    """Pinned host and device int32 buffers of fixed capacity, reused every step."""
+
+    def __init__(self, device: torch.device, max_tokens: int, max_seqs: int, max_pages: int, num_groups: int,
+                 max_want: Optional[int] = None):
+        self.device = device
+        self.max_tokens, self.max_seqs, self.max_pages, self.num_groups = max_tokens, max_seqs, max_pages, num_groups
+        self.max_want = max_want if max_want is not None else max_tokens
+        n = 3 * max_tokens + (max_seqs + 1) + 2 * max_seqs + self.max_want + num_groups * max_seqs * max_pages
+        self.host = torch.zeros(n, dtype=torch.int32, pin_memory=torch.cuda.is_available())
+        self.dev = torch.zeros(n, dtype=torch.int32, device=device)
+        self.copied = torch.cuda.Event() if torch.cuda.is_available() else None
+
+
+def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers, act_dtype: torch.dtype,
+                  vocab_size: int, pad_to: Optional[int] = None) -> StepContext:
+    """Pack ``seqs`` into ``buf`` and describe the device views.
+
+    ``pad_to``: pad a pure-decode batch with empty rows up to that many
+    sequences (for replaying a graph captured at that size); a padded row has a
+    block table of -1, so nothing is written for it, and its output is ignored.
+    """
+    B = len(seqs)
+    if B == 0:
+        raise BatchError("a step needs at least one sequence")
+    rows = max(B, pad_to or 0)
+    lens = [len(s.tokens) for s in seqs]
+    if min(lens) < 1:
+        raise BatchError("every sequence of a step brings at least one token")
+    T = sum(lens) + (rows - B)
+    R = sum(len(s.want) for s in seqs) + (rows - B if pad_to else 0)
+    P = manager.page_size
+    if T > buf.max_tokens or rows > buf.max_seqs or R > buf.max_want:
+        raise BatchError(f"step of {T} tokens / {rows} sequences / {R} wanted rows exceeds the buffers "
+                         f"({buf.max_tokens} / {buf.max_seqs} / {buf.max_want})")
+    G = len(manager.groups)
+    if buf.copied is not None:
+        buf.copied.synchronize()          # the previous step's copy has left the pinned buffer
+    h = buf.host.numpy()
+    h_tok, h_pos, h_seq = h[0:T], h[buf.max_tokens:buf.max_tokens + T], h[2 * buf.max_tokens:2 * buf.max_tokens + T]
+    o = 3 * buf.max_tokens
+    h_cu = h[o:o + rows + 1]; o += buf.max_seqs + 1
+    h_ctx = h[o:o + rows]; o += buf.max_seqs
+    h_slot = h[o:o + rows]; o += buf.max_seqs
+    h_want = h[o:o + R]; o += buf.max_want
+    bt_off = o
+    max_ctx = 1
+    need_pages = 1
+    t = 0
+    r = 0
+    h_cu[0] = 0
+    for b, s in enumerate(seqs):
+        n = lens[b]
+        cached = manager.num_computed(s.req)
+        toks = np.asarray(s.tokens, dtype=np.int64)
+        if toks.min() < 0 or toks.max() >= vocab_size:
+            raise BatchError(f"request {s.req!r}: token id outside [0, {vocab_size})")
+        h_tok[t:t + n] = toks
+        h_pos[t:t + n] = np.arange(cached, cached + n)
+        h_seq[t:t + n] = b
+        for w in s.want:
+            if not 0 <= w < n:
+                raise BatchError(f"request {s.req!r}: wanted place {w} is outside its {n} tokens")
+            h_want[r] = t + w
+            r += 1
+        t += n
+        h_cu[b + 1] = t
+        h_ctx[b] = cached + n
+        h_slot[b] = manager.slot(s.req)
+        max_ctx = max(max_ctx, cached + n)
+        need_pages = max(need_pages, -(-(cached + n) // P))
+    for b in range(B, rows):                       # padding rows of a captured decode batch
+        h_tok[t] = 0; h_pos[t] = 0; h_seq[t] = b
+        h_want[r] = t; r += 1
+        t += 1
+        h_cu[b + 1] = t
+        h_ctx[b] = 0
+        h_slot[b] = 0
+    width = buf.max_pages if pad_to else need_pages
+    if width > buf.max_pages:
+        raise BatchError(f"a sequence needs {width} pages, the buffers hold {buf.max_pages} per sequence")
+    tables = h[bt_off:bt_off + G * rows * width].reshape(G, rows, width)
+    tables[:] = -1
+    for b, s in enumerate(seqs):
+        need = -(-int(h_ctx[b]) // P)
+        for g in range(G):
+            table = manager.block_table(s.req, g)
+            if len(table) < need:
+                raise BatchError(f"request {s.req!r}: {need} pages are needed, {len(table)} are allocated")
+            tables[g, b, :need] = table[:need]
+    used = bt_off + G * rows * width
+    buf.dev[:used].copy_(buf.host[:used], non_blocking=True)
+    if buf.copied is not None:
+        buf.copied.record()
+    d = buf.dev
+    o = 3 * buf.max_tokens
+    ctx = StepContext(
+        num_tokens=T, num_seqs=rows,
+        token_ids=d[0:T], positions=d[buf.max_tokens:buf.max_tokens + T],
+        token_seq=d[2 * buf.max_tokens:2 * buf.max_tokens + T],
+        cu_seqlens=d[o:o + rows + 1],
+        context_lens=d[o + buf.max_seqs + 1:o + buf.max_seqs + 1 + rows],
+        state_slots=d[o + 2 * buf.max_seqs + 1:o + 2 * buf.max_seqs + 1 + rows],
+        want_rows=d[o + 3 * buf.max_seqs + 1:o + 3 * buf.max_seqs + 1 + R],
+        block_tables=[d[bt_off + g * rows * width:bt_off + (g + 1) * rows * width].view(rows, width) for g in range(G)],
+        act_dtype=act_dtype,
+        max_new_tokens=max(lens), max_context=max_ctx, all_decode=max(lens) == 1,
+        host={"cu_seqlens": h_cu.copy(), "context_lens": h_ctx.copy()},
+    )
+    return ctx

@@ -1,0 +1,155 @@
+"""The engine and its Python entry point.
+
+In the manner of the reference's entry script (pico_vllm/run_single.py:10-37:
+build the model, load weights, make the block manager and the engine, then
+``submit`` and loop ``step()`` until done): ``LLMEngine.submit`` /
+``step`` / ``is_done`` have the reference's names and meanings
+(engine.py:243,282,465); ``LLM.generate`` wraps the loop.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple, Union
+
+import torch
+
+from ..config.engine_args import EngineArgs
+from ..parts.model import DecoderModel, load_model
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .batch import SeqStep
+from .request import Request, RequestStatus
+from .scheduler import Scheduler
+from .step import ModelRunner
+
+
+@dataclass
+class RequestOutput:
+    request_id: int
+    prompt_token_ids: List[int]
+    token_ids: List[int]
+    finish_reason: str
+    text: Optional[str] = None
+    num_preemptions: int = 0
+
+
+class LLMEngine:
+    def __init__(self, args: EngineArgs, model: Optional[DecoderModel] = None, tokenizer=None):
+        args.validate()
+        if not torch.cuda.is_available():
+            raise RuntimeError("pico_vllm_amd runs on an AMD GPU only; no GPU is visible to torch")
+        self.args = args
+        self.model = model if model is not None else load_model(args.model, args.dtype, args.device)
+        num_pages = args.num_gpu_blocks
+        if num_pages is None:
+            num_pages = args.max_num_seqs * (-(-args.max_seq_len // args.block_size))
+        self.runner = ModelRunner(self.model, args.block_size, num_pages, args.max_num_seqs,
+                                  args.max_num_batched_tokens, args.max_seq_len,
+                                  use_graph=args.use_cuda_graph, max_graph_batch=args.max_batch_size)
+        self.scheduler = Scheduler(self.runner.manager, args.max_num_seqs, args.max_num_batched_tokens,
+                                   args.max_seq_len)
+        self.sampler = Sampler(self.model.device, args.max_num_seqs)
+        self.eos_token_id = self.model.spec.eos_token_id
+        self.tokenizer = tokenizer
+        self._next_id = 0
+        self.requests: Dict[int, Request] = {}
+        self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+
+    # ---- the reference's trio -------------------------------------------
+    def submit(self, prompt: Union[str, Sequence[int]], max_new_tokens: int = 16, temperature: float = 0.0,
+               top_p: float = 1.0, seed: Optional[int] = None, ignore_eos: bool = False) -> int:
+        """Queue a request; returns its id (pico_vllm/engine.py:243-276)."""
+        params = SamplingParams(max_new_tokens, temperature, top_p, seed, ignore_eos)
+        params.validate()
+        ids = self._encode(prompt)
+        V = self.model.spec.vocab_size
+        if any(not 0 <= t < V for t in ids):
+            raise ValueError(f"prompt holds a token id outside [0, {V})")
+        rid = self._next_id
+        self._next_id += 1
+        req = Request(rid, list(ids), params, seed=seed if seed is not None else self.args.manual_seed * 1000003 + rid)
+        self.scheduler.add_request(req)
+        self.requests[rid] = req
+        return rid
+
+    def step(self) -> List[RequestOutput]:
+        """One scheduling decision and one model step; returns the requests that finished in it."""
+        plan = self.scheduler.schedule()
+        self.stats["preemptions"] += len(plan.preempted)
+        if not plan.seqs:
+            if self.scheduler.has_unfinished():
+                raise RuntimeError("the scheduler found nothing to run although requests are unfinished")
+            return []
+        seqs = []
+        for s in plan.seqs:
+            r = s.request
+            toks = r.all_ids[r.num_computed:r.num_computed + s.num_tokens]
+            seqs.append(SeqStep(r.request_id, toks, [s.num_tokens - 1] if s.samples else []))
+        logits = self.runner.step(seqs)
+        sampling = [s for s in plan.seqs if s.samples]
+        new_tokens = self.sampler.sample(
+            logits,
+            [s.request.params.temperature for s in sampling], [s.request.params.top_p for s in sampling],
+            [s.request.seed for s in sampling], [len(s.request.generated_ids) for s in sampling])
+        done: List[RequestOutput] = []
+        for s in plan.seqs:
+            self.scheduler.on_step_done(s)
+            self.stats["decode_tokens" if s.num_tokens == 1 and s.request.generated_ids else "prefill_tokens"] += s.num_tokens
+        for s, tok in zip(sampling, new_tokens):
+            r = s.request
+            r.generated_ids.append(int(tok))
+            reason = None
+            # the end-of-sequence token is kept in the output (pico_vllm/engine.py:380-385)
+            if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
+                reason = "eos"
+            elif r.is_max_len_finished():
+                reason = "length"
+            if reason:
+                self.scheduler.finish(r, reason)
+                done.append(self._output(r))
+        self.stats["steps"] += 1
+        return done
+
+    def is_done(self) -> bool:
+        return not self.scheduler.has_unfinished()
+
+    # ---- helpers --------------------------------------------------------
+    def _encode(self, prompt) -> List[int]:
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer; pass token ids or give the engine a tokenizer")
+            return list(self.tokenizer.encode(prompt))
+        return [int(t) for t in prompt]
+
+    def _output(self, r: Request) -> RequestOutput:
+        text = None
+        if self.tokenizer is not None:
+            text = self.tokenizer.decode(r.input_ids + r.generated_ids)     # prompt + generated, engine.py:385
+        return RequestOutput(r.request_id, list(r.input_ids), list(r.generated_ids), r.finish_reason or "",
+                             text, r.num_preemptions)
+
+
+class LLM:
+    """``LLM(model=DIR, dtype=...).generate(prompts, sampling_params)``."""
+
+    def __init__(self, model: str = "", tokenizer=None, engine_args: Optional[EngineArgs] = None, **kw):
+        args = engine_args or EngineArgs(model=model, **kw)
+        if model:
+            args.model = model
+        self.engine = LLMEngine(args, tokenizer=tokenizer)
+
+    def generate(self, prompts: Sequence[Union[str, Sequence[int]]],
+                 sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[RequestOutput]:
+        if sampling_params is None:
+            sampling_params = SamplingParams()
+        if isinstance(sampling_params, SamplingParams):
+            sampling_params = [sampling_params] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt, or one for all")
+        ids = [self.engine.submit(p, sp.max_new_tokens, sp.temperature, sp.top_p, sp.seed, sp.ignore_eos)
+               for p, sp in zip(prompts, sampling_params)]
+        outs: Dict[int, RequestOutput] = {}
+        while not self.engine.is_done():
+            for o in self.engine.step():
+                outs[o.request_id] = o
+        return [outs[i] for i in ids]

@@ -1,0 +1,105 @@
+"""The step function: run one batch of (request, its next tokens) through the
+model from the cache and return the logits at the wanted places.
+
+There is one step for every mixture of prompt portions and single decode
+tokens.  The reference has no such function: it prefills each request alone
+and whole (pico_vllm/engine.py:299-357) and then decodes all decoding requests
+together (:403-410) through two different model entry points.
+
+A pure-decode step whose batch fits ``max_batch_size`` replays a HIP graph
+captured for its size (the reference captures one CUDA graph at a fixed batch
+of 8, engine.py:98-137).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.storage import CacheStorage
+from ..parts.model import DecoderModel
+from .batch import BatchBuffers, BatchError, SeqStep, build_context
+
+
+def _bucket(n: int) -> int:
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, page_size: int, num_pages: int, max_seqs: int,
+                 max_tokens_per_step: int, max_seq_len: int, use_graph: bool = False, max_graph_batch: int = 8):
+        self.model = model
+        self.device = model.device
+        specs = model.cache_specs()
+        self.manager = CacheManager(specs, page_size, num_pages, max_seqs)
+        self.storage = CacheStorage(self.manager, specs, model.dtype, self.device)
+        self.max_pages = -(-max_seq_len // page_size)
+        self.max_seq_len = max_seq_len
+        self.buffers = BatchBuffers(self.device, max_tokens_per_step, max_seqs, self.max_pages,
+                                    max(1, len(self.manager.groups)))
+        self.use_graph = use_graph
+        self.max_graph_batch = max_graph_batch
+        self._graphs: Dict[int, tuple] = {}
+        self.steps = 0
+        self.tokens = 0
+
+    # ---- one step -------------------------------------------------------
+    def step(self, seqs: List[SeqStep]) -> torch.Tensor:
+        """Logits float32 [wanted, vocab] in the order of ``seqs`` and their ``want``.
+
+        Pages for the new tokens must have been allocated (``manager.grow``);
+        afterwards the caller records the new lengths (``manager.advance``)."""
+        for s in seqs:
+            if self.manager.num_computed(s.req) + len(s.tokens) > self.max_seq_len:
+                raise BatchError(f"request {s.req!r} would grow beyond max_seq_len={self.max_seq_len}")
+        decode_only = all(len(s.tokens) == 1 and list(s.want) == [0] for s in seqs)
+        if self.use_graph and decode_only and len(seqs) <= self.max_graph_batch:
+            logits = self._step_graph(seqs)
+        else:
+            ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size)
+            logits = self.model.forward(ctx, self.storage)
+        self.steps += 1
+        self.tokens += sum(len(s.tokens) for s in seqs)
+        return logits
+
+    def advance(self, seqs: List[SeqStep]) -> None:
+        for s in seqs:
+            self.manager.advance(s.req, self.manager.num_computed(s.req) + len(s.tokens))
+
+    # ---- graph replay of decode steps -----------------------------------
+    def _step_graph(self, seqs: List[SeqStep]) -> torch.Tensor:
+        B = len(seqs)
+        size = _bucket(B)
+        if size not in self._graphs:
+            self._capture(size, seqs)
+        graph, out = self._graphs[size]
+        build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size, pad_to=size)
+        graph.replay()
+        return out[:B]
+
+    def _capture(self, size: int, seqs: List[SeqStep]) -> None:
+        """Warm up on the real batch (which also writes this step's keys; the replay
+        that follows writes the same values again), then record the graph."""
+        ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
+                            pad_to=size)
+        ctx.max_context = self.max_seq_len          # kernel choices must hold for every later replay
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                self.model.forward(ctx, self.storage)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self.model.forward(ctx, self.storage)
+        self._graphs[size] = (graph, out)
+
+    # ---- sizes for reports ----------------------------------------------
+    def decode_bytes(self, context_lens: List[int]) -> int:
+        """Bytes a decode step has to read: every weight once and the cache of the live requests."""
+        return self.model.num_weight_bytes() + self.storage.bytes_per_token() * sum(context_lens)

@@ -1,0 +1,255 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that shapes, dtypes and layouts are what the
+kernel and its grid assume, then launches on torch's current stream.  Tensors
+must live on the GPU; there is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+c_int, c_float, c_void_p, c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"dtype {t.dtype} is not supported by the kernels (float32 or bfloat16)") from None
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("the kernels run on the GPU only; got a CPU tensor")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(lib, code: int) -> None:
+    if code != 0:
+        lib.pico_last_error.restype = ctypes.c_char_p
+        raise KernelError(lib.pico_last_error().decode())
+
+
+def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{name} must be a contiguous int32 tensor")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name} has {t.numel()} entries, {n} are needed")
+
+
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = table[ids[t]] as float32 rows (the residual stream)."""
+    _gpu(table, ids)
+    V, H = table.shape
+    T = ids.numel()
+    _i32(ids, "ids")
+    if not table.is_contiguous():
+        raise KernelError("embedding table must be contiguous")
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    elif out.shape != (T, H) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise KernelError("embedding: out must be a contiguous float32 [T, H] tensor")
+    lib = library.core()
+    _check(lib, lib.pico_embedding(_ptr(table), _dt(table), _ptr(ids), _ptr(out), T, H, V, _stream()))
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """rows is None: resid += delta (if given), returns norm(resid).
+    rows given: returns norm(resid[rows] + delta[rows]); resid is left alone."""
+    _gpu(resid, delta, weight, rows)
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    if weight.dtype != torch.float32 or weight.shape != (H,) or not weight.is_contiguous():
+        raise KernelError(f"norm weight must be float32 of shape [{H}]")
+    if delta is not None and (delta.shape != resid.shape or not delta.is_contiguous()):
+        raise KernelError("delta must be contiguous and shaped like the residual stream")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    if out is None:
+        out = torch.empty(n, H, dtype=out_dtype, device=resid.device)
+    elif out.shape != (n, H) or out.dtype != out_dtype or not out.is_contiguous():
+        raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
+    lib = library.core()
+    ddt = _dt(delta) if delta is not None else F32
+    _check(lib, lib.pico_add_rmsnorm(_ptr(resid), _ptr(delta), ddt, _ptr(weight), _ptr(out), _DT[out_dtype],
+                                     _ptr(rows), n, H, c_float(eps), _stream()))
+    return out
+
+
+def residual_add(resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _gpu(resid, delta)
+    if resid.dtype != torch.float32 or not resid.is_contiguous() or delta.shape != resid.shape \
+            or not delta.is_contiguous():
+        raise KernelError("residual_add: float32 contiguous residual and an equally shaped contiguous delta")
+    lib = library.core()
+    _check(lib, lib.pico_residual_add(_ptr(resid), _ptr(delta), _dt(delta), c_ll(resid.numel()), _stream()))
+    return resid
+
+
+def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _gpu(gate_up)
+    T, I2 = gate_up.shape
+    if I2 % 2 or not gate_up.is_contiguous():
+        raise KernelError("swiglu: input must be contiguous [T, 2 I]")
+    I = I2 // 2
+    if out is None:
+        out = torch.empty(T, I, dtype=gate_up.dtype, device=gate_up.device)
+    elif out.shape != (T, I) or out.dtype != gate_up.dtype or not out.is_contiguous():
+        raise KernelError("swiglu: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_swiglu(_ptr(gate_up), _ptr(out), _dt(gate_up), T, I, _stream()))
+    return out
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 out = a @ w.T + bias with plain FMA.  a: [M, K] float32 or bfloat16 (rows may be
+    strided), w: [N, K] float32."""
+    _gpu(a, w, bias)
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise KernelError(f"gemm: inner sizes differ ({K} and {K2})")
+    if w.dtype != torch.float32 or w.stride(1) != 1 or a.stride(1) != 1:
+        raise KernelError("gemm_f32: w must be float32 and both operands contiguous along K")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (N,) or not bias.is_contiguous()):
+        raise KernelError("gemm_f32: bias must be contiguous float32 [N]")
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=a.device)
+    elif out.shape != (M, N) or out.dtype != torch.float32 or out.stride(1) != 1:
+        raise KernelError("gemm_f32: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_gemm_f32(_ptr(a), _dt(a), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
+                                  a.stride(0) if M > 1 else K, w.stride(0), out.stride(0) if M > 1 else N, _stream()))
+    return out
+
+
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              out_dtype: torch.dtype = torch.bfloat16, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = a @ w.T + bias on the matrix cores; a [M, K], w [N, K] bfloat16, bias float32,
+    out float32 or bfloat16."""
+    _gpu(a, w, bias)
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise KernelError(f"gemm: inner sizes differ ({K} and {K2})")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError("gemm_bf16: operands must be bfloat16 and contiguous along K")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (N,) or not bias.is_contiguous()):
+        raise KernelError("gemm_bf16: bias must be contiguous float32 [N]")
+    if out is None:
+        out = torch.empty(M, N, dtype=out_dtype, device=a.device)
+    elif out.shape != (M, N) or out.dtype != out_dtype or out.stride(1) != 1:
+        raise KernelError("gemm_bf16: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_gemm_bf16(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _DT[out_dtype], M, N, K,
+                                   a.stride(0) if M > 1 else K, w.stride(0), out.stride(0) if M > 1 else N,
+                                   _stream()))
+    return out
+
+
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int):
+    """K pages [pages, nkv, P, d]; V pages [pages, nkv, d, P]."""
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("cache tensors must be contiguous and 4-dimensional")
+    pages, h, P, dd = k_cache.shape
+    if (h, dd) != (nkv, d) or tuple(v_cache.shape) != (pages, nkv, d, P) or v_cache.dtype != k_cache.dtype:
+        raise KernelError(f"cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                          f"{nkv} kv heads of size {d}")
+    return pages, P
+
+
+def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
+                  inv_freq: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, nq: int, nkv: int, d: int,
+                  rotary_dim: int) -> None:
+    """Rotate q (in place) and k, write k and v of every token into its page."""
+    _gpu(qkv, positions, token_seq, block_table, inv_freq, k_cache, v_cache)
+    T = qkv.shape[0]
+    if qkv.shape != (T, (nq + 2 * nkv) * d) or not qkv.is_contiguous():
+        raise KernelError(f"qkv must be contiguous [T, {(nq + 2 * nkv) * d}], got {tuple(qkv.shape)}")
+    pages, P = _check_cache(k_cache, v_cache, nkv, d)
+    if k_cache.dtype != qkv.dtype:
+        raise KernelError("cache and activations differ in dtype")
+    _i32(positions, "positions", T)
+    _i32(token_seq, "token_seq", T)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2 or not inv_freq.is_contiguous():
+        raise KernelError("inv_freq must be float32 of rotary_dim / 2 entries")
+    lib = library.core()
+    _check(lib, lib.pico_rope_kv_store(_ptr(qkv), _dt(qkv), _ptr(positions), _ptr(token_seq), _ptr(block_table),
+                                       block_table.shape[1], _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), T, nq,
+                                       nkv, d, rotary_dim, P, pages, _stream()))
+
+
+def paged_attention_ref(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                        positions: torch.Tensor, token_seq: torch.Tensor, nq: int, nkv: int, d: int,
+                        scale: float, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q: [T, >= nq*d] (row stride free, heads first in the row); returns [T, nq*d]."""
+    _gpu(q, k_cache, v_cache, block_table, positions, token_seq)
+    T = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < nq * d:
+        raise KernelError("q must be [T, >= nq*d] with unit stride along the row")
+    pages, P = _check_cache(k_cache, v_cache, nkv, d)
+    if k_cache.dtype != q.dtype:
+        raise KernelError("cache and activations differ in dtype")
+    _i32(positions, "positions", T)
+    _i32(token_seq, "token_seq", T)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+    if out is None:
+        out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
+    elif out.shape != (T, nq * d) or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError("attention: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_paged_attention_ref(_ptr(q), q.stride(0) if T > 1 else q.shape[1], _dt(q), _ptr(k_cache),
+                                             _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                                             _ptr(positions), _ptr(token_seq), _ptr(out), T, nq, nkv, d, P, window,
+                                             c_float(scale), pages, _stream()))
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, u: torch.Tensor,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token id per row of float32 logits; per-row temperature (0 = greedy), top_p and
+    uniform number."""
+    _gpu(logits, temperature, top_p, u)
+    R, V = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be float32 with unit stride along the vocabulary")
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("u", u)):
+        if t.dtype != torch.float32 or t.numel() < R or not t.is_contiguous():
+            raise KernelError(f"sample: {name} must be contiguous float32 with one entry per row")
+    if out is None:
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    elif out.dtype != torch.int32 or out.numel() < R or not out.is_contiguous():
+        raise KernelError("sample: out must be contiguous int32 with one entry per row")
+    lib = library.core()
+    _check(lib, lib.pico_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature),
+                                _ptr(top_p), _ptr(u), _ptr(out), _stream()))
+    return out

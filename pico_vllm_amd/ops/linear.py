@@ -1,0 +1,42 @@
+"""y = x W^T (+ b) with W stored [out, in] as in the checkpoint.
+
+bfloat16 weights: the library GEMM (hipBLASLt through torch), as the
+reference uses the library for every projection (pico_vllm/model.py:200,225,
+316,318); a float32 result (logits) comes from the matrix-core kernel of this
+package.  float32 weights: this package's plain-FMA kernel, never a library
+call, so the 32-bit engine has no reduced-precision matrix mode anywhere; if
+the activations are bfloat16 (a tensor stored in 32 bit inside a bfloat16
+engine) they are widened on load and the result is rounded once.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import kernels
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
+        if weight.dim() != 2:
+            raise ValueError("a linear weight is a matrix")
+        self.weight = weight.contiguous()
+        self.bias = None if bias is None else bias.to(self.weight.dtype).contiguous()
+        self.bias_f32 = None if bias is None else bias.float().contiguous()
+        self.out_features, self.in_features = weight.shape
+
+    def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        out_dtype = out_dtype or x.dtype
+        if x.shape[-1] != self.in_features:
+            raise ValueError(f"linear: input has {x.shape[-1]} features, the weight wants {self.in_features}")
+        if self.weight.dtype == torch.float32:
+            y = kernels.gemm_f32(x, self.weight, self.bias_f32)
+            return y if out_dtype == torch.float32 else y.to(out_dtype)
+        if x.dtype != torch.bfloat16:
+            raise ValueError("linear: bfloat16 weights need bfloat16 activations")
+        if out_dtype == torch.float32:
+            return kernels.gemm_bf16(x, self.weight, self.bias_f32, torch.float32)
+        if self.bias is not None:
+            return torch.addmm(self.bias, x, self.weight.t())
+        return torch.mm(x, self.weight.t())

@@ -1,0 +1,79 @@
+"""Grouped-query attention over the paged cache."""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from ..ops import kernels
+from ..ops.linear import Linear
+from .base import Mixer, StepContext
+from .registry import build_part, register_part
+from .spec import CacheSpec, ParamSpec, PartSpec
+
+
+@register_part("mixer", "gqa_attention")
+class GQAAttention(Mixer):
+    """qkv = x Wqkv^T (+ b); position encoding on q, k; k, v into the cache;
+    attention of every new token over its request's cache; o = a Wo^T.
+
+    Order and shapes follow pico_vllm/model.py:187-228 (fused qkv with bias
+    :148-152, rows [q; k; v] :42-43 of weights.py, o_proj without bias :147).
+    Keys and values of the new tokens are written first and attention then
+    reads old and new alike from the cache (model.py:216-221), which is what
+    makes a prompt cut into portions equal the whole prompt.  The checkpoint
+    holds q_proj, k_proj and v_proj separately; they are concatenated at load.
+    ``window`` > 0 restricts every query to the last ``window`` keys."""
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 qkv_bias: bool, position: PartSpec, window: int = 0,
+                 act_dtype: torch.dtype = torch.bfloat16):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size, self.nq, self.nkv, self.d = hidden_size, num_heads, num_kv_heads, head_dim
+        self.qkv_bias, self.window, self.act_dtype = qkv_bias, window, act_dtype
+        self.scale = 1.0 / math.sqrt(head_dim)          # pico_vllm/kernels/attention.py:92,231
+        self.position = build_part("position", position, act_dtype=act_dtype)
+        self.qkv: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+        self.fast = None                                # matrix-core kernels, chosen at load
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec("paged_kv", num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
+
+    def param_specs(self) -> List[ParamSpec]:
+        H, nq, nkv, d = self.hidden_size, self.nq, self.nkv, self.d
+        out = [ParamSpec("q_proj.weight", (nq * d, H)), ParamSpec("k_proj.weight", (nkv * d, H)),
+               ParamSpec("v_proj.weight", (nkv * d, H)), ParamSpec("o_proj.weight", (H, nq * d))]
+        if self.qkv_bias:
+            out += [ParamSpec("q_proj.bias", (nq * d,), role="bias"), ParamSpec("k_proj.bias", (nkv * d,), role="bias"),
+                    ParamSpec("v_proj.bias", (nkv * d,), role="bias")]
+        return out + [ParamSpec("position." + p.name, p.shape, p.role, p.std) for p in self.position.param_specs()]
+
+    def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
+        ws = [tensors[f"{n}_proj.weight"] for n in "qkv"]
+        wdt = torch.float32 if any(w.dtype == torch.float32 for w in ws) else ws[0].dtype
+        w = torch.cat([t.to(wdt) for t in ws], dim=0).to(device)
+        b = None
+        if self.qkv_bias:
+            b = torch.cat([tensors[f"{n}_proj.bias"].float() for n in "qkv"], dim=0).to(device)
+        self.qkv = Linear(w, b)
+        self.o = Linear(tensors["o_proj.weight"].to(device))
+        self.position.load({k[len("position."):]: v for k, v in tensors.items() if k.startswith("position.")},
+                           device, dtype)
+        if self.act_dtype == torch.bfloat16:
+            from ..ops import attention_fast
+            self.fast = attention_fast.choose(self.nq, self.nkv, self.d, self.window)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
+        nq, nkv, d = self.nq, self.nkv, self.d
+        bt = ctx.block_tables[cache.group]
+        qkv = self.qkv(x)                                         # [T, (nq + 2 nkv) d]
+        self.position.rotate_and_store(qkv, ctx, cache, bt, nq, nkv, d)
+        if self.fast is not None and cache.k.dtype == torch.bfloat16:
+            a = self.fast(qkv, cache, bt, ctx, self.scale)
+        else:
+            a = kernels.paged_attention_ref(qkv, cache.k, cache.v, bt, ctx.positions, ctx.token_seq,
+                                            nq, nkv, d, self.scale, self.window)
+        return self.o(a)

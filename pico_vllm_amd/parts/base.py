@@ -1,0 +1,106 @@
+"""Interfaces of the parts a layer is made of.
+
+A part is built from the constants in its ``PartSpec`` (sizes, eps, theta,
+flags); it never sees a model configuration and does not know which model it
+is in.  Parts can be constructed without a GPU: ``param_specs`` only needs the
+constants.  ``load`` receives the part's CPU tensors by name (relative to the
+part's prefix) and puts what it needs on the device; ``forward`` runs on the
+GPU.
+
+Interfaces:
+  Norm.add_norm(resid, delta, rows=None) -> normed
+  PositionEncoding.rotate_and_store(qkv, ctx, kv, block_table, nq, nkv, d)
+  Mixer.cache_spec() -> CacheSpec;  Mixer.forward(x, ctx, cache) -> y
+  FeedForward.forward(x, ctx) -> y
+  Block.forward(resid, pending, ctx, cache) -> (resid, pending)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+import torch
+
+from .spec import CacheSpec, ParamSpec
+
+
+@dataclass
+class StepContext:
+    """What one step gives every part: the flattened batch on the device.
+
+    Tokens of all sequences lie one after the other ([T] arrays); sequence b
+    owns tokens cu_seqlens[b] .. cu_seqlens[b+1]."""
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor          # int32 [T]
+    positions: torch.Tensor          # int32 [T]   absolute position of each token in its request
+    token_seq: torch.Tensor          # int32 [T]   row of the token's sequence in the per-sequence arrays
+    cu_seqlens: torch.Tensor         # int32 [B+1]
+    context_lens: torch.Tensor       # int32 [B]   cached + new tokens
+    state_slots: torch.Tensor        # int32 [B]   slot of fixed-size state
+    block_tables: List[torch.Tensor]  # per cache group: int32 [B, max_pages]
+    want_rows: torch.Tensor          # int32 [R]   flat token indices whose logits are wanted
+    act_dtype: torch.dtype
+    # host-side facts for choosing kernels (fixed at capture time under a graph)
+    max_new_tokens: int = 1          # longest portion in the batch
+    max_context: int = 1             # longest context in the batch
+    all_decode: bool = False         # every sequence brings exactly one token
+    host: Dict[str, Any] = field(default_factory=dict)   # numpy copies of the arrays above
+
+
+class Part:
+    """Common to all parts: declared tensors and loading."""
+
+    def param_specs(self) -> List[ParamSpec]:
+        return []
+
+    def load(self, tensors: Dict[str, torch.Tensor], device: torch.device, dtype: torch.dtype) -> None:
+        pass
+
+
+class Norm(Part):
+    def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """resid (float32 [T, H]) += delta, returns the normed rows in the activation dtype;
+        with ``rows`` only those rows are produced and resid is left unchanged."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotate_and_store(self, qkv: torch.Tensor, ctx: StepContext, kv, block_table: torch.Tensor,
+                         nq: int, nkv: int, d: int) -> None:
+        """Encode positions into q (in place) and k, and write k, v into the pages of ``kv``."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec("none")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
+        """x: normed activations [T, H]; cache: this run's cache entry
+        (``cache.storage.PagedKVLayer`` or ``StateLayer`` or None); returns [T, H]."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of parts.  ``slot_categories`` names its slots and the
+    registry category each is built from."""
+    slot_categories: Dict[str, str] = {}
+
+    def __init__(self, parts: Dict[str, Part]):
+        self.parts = parts
+
+    @property
+    def mixer(self) -> Mixer:
+        return self.parts["mixer"]
+
+    def forward(self, resid: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext, cache):
+        """resid: float32 residual stream; pending: a delta not yet added to it
+        (or None).  Returns (resid, pending) for the next block."""
+        raise NotImplementedError

@@ -1,0 +1,47 @@
+"""Rotate-half rotary position encoding."""
+from __future__ import annotations
+
+import torch
+
+from ..ops import kernels
+from .base import PositionEncoding
+from .registry import register_part
+
+
+@register_part("position", "rotary_half")
+class RotaryHalf(PositionEncoding):
+    """Pairs (j, j + rotary_dim/2) are rotated by position * theta^(-2j/rotary_dim)
+    (pico_vllm/model.py:80-86,116-123).  Angles, cosines and sines are float32
+    and are computed inside the kernel from the position, so there is no table
+    whose length bounds the sequence (the reference keeps a [131072, d] table)."""
+
+    def __init__(self, rotary_dim: int, theta: float, act_dtype: torch.dtype = torch.bfloat16):
+        if rotary_dim % 2:
+            raise ValueError(f"rotary_dim must be even, got {rotary_dim}")
+        self.rotary_dim, self.theta = rotary_dim, theta
+        self.inv_freq = None
+
+    def load(self, tensors, device, dtype) -> None:
+        d = self.rotary_dim
+        # same float32 arithmetic as pico_vllm/model.py:80-82
+        inv = 1.0 / (self.theta ** (torch.arange(0, d, 2).float() / d))
+        self.inv_freq = inv.to(device).contiguous()
+
+    def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
+        kernels.rope_kv_store(qkv, ctx.positions, ctx.token_seq, block_table, self.inv_freq,
+                              kv.k, kv.v, nq, nkv, d, self.rotary_dim)
+
+
+@register_part("position", "none")
+class NoPosition(PositionEncoding):
+    """No position encoding: keys and values are stored as they are."""
+
+    def __init__(self, act_dtype: torch.dtype = torch.bfloat16):
+        self._empty = None
+
+    def load(self, tensors, device, dtype) -> None:
+        self._empty = torch.zeros(0, dtype=torch.float32, device=device)
+
+    def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
+        kernels.rope_kv_store(qkv, ctx.positions, ctx.token_seq, block_table, self._empty,
+                              kv.k, kv.v, nq, nkv, d, 0)

@@ -1,0 +1,96 @@
+"""Descriptions of a model as data: which parts each layer is made of, with
+which constants, in which order the layers run and whose cache each run reads.
+
+Nothing here touches a device.  An architecture turns its typed configuration
+into a ``ModelSpec``; ``parts.model.DecoderModel`` builds the runnable parts
+from it through the part registries in ``parts.registry``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Tuple
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A part chosen by name with its sizes and constants."""
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor a part wants from the checkpoint.
+
+    ``role`` decides the dtype it is kept in and how random weights draw it:
+      matrix  - bfloat16 (float32 in the 32-bit engine, or if stored in 32 bit); N(0, std)
+      bias    - like matrix; N(0, std)
+      norm    - float32 always; 1 + U(-0.1, 0.1)
+      table   - int32 integer table; zeros
+    """
+    name: str
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    std: float = 0.02
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """What a mixer keeps per request between steps.
+
+    kind "paged_kv": keys and values of ``num_kv_heads`` x ``head_dim`` per
+    token in pages; ``window`` > 0 means only the last ``window`` positions
+    are ever read again, so older pages can be given back early.
+    kind "state": a fixed-size tensor of ``state_shape`` per request.
+    kind "none": nothing.
+    """
+    kind: str = "none"
+    num_kv_heads: int = 0
+    head_dim: int = 0
+    window: int = 0
+    state_shape: Tuple[int, ...] = ()
+    state_dtype: str = "float32"
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer: an arrangement (``block``) whose slots are filled with
+    parts.  ``slots`` maps a slot name of the arrangement (for the pre-norm
+    block: norm1, mixer, norm2, ff) to (sub-prefix of the part's tensors in
+    the checkpoint, the part).  ``prefix`` is the layer's own prefix."""
+    prefix: str
+    block: str
+    slots: Dict[str, Tuple[str, PartSpec]]
+
+
+@dataclass(frozen=True)
+class RunEntry:
+    """One entry of the run order: run ``layer`` (an index into ``layers``; a
+    layer may be named by several entries, which then share its weights).
+    Every entry owns a cache of its own unless ``cache_of`` names an EARLIER
+    entry of the run order, whose cache this run's mixer is then given."""
+    layer: int
+    cache_of: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    embed_name: str
+    layers: List[LayerSpec]
+    run_order: List[RunEntry]
+    final_norm: PartSpec
+    final_norm_name: str
+    head_name: Optional[str]          # None: output matrix is the embedding matrix
+    eos_token_id: Optional[int] = None
+    max_position: int = 131072
+
+    def cache_id(self, entry_index: int) -> int:
+        """The run entry whose cache entry ``entry_index`` uses."""
+        e = self.run_order[entry_index]
+        return entry_index if e.cache_of is None else e.cache_of
+
+    def cache_owners(self) -> List[int]:
+        """Run entries that own a cache."""
+        return [i for i, e in enumerate(self.run_order) if e.cache_of is None]

@@ -1,0 +1,60 @@
+"""Sampling one token per row of logits on the GPU.
+
+Strategy per row as in pico_vllm/sampler.py:40-88 (greedy / temperature /
+temperature with top-p), but in one kernel launch with per-row parameters
+instead of one torch call per group of equal parameters.  Randomness comes from
+a counter-based generator on the host: the uniform number of a draw depends
+only on (seed, index of the token in its request), so a request samples the
+same tokens whatever else is in the batch.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from ..ops import kernels
+
+_MASK = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    z = x
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
+def uniform(seed: int, index: int) -> float:
+    """A number in [0, 1) with 24 random bits, a pure function of (seed, index)."""
+    z = _splitmix64(_splitmix64(seed & _MASK) ^ ((index * 0xD6E8FEB86659FD93) & _MASK))
+    return (z >> 40) / float(1 << 24)
+
+
+class Sampler:
+    def __init__(self, device: torch.device, max_rows: int):
+        self.device = device
+        self.max_rows = max_rows
+        self._host = torch.zeros(3, max_rows, dtype=torch.float32, pin_memory=torch.cuda.is_available())
+        self._dev = torch.zeros(3, max_rows, dtype=torch.float32, device=device)
+        self._out = torch.zeros(max_rows, dtype=torch.int32, device=device)
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
+               seeds: Sequence[int], indices: Sequence[int]) -> List[int]:
+        """logits: float32 [R, V]; one (temperature, top_p, seed, token index) per row."""
+        R = logits.shape[0]
+        if not (len(temperatures) == len(top_ps) == len(seeds) == len(indices) == R):
+            raise ValueError("one set of sampling parameters per row of logits is needed")
+        if R > self.max_rows:
+            raise ValueError(f"{R} rows to sample, the sampler was made for {self.max_rows}")
+        if R == 0:
+            return []
+        h = self._host
+        for i in range(R):
+            h[0, i] = temperatures[i]
+            h[1, i] = top_ps[i]
+            h[2, i] = uniform(seeds[i], indices[i]) if temperatures[i] > 0 else 0.0
+        self._dev.copy_(h, non_blocking=True)
+        kernels.sample(logits, self._dev[0], self._dev[1], self._dev[2], self._out)
+        return self._out[:R].tolist()      # the one device-to-host sync of a step

@@ -1,0 +1,260 @@
+"""Plain, slow, whole-sequence implementation of the Qwen2 dense decoder.
+
+Written from the formulas of the reference (paths below are relative to the
+reference checkout, ``pico_vllm/...``).  One function per part, float32
+everywhere, no cache, no batching, no code shared with the engine.  It is the
+oracle every engine test compares against.
+
+Two places differ from the reference on purpose, both documented where they
+occur: rotation tables stay in float32 (the reference's tables become bfloat16
+only because the whole module is cast, run_single.py:13), and an untied model
+multiplies by ``lm_head.weight`` (the reference always multiplies by the
+embedding matrix, model.py:445, even when ``tie_word_embeddings`` is false).
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+from safetensors import safe_open
+
+
+# --------------------------------------------------------------------------
+# configuration and weights (read with the safetensors package, not with the
+# engine's own reader)
+# --------------------------------------------------------------------------
+@dataclass
+class PlainConfig:
+    vocab_size: int
+    hidden_size: int
+    num_hidden_layers: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    intermediate_size: int
+    rms_norm_eps: float
+    rope_theta: float
+    tie_word_embeddings: bool
+    head_dim: int
+
+
+def read_config(model_dir: str) -> PlainConfig:
+    """Field names are the reference dataclass's (model.py:16-26); head_dim
+    defaults to hidden/heads (model.py:37-38)."""
+    with open(os.path.join(model_dir, "config.json")) as f:
+        c = json.load(f)
+    hd = c.get("head_dim") or c["hidden_size"] // c["num_attention_heads"]
+    return PlainConfig(
+        vocab_size=c["vocab_size"], hidden_size=c["hidden_size"],
+        num_hidden_layers=c["num_hidden_layers"],
+        num_attention_heads=c["num_attention_heads"],
+        num_key_value_heads=c["num_key_value_heads"],
+        intermediate_size=c["intermediate_size"],
+        rms_norm_eps=c["rms_norm_eps"], rope_theta=c["rope_theta"],
+        tie_word_embeddings=c["tie_word_embeddings"], head_dim=hd)
+
+
+def read_weights(model_dir: str) -> Dict[str, torch.Tensor]:
+    """Every tensor as float32, by its name in the file (weights.py:10-15)."""
+    out: Dict[str, torch.Tensor] = {}
+    for name in sorted(os.listdir(model_dir)):
+        if name.endswith(".safetensors"):
+            with safe_open(os.path.join(model_dir, name), framework="pt", device="cpu") as st:
+                for key in st.keys():
+                    out[key] = st.get_tensor(key).float()
+    return out
+
+
+# --------------------------------------------------------------------------
+# parts
+# --------------------------------------------------------------------------
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """y = x * 1/sqrt(mean(x^2) + eps) * w   (RMSNorm.py:22-31; eager twin
+    model.py:63-66).  eps sits inside the square root; the weight multiplies
+    (it is not 1+w)."""
+    x = x.float()
+    var = (x * x).sum(dim=-1, keepdim=True) / x.shape[-1]
+    return x * (1.0 / torch.sqrt(var + eps)) * weight.float()
+
+
+def rope_tables(positions: torch.Tensor, head_dim: int, theta: float):
+    """cos/sin rows for the given absolute positions (model.py:80-90).
+
+    f_j = 1 / theta^(2j/d), j < d/2; angle = p * f_j in float32; each table
+    row is the half-row repeated twice."""
+    freqs = 1.0 / (theta ** (torch.arange(0, head_dim, 2).float() / head_dim))
+    angles = torch.outer(positions.float(), freqs)
+    cos = torch.cat([angles.cos(), angles.cos()], dim=-1)
+    sin = torch.cat([angles.sin(), angles.sin()], dim=-1)
+    return cos, sin
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x: [S, heads, d]; cos/sin: [S, d].  x*cos + rotate_half(x)*sin with
+    rotate_half(x) = [-x2, x1], the halves being the first and last d/2
+    entries (model.py:116-123).  So pairs are (j, j + d/2)."""
+    half = x.shape[-1] // 2
+    x1, x2 = x[..., :half], x[..., half:]
+    rot = torch.cat([-x2, x1], dim=-1)
+    return x * cos[:, None, :] + rot * sin[:, None, :]
+
+
+def split_qkv(qkv: torch.Tensor, n_q: int, n_kv: int, d: int):
+    """Rows of the fused projection are [q; k; v] (weights.py:42-43), split
+    into sizes [nq*d, nkv*d, nkv*d] and viewed per head (model.py:205-208)."""
+    q, k, v = qkv.split([n_q * d, n_kv * d, n_kv * d], dim=-1)
+    S = qkv.shape[0]
+    return q.reshape(S, n_q, d), k.reshape(S, n_kv, d), v.reshape(S, n_kv, d)
+
+
+def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                     q_positions: Optional[torch.Tensor] = None,
+                     window: int = 0) -> torch.Tensor:
+    """q: [M, nq, d]; k, v: [N, nkv, d]; returns [M, nq, d].
+
+    Query head h reads KV head h // (nq/nkv) (kernels/attention.py:31,139).
+    Scores (q.k) * d^-0.5 (attention.py:92,231); key n is visible to the
+    query at absolute position p iff n <= p (attention.py:193-197); softmax
+    over visible keys; weighted sum of V.  Without q_positions the M queries
+    are the last M of the N positions (tests/test_prefill_paged_attn.py:38-44).
+    ``window`` > 0 additionally hides keys with n <= p - window (not in the
+    reference; used only for the windowed-attention part test)."""
+    M, nq, d = q.shape
+    N, nkv, _ = k.shape
+    G = nq // nkv
+    if q_positions is None:
+        q_positions = torch.arange(N - M, N)
+    scale = 1.0 / math.sqrt(d)
+    out = torch.empty(M, nq, d, dtype=torch.float32)
+    k_pos = torch.arange(N)
+    visible = k_pos[None, :] <= q_positions[:, None]
+    if window > 0:
+        visible &= k_pos[None, :] > (q_positions[:, None] - window)
+    for h in range(nq):
+        g = h // G
+        s = (q[:, h, :].float() @ k[:, g, :].float().T) * scale
+        s = s.masked_fill(~visible, float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        out[:, h, :] = p @ v[:, g, :].float()
+    return out
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """gate = first half, up = second half of the last dim (weights.py:58);
+    out = gate * sigmoid(gate) * up  (kernels/swiglu.py:36-41, model.py:318)."""
+    I = gate_up.shape[-1] // 2
+    gate, up = gate_up[..., :I].float(), gate_up[..., I:].float()
+    return gate * torch.sigmoid(gate) * up
+
+
+def attention_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
+                    cfg: PlainConfig, positions: torch.Tensor) -> torch.Tensor:
+    """qkv = h W^T + b with bias on q, k, v only (model.py:148-152); RoPE on
+    q and k (model.py:211); attention; o_proj without bias (model.py:147,225)."""
+    nq, nkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    W = torch.cat([w[f"{prefix}.self_attn.q_proj.weight"],
+                   w[f"{prefix}.self_attn.k_proj.weight"],
+                   w[f"{prefix}.self_attn.v_proj.weight"]], dim=0)
+    b = torch.cat([w[f"{prefix}.self_attn.q_proj.bias"],
+                   w[f"{prefix}.self_attn.k_proj.bias"],
+                   w[f"{prefix}.self_attn.v_proj.bias"]], dim=0)
+    qkv = h @ W.T + b
+    q, k, v = split_qkv(qkv, nq, nkv, d)
+    cos, sin = rope_tables(positions, d, cfg.rope_theta)
+    q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+    o = causal_attention(q, k, v, q_positions=positions - positions[0])
+    return o.reshape(h.shape[0], nq * d) @ w[f"{prefix}.self_attn.o_proj.weight"].T
+
+
+def mlp_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str) -> torch.Tensor:
+    """down( swiglu( h [gate; up]^T ) ), no biases (model.py:309-318)."""
+    Wgu = torch.cat([w[f"{prefix}.mlp.gate_proj.weight"], w[f"{prefix}.mlp.up_proj.weight"]], dim=0)
+    return swiglu(h @ Wgu.T) @ w[f"{prefix}.mlp.down_proj.weight"].T
+
+
+def block(x: torch.Tensor, w: Dict[str, torch.Tensor], i: int, cfg: PlainConfig,
+          positions: torch.Tensor) -> torch.Tensor:
+    """x += attn(norm1(x)); x += ffn(norm2(x))   (model.py:361-374)."""
+    p = f"model.layers.{i}"
+    x = x + attention_layer(rms_norm(x, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps),
+                            w, p, cfg, positions)
+    x = x + mlp_layer(rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], cfg.rms_norm_eps), w, p)
+    return x
+
+
+def forward(tokens: Sequence[int], w: Dict[str, torch.Tensor], cfg: PlainConfig,
+            first_position: int = 0) -> torch.Tensor:
+    """Logits [S, V] for one whole sequence (model.py:427-445): embedding,
+    L blocks, final norm, output matrix.  Tied models multiply by the
+    embedding matrix; untied ones by lm_head.weight (our deliberate
+    difference, see the module docstring)."""
+    ids = torch.as_tensor(list(tokens), dtype=torch.long)
+    x = w["model.embed_tokens.weight"][ids].float()
+    positions = torch.arange(first_position, first_position + len(ids))
+    for i in range(cfg.num_hidden_layers):
+        x = block(x, w, i, cfg, positions)
+    x = rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps)
+    out_w = w["model.embed_tokens.weight"] if cfg.tie_word_embeddings else w["lm_head.weight"]
+    return x @ out_w.float().T
+
+
+class PlainModel:
+    """A model folder read once; ``logits(tokens)`` runs the whole sequence."""
+
+    def __init__(self, model_dir: str):
+        self.cfg = read_config(model_dir)
+        self.w = read_weights(model_dir)
+
+    def logits(self, tokens: Sequence[int]) -> torch.Tensor:
+        with torch.no_grad():
+            return forward(tokens, self.w, self.cfg)
+
+    def greedy(self, prompt: Sequence[int], n: int) -> List[int]:
+        toks = list(prompt)
+        out: List[int] = []
+        for _ in range(n):
+            t = int(torch.argmax(self.logits(toks)[-1]))
+            out.append(t)
+            toks.append(t)
+        return out
+
+
+# --------------------------------------------------------------------------
+# sampling
+# --------------------------------------------------------------------------
+def sample_greedy(logits: torch.Tensor) -> int:
+    """argmax (sampler.py:8); the first index wins a tie."""
+    return int(torch.argmax(logits.float()))
+
+
+def temperature_probs(logits: torch.Tensor, temperature: float) -> torch.Tensor:
+    """softmax(logits / T)  (sampler.py:16)."""
+    return torch.softmax(logits.double() / temperature, dim=-1)
+
+
+def top_p_probs(logits: torch.Tensor, temperature: float, top_p: float) -> torch.Tensor:
+    """Sort descending, drop entries whose preceding cumulative mass is
+    >= top_p (so the first token that crosses is kept), renormalise
+    (sampler.py:25-32).  Returned in vocabulary order."""
+    probs = temperature_probs(logits, temperature)
+    sp, si = torch.sort(probs, descending=True)
+    cum = torch.cumsum(sp, dim=-1)
+    sp = sp.masked_fill(cum - sp >= top_p, 0.0)
+    sp = sp / sp.sum()
+    out = torch.zeros_like(probs)
+    out[si] = sp
+    return out
+
+
+def inverse_cdf(probs: torch.Tensor, u: float) -> int:
+    """Smallest index whose cumulative probability exceeds u * total: how the
+    engine turns one uniform number into a draw from ``probs`` (the reference
+    draws with torch.multinomial, sampler.py:17, which fixes only the
+    distribution)."""
+    cum = torch.cumsum(probs.double(), dim=-1)
+    idx = int(torch.searchsorted(cum, torch.tensor(u * float(cum[-1]), dtype=torch.float64), right=True))
+    nz = torch.nonzero(probs > 0).flatten()
+    return min(max(idx, int(nz[0])), int(nz[-1]))

@@ -1,0 +1,184 @@
+"""Configuration, registry, safetensors reading and the loader's errors (no GPU)."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+from safetensors import safe_open
+from safetensors.torch import save_file
+
+from pico_vllm_amd.config import (ConfigError, EngineArgs, Qwen2Config, known_architectures,
+                                  load_model_description, resolve_architecture)
+from pico_vllm_amd.parts.model import model_param_specs
+from pico_vllm_amd.parts.spec import ParamSpec
+from pico_vllm_amd.weights.loader import WeightsError, load_checkpoint
+from pico_vllm_amd.weights.random_init import write_random_model
+from pico_vllm_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
+from tiny_configs import CONFIGS, TINY_A, TINY_B, TINY_C, model_dir
+
+
+def test_config_reads_every_key_and_has_no_size_defaults():
+    for raw in CONFIGS.values():
+        cfg = Qwen2Config.from_dict(raw)
+        for k in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads", "num_key_value_heads",
+                  "intermediate_size", "rms_norm_eps", "rope_theta", "tie_word_embeddings"):
+            assert getattr(cfg, k) == raw[k]
+        assert cfg.head_dim == raw.get("head_dim", raw["hidden_size"] // raw["num_attention_heads"])
+    for k in ("vocab_size", "hidden_size", "num_hidden_layers", "intermediate_size", "rms_norm_eps", "rope_theta",
+              "tie_word_embeddings", "num_key_value_heads"):
+        bad = dict(TINY_A)
+        del bad[k]
+        with pytest.raises(ConfigError, match=k):
+            Qwen2Config.from_dict(bad)
+
+
+@pytest.mark.parametrize("patch,word", [
+    ({"num_key_value_heads": 3}, "multiple"), ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"use_sliding_window": True}, "sliding"), ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"),
+    ({"hidden_size": 66}, "head_dim"), ({"head_dim": 15}, "even"), ({"attention_bias": False}, "bias"),
+    ({"vocab_size": 0}, "vocab_size"),
+])
+def test_config_rejects_what_the_engine_cannot_run(patch, word):
+    with pytest.raises(ConfigError, match=word):
+        Qwen2Config.from_dict({**TINY_A, **patch})
+
+
+def test_registry_resolves_by_name_and_lists_known_names():
+    assert "Qwen2ForCausalLM" in known_architectures()
+    assert resolve_architecture(TINY_A).name == "Qwen2ForCausalLM"
+    with pytest.raises(ConfigError, match="Qwen2ForCausalLM"):
+        resolve_architecture({**TINY_A, "architectures": ["LlamaForCausalLM"]})
+    with pytest.raises(ConfigError, match="architectures"):
+        resolve_architecture({k: v for k, v in TINY_A.items() if k != "architectures"})
+
+
+def test_spec_is_data_layer_by_layer():
+    _, cfg, spec = load_model_description(model_dir("B"))
+    assert len(spec.layers) == 3 and [e.layer for e in spec.run_order] == [0, 1, 2]
+    attn = spec.layers[1].slots["mixer"][1]
+    assert attn.kind == "gqa_attention" and attn.params["num_kv_heads"] == 3 and attn.params["head_dim"] == 32
+    assert attn.params["position"].params["theta"] == 1e6
+    assert spec.layers[0].slots["norm1"][1].params["eps"] == 1e-5
+    assert spec.head_name == "lm_head.weight"
+    names = {p.name for p in model_param_specs(spec)}
+    assert "model.layers.2.self_attn.k_proj.bias" in names and "model.layers.0.mlp.gate_proj.weight" in names
+    assert "lm_head.weight" in names and "model.norm.weight" in names
+    _, _, spec_a = load_model_description(model_dir("A"))
+    assert spec_a.head_name is None and "lm_head.weight" not in {p.name for p in model_param_specs(spec_a)}
+
+
+def test_engine_args_validate():
+    EngineArgs(model="x").validate()
+    with pytest.raises(ValueError):
+        EngineArgs(dtype="float16").validate()
+    with pytest.raises(ValueError):
+        EngineArgs(block_size=12).validate()
+
+
+# ---- safetensors -----------------------------------------------------------
+def test_own_reader_agrees_with_the_safetensors_package(tmp_path):
+    t = {"a": torch.randn(3, 5), "b": torch.randn(7).to(torch.bfloat16), "c": torch.arange(6, dtype=torch.int32)}
+    save_file(t, str(tmp_path / "x.safetensors"))
+    with SafetensorsFile(str(tmp_path / "x.safetensors")) as sf:
+        assert set(sf.entries) == set(t)
+        for k, v in t.items():
+            assert torch.equal(sf.tensor(k), v) and sf.tensor(k).dtype == v.dtype
+
+
+def test_own_writer_is_read_by_the_safetensors_package(tmp_path):
+    t = {"w": torch.randn(4, 6).to(torch.bfloat16), "n": torch.rand(6)}
+    write_safetensors(str(tmp_path / "y.safetensors"), [(k, tuple(v.shape), v.dtype) for k, v in t.items()],
+                      lambda name: t[name])
+    with safe_open(str(tmp_path / "y.safetensors"), framework="pt") as f:
+        assert set(f.keys()) == set(t)
+        for k in t:
+            assert torch.equal(f.get_tensor(k), t[k])
+
+
+def test_random_model_is_seeded_and_typed():
+    a1, a2, b = model_dir("A", 0), model_dir("A", 0), model_dir("A", 1)
+    with SafetensorsFile(os.path.join(a1, "model.safetensors")) as f1, \
+            SafetensorsFile(os.path.join(b, "model.safetensors")) as f2:
+        q1, q2 = f1.tensor("model.layers.0.self_attn.q_proj.weight"), f2.tensor("model.layers.0.self_attn.q_proj.weight")
+        assert q1.dtype == torch.bfloat16 and not torch.equal(q1, q2)
+        n = f1.tensor("model.norm.weight")
+        assert n.dtype == torch.float32 and float(n.min()) >= 0.9 and float(n.max()) <= 1.1
+    assert json.load(open(os.path.join(a1, "config.json")))["vocab_size"] == 256
+    assert a1 == a2
+
+
+def test_random_model_distributions(tmp_path):
+    d = write_random_model(str(tmp_path / "m"), TINY_B, seed=3)
+    with SafetensorsFile(os.path.join(d, "model.safetensors")) as f:
+        w = f.tensor("model.layers.1.mlp.gate_proj.weight").float()
+        assert abs(float(w.std()) - 0.02) < 0.002 and abs(float(w.mean())) < 0.001
+        b = f.tensor("model.layers.1.self_attn.q_proj.bias").float()
+        assert abs(float(b.std()) - 0.02) < 0.006
+
+
+# ---- loader ----------------------------------------------------------------
+def _specs(name):
+    return model_param_specs(load_model_description(model_dir(name))[2])
+
+
+def test_loader_keeps_bf16_and_widens_for_the_32_bit_engine():
+    d = model_dir("A")
+    t = load_checkpoint(d, _specs("A"), torch.bfloat16)
+    assert t["model.layers.0.mlp.down_proj.weight"].dtype == torch.bfloat16
+    assert t["model.norm.weight"].dtype == torch.float32               # norm weights are always 32 bit
+    t32 = load_checkpoint(d, _specs("A"), torch.float32)
+    assert all(v.dtype == torch.float32 for v in t32.values())
+    assert torch.equal(t32["model.embed_tokens.weight"], t["model.embed_tokens.weight"].float())
+
+
+def test_a_tensor_stored_in_32_bit_stays_so_and_tables_are_int32(tmp_path):
+    save_file({"m": torch.randn(4, 4), "h": torch.randn(4, 4).half(), "t": torch.arange(4, dtype=torch.int64)},
+              str(tmp_path / "model.safetensors"))
+    specs = [ParamSpec("m", (4, 4)), ParamSpec("h", (4, 4)), ParamSpec("t", (4,), role="table")]
+    out = load_checkpoint(str(tmp_path), specs, torch.bfloat16)
+    assert out["m"].dtype == torch.float32 and out["h"].dtype == torch.bfloat16 and out["t"].dtype == torch.int32
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    d = model_dir("A")
+    with safe_open(os.path.join(d, "model.safetensors"), framework="pt") as f:
+        t = {k: f.get_tensor(k) for k in f.keys()}
+    del t["model.layers.1.self_attn.v_proj.bias"]
+    del t["model.norm.weight"]
+    t["model.layers.0.mlp.up_proj.weight"] = torch.zeros(10, 64, dtype=torch.bfloat16)
+    t["model.layers.7.extra.weight"] = torch.zeros(2)
+    os.makedirs(tmp_path / "m")
+    save_file(t, str(tmp_path / "m" / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_checkpoint(str(tmp_path / "m"), _specs("A"), torch.bfloat16)
+    err = e.value
+    assert err.missing == ["model.layers.1.self_attn.v_proj.bias", "model.norm.weight"]
+    assert err.unexpected == ["model.layers.7.extra.weight"]
+    assert [(n, tuple(x), tuple(y)) for n, x, y in err.wrong_shape] == [("model.layers.0.mlp.up_proj.weight", (172, 64), (10, 64))]
+    msg = str(err)
+    for word in ("missing", "unexpected", "wrong shapes", "v_proj.bias", "extra.weight", "[172, 64]", "[10, 64]"):
+        assert word in msg
+
+
+def test_tied_model_ignores_a_stored_lm_head_and_untied_needs_it(tmp_path):
+    d = model_dir("A")
+    with safe_open(os.path.join(d, "model.safetensors"), framework="pt") as f:
+        t = {k: f.get_tensor(k) for k in f.keys()}
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    os.makedirs(tmp_path / "m")
+    save_file(t, str(tmp_path / "m" / "model.safetensors"))
+    load_checkpoint(str(tmp_path / "m"), _specs("A"), torch.bfloat16, optional=["lm_head.weight"])
+    with pytest.raises(WeightsError) as e:
+        load_checkpoint(d, _specs("A") + [ParamSpec("lm_head.weight", (256, 64))], torch.bfloat16)
+    assert e.value.missing == ["lm_head.weight"]
+
+
+def test_truncated_and_empty_folders(tmp_path):
+    with pytest.raises(WeightsError, match="no .safetensors"):
+        load_checkpoint(str(tmp_path), _specs("A"), torch.bfloat16)
+    src = os.path.join(model_dir("A"), "model.safetensors")
+    data = open(src, "rb").read()
+    (tmp_path / "model.safetensors").write_bytes(data[:len(data) // 2])
+    with pytest.raises(WeightsError, match="truncated"):
+        load_checkpoint(str(tmp_path), _specs("A"), torch.bfloat16)

@@ -1,0 +1,131 @@
+"""The scheduler's decisions, with a fake model step (no GPU)."""
+import random
+
+import pytest
+
+from pico_vllm_amd.cache.manager import CacheManager
+from pico_vllm_amd.engine.request import Request, RequestStatus
+from pico_vllm_amd.engine.scheduler import Scheduler
+from pico_vllm_amd.parts.spec import CacheSpec
+from pico_vllm_amd.sampling.params import SamplingParams
+from pico_vllm_amd.sampling.sampler import uniform
+
+SPEC = {0: CacheSpec("paged_kv", num_kv_heads=1, head_dim=16)}
+
+
+def make(num_pages=64, page=16, max_seqs=4, budget=32, max_len=512):
+    m = CacheManager(SPEC, page, num_pages, max_seqs)
+    return m, Scheduler(m, max_seqs, budget, max_len)
+
+
+def req(i, n_prompt, n_new):
+    return Request(i, list(range(1, n_prompt + 1)), SamplingParams(max_new_tokens=n_new))
+
+
+def drive(s: Scheduler, requests, max_steps=10000, log=None):
+    """Run to completion with a fake step: the 'sampled' token is a function of what was run."""
+    order = []
+    for _ in range(max_steps):
+        if not s.has_unfinished():
+            return order
+        plan = s.schedule()
+        assert plan.seqs, "nothing scheduled although requests are unfinished"
+        assert plan.num_tokens <= s.max_num_batched_tokens
+        assert len(s.running) <= s.max_num_seqs
+        if log is not None:
+            log.append([(x.request.request_id, x.request.num_computed, x.num_tokens) for x in plan.seqs])
+        for x in plan.seqs:
+            samples = x.samples
+            s.on_step_done(x)
+            if samples:
+                r = x.request
+                r.generated_ids.append((sum(r.all_ids) * 31 + len(r.all_ids)) % 1000)
+                if r.is_max_len_finished():
+                    s.finish(r, "length")
+                    order.append(r.request_id)
+        s.manager.check()
+    raise AssertionError("did not finish")
+
+
+def test_fcfs_admission_and_token_budget_cut_prompts_into_portions():
+    m, s = make(budget=32, max_seqs=4)
+    for i, n in enumerate([50, 10, 70]):
+        s.add_request(req(i, n, 3))
+    log = []
+    drive(s, None, log=log)
+    # step 0: request 0 gets the whole budget; request 1 is not admitted before request 0's turn is served
+    assert log[0] == [(0, 0, 32)]
+    assert log[1] == [(0, 32, 18), (1, 0, 10), (2, 0, 4)]
+    # decode tokens come first afterwards, then the prompt portion of request 2
+    assert log[2][:2] == [(0, 50, 1), (1, 10, 1)] and log[2][2] == (2, 4, 30)
+
+
+def test_finishing_frees_pages_in_the_same_step_and_first_token_counts():
+    m, s = make()
+    s.add_request(req(0, 5, 1))
+    plan = s.schedule()
+    assert plan.seqs[0].samples and plan.seqs[0].num_tokens == 5
+    s.on_step_done(plan.seqs[0])
+    plan.seqs[0].request.generated_ids.append(7)
+    assert plan.seqs[0].request.is_max_len_finished()       # max_new_tokens = 1: done after the prefill step
+    s.finish(plan.seqs[0].request, "length")
+    assert not s.has_unfinished() and m.groups[0].pool.num_free == 64 and m.slots.num_free == 4
+    assert plan.seqs[0].request.status is RequestStatus.FINISHED
+
+
+def test_request_that_can_never_fit_is_refused_at_once():
+    m, s = make(num_pages=4, page=16)
+    with pytest.raises(ValueError, match="never finish"):
+        s.add_request(req(0, 60, 10))
+    with pytest.raises(ValueError, match="max_seq_len"):
+        make(max_len=32)[1].add_request(req(0, 30, 10))
+    s.add_request(req(1, 60, 4))                              # exactly 4 pages
+
+
+def test_pages_running_out_preempts_the_last_admitted_which_recomputes():
+    m, s = make(num_pages=6, page=16, max_seqs=3, budget=64)
+    a, b = req(0, 30, 40), req(1, 30, 40)                      # each grows to 70 tokens = 5 pages; pool has 6
+    s.add_request(a); s.add_request(b)
+    log = []
+    done = drive(s, None, log=log)
+    assert done == [0, 1]                                      # the older request is never the victim
+    assert b.num_preemptions >= 1 and a.num_preemptions == 0 and s.num_preemptions == b.num_preemptions
+    # after its preemption, b ran its prompt AND its generated tokens again from position 0
+    restart = [e for step in log for e in step if e[0] == 1 and e[1] == 0]
+    assert len(restart) == 1 + b.num_preemptions and restart[-1][2] > 30
+    assert len(a.generated_ids) == 40 and len(b.generated_ids) == 40
+    # the same tokens as with plenty of pages: the fake token depends only on the request's own history
+    m2, s2 = make(num_pages=64, page=16, max_seqs=3, budget=64)
+    a2, b2 = req(0, 30, 40), req(1, 30, 40)
+    s2.add_request(a2); s2.add_request(b2)
+    drive(s2, None)
+    assert a2.generated_ids == a.generated_ids and b2.generated_ids == b.generated_ids
+    assert m.groups[0].pool.reuse_count > 0
+
+
+def test_no_admission_without_pages_or_slots():
+    m, s = make(num_pages=4, page=16, max_seqs=2, budget=64)
+    s.add_request(req(0, 40, 2)); s.add_request(req(1, 40, 2)); s.add_request(req(2, 5, 2))
+    plan = s.schedule()
+    # request 0 takes 3 of 4 pages; request 1 needs 3: not admitted, and request 2 does not jump the queue
+    assert [x.request.request_id for x in plan.seqs] == [0]
+    assert [r.request_id for r in s.waiting] == [1, 2]
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_every_request_finishes_under_random_load_and_a_tiny_pool(seed):
+    rng = random.Random(seed)
+    m, s = make(num_pages=12, page=8, max_seqs=4, budget=24, max_len=96)
+    reqs = [req(i, rng.randint(1, 40), rng.randint(1, 30)) for i in range(12)]
+    for r in reqs:
+        s.add_request(r)
+    done = drive(s, None)
+    assert sorted(done) == list(range(12))
+    assert all(len(r.generated_ids) == r.params.max_new_tokens for r in reqs)
+    assert m.groups[0].pool.num_free == 12 and m.slots.num_free == 4
+
+
+def test_uniform_numbers_are_a_pure_function_of_seed_and_index():
+    a = [uniform(5, i) for i in range(1000)]
+    assert a == [uniform(5, i) for i in range(1000)] and a != [uniform(6, i) for i in range(1000)]
+    assert all(0.0 <= x < 1.0 for x in a) and 0.45 < sum(a) / 1000 < 0.55

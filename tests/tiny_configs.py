@@ -1,0 +1,44 @@
+"""The small configurations the tests run: they differ in every size and option."""
+import os
+import tempfile
+
+TINY_A = {   # MQA, tied, head 16
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 256, "hidden_size": 64, "num_hidden_layers": 2, "num_attention_heads": 4,
+    "num_key_value_heads": 1, "intermediate_size": 172, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+    "tie_word_embeddings": True, "max_position_embeddings": 2048, "hidden_act": "silu", "eos_token_id": 255,
+}
+TINY_B = {   # groups of 2, untied, head 32
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 384, "hidden_size": 192, "num_hidden_layers": 3, "num_attention_heads": 6,
+    "num_key_value_heads": 3, "intermediate_size": 320, "rms_norm_eps": 1e-5, "rope_theta": 1000000.0,
+    "tie_word_embeddings": False, "max_position_embeddings": 4096, "hidden_act": "silu", "eos_token_id": 383,
+}
+TINY_C = {   # head size 48 given explicitly (hidden != heads * head), 5 heads without grouping, odd vocabulary
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 301, "hidden_size": 136, "num_hidden_layers": 1, "num_attention_heads": 5,
+    "num_key_value_heads": 5, "head_dim": 48, "intermediate_size": 200, "rms_norm_eps": 1e-6,
+    "rope_theta": 50000.0, "tie_word_embeddings": True, "max_position_embeddings": 1024, "hidden_act": "silu",
+}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+_made = {}
+
+
+# larger q/k/v/o and MLP matrices than N(0, 0.02): attention scores then spread over several units and
+# the layers change the residual stream visibly, so a wrong rotation, mask or page shows in the logits
+STRONG = {"q_proj.weight": 0.25, "k_proj.weight": 0.25, "v_proj.weight": 0.1, "o_proj.weight": 0.1,
+          "gate_proj": 0.1, "up_proj": 0.1, "down_proj": 0.1, "_proj.bias": 0.2, "embed_tokens": 0.1,
+          "lm_head": 0.1}
+
+
+def model_dir(name: str, seed: int = 0, strong: bool = True) -> str:
+    """A random-weights model folder in a temporary place, made once per process."""
+    from pico_vllm_amd.weights.random_init import write_random_model
+    key = (name, seed, strong)
+    if key not in _made:
+        d = tempfile.mkdtemp(prefix=f"pico_tiny_{name}_")
+        write_random_model(d, CONFIGS[name], seed, STRONG if strong else None)
+        _made[key] = d
+    return _made[key]
