@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput at the Qwen2.5-1.5B shape with random weights on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the engine (scheduler, model step from a HIP graph, sampling) at
+batch 8 with every request's context ending at 4096 tokens.  One JSON line goes to stdout:
+decoded tokens a second as ``value``; ``prefill`` (one 2,048-token prompt in one step) with its
+fraction of the bf16 matrix-core peak; ``roofline`` (bytes the decode step has to read: every
+weight once plus the cache of the live requests, over its time, against 8 TB/s); ``points``
+with decode at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import shutil
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12            # bytes/s, MI355X HBM3E
+MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+# BASELINE.json configs[2]: Qwen2.5-1.5B
+CONFIG_1P5B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 151936, "hidden_size": 1536, "num_hidden_layers": 28, "num_attention_heads": 12,
+    "num_key_value_heads": 2, "intermediate_size": 8960, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
+    "tie_word_embeddings": True, "max_position_embeddings": 131072, "hidden_act": "silu",
+}
+CONTEXT = 4096
+PREFILL_TOKENS = 2048
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def prefill_flops(cfg, T: int) -> float:
+    """GEMM flops of T prompt tokens, causal attention flops, and the output matrix on one row."""
+    H, L, nq, nkv = cfg["hidden_size"], cfg["num_hidden_layers"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d = cfg.get("head_dim") or H // nq
+    I, V = cfg["intermediate_size"], cfg["vocab_size"]
+    per_token = 2.0 * L * (H * (nq + 2 * nkv) * d + nq * d * H + 2 * H * I + I * H)
+    attn = 4.0 * nq * d * (T * (T + 1) / 2) * L
+    return per_token * T + attn + 2.0 * H * V
+
+
+def make_engine(model_dir, dtype, batch, layers_model=None):
+    from pico_vllm_amd import EngineArgs
+    from pico_vllm_amd.engine.llm import LLMEngine
+    block = 16
+    args = EngineArgs(model=model_dir, dtype=dtype, block_size=block,
+                      num_gpu_blocks=batch * (CONTEXT // block + 1) + 8, max_seq_len=CONTEXT + 16,
+                      max_num_seqs=batch, max_num_batched_tokens=max(PREFILL_TOKENS, batch),
+                      use_cuda_graph=True, max_batch_size=64)
+    return LLMEngine(args, model=layers_model)
+
+
+def decode_point(model_dir, model, dtype, batch, steps, warmup):
+    """Fill `batch` requests so that the timed steps end at CONTEXT tokens, then time `steps` decode steps."""
+    import torch
+    eng = make_engine(model_dir, dtype, batch, model)
+    V = CONFIG_1P5B["vocab_size"]
+    g = torch.Generator().manual_seed(batch)
+    prompt_len = CONTEXT - (warmup + steps) - 1
+    for i in range(batch):
+        ids = torch.randint(0, V, (prompt_len,), generator=g).tolist()
+        eng.submit(ids, max_new_tokens=warmup + steps + 1, temperature=0.0, ignore_eos=True)
+    t0 = time.time()
+    while any(r.num_uncomputed > 1 or not r.generated_ids for r in eng.requests.values()):
+        eng.step()                                   # prompt portions (and the first decodes of early requests)
+    torch.cuda.synchronize()
+    log(f"batch {batch}: prompts of {prompt_len} tokens in the cache after {time.time() - t0:.1f}s")
+    # bring every request to the same number of generated tokens is not needed: all decode from here on
+    for _ in range(warmup):
+        eng.step()
+    torch.cuda.synchronize()
+    ctx_start = [r.total_len - 1 for r in eng.requests.values()]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        done = eng.step()
+        if done:
+            raise RuntimeError("a request finished inside the timed region")
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx_mean = [c + (steps - 1) / 2 + 1 for c in ctx_start]          # keys read per step, averaged over the region
+    nbytes = eng.runner.decode_bytes([int(c) for c in ctx_mean])
+    ms = dt / steps * 1e3
+    res = {"tok_s": batch * steps / dt, "ms_per_step": ms, "bytes": nbytes, "gbps": nbytes / (dt / steps) / 1e9,
+           "context": sum(ctx_mean) / batch}
+    model = eng.model
+    del eng
+    torch.cuda.empty_cache()
+    return res, model
+
+
+def prefill_point(model_dir, model, dtype, reps=3):
+    import torch
+    from pico_vllm_amd.engine.batch import SeqStep
+    eng = make_engine(model_dir, dtype, 1, model)
+    V = CONFIG_1P5B["vocab_size"]
+    ids = torch.randint(0, V, (PREFILL_TOKENS,), generator=torch.Generator().manual_seed(7)).tolist()
+    m = eng.runner.manager
+    times = []
+    for i in range(reps + 1):
+        rid = f"p{i}"
+        m.add_request(rid)
+        assert m.grow(rid, PREFILL_TOKENS)
+        seq = [SeqStep(rid, ids, [PREFILL_TOKENS - 1])]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.runner.step(seq)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        m.free_request(rid)
+    dt = min(times[1:])
+    return {"value": PREFILL_TOKENS / dt, "tokens": PREFILL_TOKENS, "ms": dt * 1e3,
+            "frac": prefill_flops(CONFIG_1P5B, PREFILL_TOKENS) / dt / MFMA_PEAK[dtype]}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--model", default=None, help="reuse a model folder instead of writing random weights")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
+        return 2
+    if a.steps + a.warmup >= CONTEXT // 2:
+        print("bench.py: steps + warmup must stay below 2048")
+        return 2
+    import torch
+    from pico_vllm_amd.weights.random_init import write_random_model
+    tmp = None
+    model_dir = a.model
+    if model_dir is None:
+        tmp = tempfile.mkdtemp(prefix="pico_bench_")
+        model_dir = tmp
+        t0 = time.time()
+        log("writing random Qwen2.5-1.5B-shaped weights ...")
+        write_random_model(model_dir, CONFIG_1P5B, seed=0)
+        log(f"... {time.time() - t0:.0f}s")
+    try:
+        main_res, model = decode_point(model_dir, None, a.dtype, a.batch, a.steps, a.warmup)
+        log(f"decode batch {a.batch}: {main_res['tok_s']:.0f} tok/s, {main_res['ms_per_step']:.3f} ms/step")
+        out = {
+            "metric": "decode tok/s @ batch 8, Qwen2.5-1.5B bf16 (plus batch 1/64 and prefill @ 2048 tok)",
+            "value": round(main_res["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
+            "warmup": a.warmup, "ms_per_step": round(main_res["ms_per_step"], 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+            "config": {"model": "Qwen2.5-1.5B shape", "global_batch": a.batch, "seq_len": CONTEXT,
+                       "parallelism": "single GPU", "layers": 28, "layers_run": 28, "hidden": 1536, "q_heads": 12,
+                       "kv_heads": 2, "head_dim": 128, "intermediate": 8960, "vocab": 151936, "tied": True,
+                       "page_size": 16, "prompt_len": CONTEXT - (a.steps + a.warmup) - 1,
+                       "context_in_timed_steps": round(main_res["context"], 1), "hip_graph": True},
+            "roofline": {"bound": "hbm", "achieved": round(main_res["gbps"], 1), "peak": HBM_PEAK / 1e9,
+                         "unit": "GB/s", "frac": round(main_res["gbps"] * 1e9 / HBM_PEAK, 4)},
+        }
+        if not a.no_points:
+            out["prefill"] = {k: (round(v, 4) if isinstance(v, float) else v)
+                              for k, v in prefill_point(model_dir, model, a.dtype).items()}
+            log(f"prefill: {out['prefill']}")
+            pts = {}
+            for b, steps in ((1, min(a.steps, 200)), (64, min(a.steps, 100))):
+                r, model = decode_point(model_dir, model, a.dtype, b, steps, min(a.warmup, 10))
+                pts[f"decode_b{b}"] = round(r["tok_s"], 1)
+                pts[f"decode_b{b}_hbm_frac"] = round(r["gbps"] * 1e9 / HBM_PEAK, 4)
+                log(f"decode batch {b}: {r['tok_s']:.0f} tok/s, {r['ms_per_step']:.3f} ms/step")
+            out["points"] = pts
+        print(json.dumps(out), flush=True)
+    finally:
+        if tmp:
+            shutil.rmtree(tmp, ignore_errors=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

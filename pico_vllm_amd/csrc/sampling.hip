@@ -29,10 +29,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
                                                                 const float* __restrict__ top_p,
                                                                 const float* __restrict__ u, int* __restrict__ out) {
   __shared__ float scratch[16];
-  __shared__ float part[SAMPLE_THREADS];
+  __shared__ double part[SAMPLE_THREADS];  // chunk sums in double: the CDF of 150k terms stays exact to ~1e-7
   __shared__ int idx_scratch[16];
   __shared__ int chosen_chunk;
-  __shared__ float chosen_before;
+  __shared__ double chosen_before;
+  __shared__ double chosen_target;
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* x = logits + (size_t)row * ld;
   const float temp = temperature[row];
@@ -79,40 +80,40 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   // inverse CDF over the kept tokens in vocabulary order; thread i owns a contiguous chunk
   const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
   const int b = min(tid * chunk, V), e_ = min(b + chunk, V);
-  float s = 0.f;
+  double s = 0.0;
   for (int i = b; i < e_; i++) {
     const float e = expf((x[i] - mx) * inv_t);
-    if (e >= thr) s += e;
+    if (e >= thr) s += (double)e;
   }
   part[tid] = s;
   __syncthreads();
   if (tid == 0) {
-    float kept = 0.f;
+    double kept = 0.0;
     for (int i = 0; i < SAMPLE_THREADS; i++) kept += part[i];
-    const float target = u[row] * kept;
-    float run = 0.f;
+    const double target = (double)u[row] * kept;
+    double run = 0.0;
     int c = -1, last_nonzero = 0;
-    float before_last = 0.f;
+    double before_last = 0.0;
     for (int i = 0; i < SAMPLE_THREADS; i++) {
-      if (part[i] > 0.f) { last_nonzero = i; before_last = run; }
+      if (part[i] > 0.0) { last_nonzero = i; before_last = run; }
       if (run + part[i] > target) { c = i; break; }
       run += part[i];
     }
     if (c < 0) { c = last_nonzero; run = before_last; }
     chosen_chunk = c;
     chosen_before = run;
-    scratch[0] = target;
+    chosen_target = target;
   }
   __syncthreads();
   if (tid == chosen_chunk) {
-    const float target = scratch[0];
-    float run = chosen_before;
+    const double target = chosen_target;
+    double run = chosen_before;
     int pick = -1, last_kept = mi;
     for (int i = b; i < e_; i++) {
       const float e = expf((x[i] - mx) * inv_t);
       if (e >= thr) {
         last_kept = i;
-        run += e;
+        run += (double)e;
         if (run > target) { pick = i; break; }
       }
     }

@@ -150,8 +150,17 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     return gate * torch.sigmoid(gate) * up
 
 
+def _same(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
+def to_bf16(x: torch.Tensor) -> torch.Tensor:
+    """Round to bfloat16 and back: what storing an activation in bfloat16 does to it."""
+    return x.to(torch.bfloat16).float()
+
+
 def attention_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
-                    cfg: PlainConfig, positions: torch.Tensor) -> torch.Tensor:
+                    cfg: PlainConfig, positions: torch.Tensor, rnd=_same) -> torch.Tensor:
     """qkv = h W^T + b with bias on q, k, v only (model.py:148-152); RoPE on
     q and k (model.py:211); attention; o_proj without bias (model.py:147,225)."""
     nq, nkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
@@ -161,42 +170,47 @@ def attention_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
     b = torch.cat([w[f"{prefix}.self_attn.q_proj.bias"],
                    w[f"{prefix}.self_attn.k_proj.bias"],
                    w[f"{prefix}.self_attn.v_proj.bias"]], dim=0)
-    qkv = h @ W.T + b
+    qkv = rnd(h @ W.T + b)
     q, k, v = split_qkv(qkv, nq, nkv, d)
     cos, sin = rope_tables(positions, d, cfg.rope_theta)
-    q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
-    o = causal_attention(q, k, v, q_positions=positions - positions[0])
-    return o.reshape(h.shape[0], nq * d) @ w[f"{prefix}.self_attn.o_proj.weight"].T
+    q, k = rnd(apply_rope(q, cos, sin)), rnd(apply_rope(k, cos, sin))
+    o = rnd(causal_attention(q, k, v, q_positions=positions - positions[0]))
+    return rnd(o.reshape(h.shape[0], nq * d) @ w[f"{prefix}.self_attn.o_proj.weight"].T)
 
 
-def mlp_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str) -> torch.Tensor:
+def mlp_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, rnd=_same) -> torch.Tensor:
     """down( swiglu( h [gate; up]^T ) ), no biases (model.py:309-318)."""
     Wgu = torch.cat([w[f"{prefix}.mlp.gate_proj.weight"], w[f"{prefix}.mlp.up_proj.weight"]], dim=0)
-    return swiglu(h @ Wgu.T) @ w[f"{prefix}.mlp.down_proj.weight"].T
+    return rnd(rnd(swiglu(rnd(h @ Wgu.T))) @ w[f"{prefix}.mlp.down_proj.weight"].T)
 
 
 def block(x: torch.Tensor, w: Dict[str, torch.Tensor], i: int, cfg: PlainConfig,
-          positions: torch.Tensor) -> torch.Tensor:
+          positions: torch.Tensor, rnd=_same) -> torch.Tensor:
     """x += attn(norm1(x)); x += ffn(norm2(x))   (model.py:361-374)."""
     p = f"model.layers.{i}"
-    x = x + attention_layer(rms_norm(x, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps),
-                            w, p, cfg, positions)
-    x = x + mlp_layer(rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], cfg.rms_norm_eps), w, p)
+    x = x + attention_layer(rnd(rms_norm(x, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps)),
+                            w, p, cfg, positions, rnd)
+    x = x + mlp_layer(rnd(rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], cfg.rms_norm_eps)), w, p, rnd)
     return x
 
 
 def forward(tokens: Sequence[int], w: Dict[str, torch.Tensor], cfg: PlainConfig,
-            first_position: int = 0) -> torch.Tensor:
+            first_position: int = 0, rnd=_same) -> torch.Tensor:
     """Logits [S, V] for one whole sequence (model.py:427-445): embedding,
     L blocks, final norm, output matrix.  Tied models multiply by the
     embedding matrix; untied ones by lm_head.weight (our deliberate
-    difference, see the module docstring)."""
+    difference, see the module docstring).
+
+    ``rnd`` is applied to every activation between the parts (not to the
+    residual stream, not to the logits); with ``to_bf16`` it shows how far
+    bfloat16 storage of activations moves the logits of this model, which is
+    the yardstick for the bfloat16 engine's tolerance."""
     ids = torch.as_tensor(list(tokens), dtype=torch.long)
     x = w["model.embed_tokens.weight"][ids].float()
     positions = torch.arange(first_position, first_position + len(ids))
     for i in range(cfg.num_hidden_layers):
-        x = block(x, w, i, cfg, positions)
-    x = rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps)
+        x = block(x, w, i, cfg, positions, rnd)
+    x = rnd(rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps))
     out_w = w["model.embed_tokens.weight"] if cfg.tie_word_embeddings else w["lm_head.weight"]
     return x @ out_w.float().T
 
@@ -208,9 +222,9 @@ class PlainModel:
         self.cfg = read_config(model_dir)
         self.w = read_weights(model_dir)
 
-    def logits(self, tokens: Sequence[int]) -> torch.Tensor:
+    def logits(self, tokens: Sequence[int], rnd=_same) -> torch.Tensor:
         with torch.no_grad():
-            return forward(tokens, self.w, self.cfg)
+            return forward(tokens, self.w, self.cfg, rnd=rnd)
 
     def greedy(self, prompt: Sequence[int], n: int) -> List[int]:
         toks = list(prompt)

@@ -1,0 +1,149 @@
+"""Generation through the entry point against the plain implementation: the workloads of the two
+tiny configurations, greedy and with temperature, chunked prompts mixed with decoding, HIP graph
+replay of decode steps, and what happens when pages run out."""
+import pytest
+import torch
+
+import plain_qwen2 as P
+from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
+
+pytestmark = pytest.mark.gpu
+
+
+def llm(name, dtype, **kw):
+    from pico_vllm_amd import LLM
+    args = dict(block_size=PAGE_SIZE[name], num_gpu_blocks=64, max_seq_len=256, max_num_seqs=4,
+                max_num_batched_tokens=64, use_cuda_graph=False)
+    args.update(kw)
+    return LLM(model=model_dir(name), dtype=dtype, **args)
+
+
+def prompts_for(name, lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    V = CONFIGS[name]["vocab_size"]
+    return [torch.randint(0, V - 1, (n,), generator=g).tolist() for n in lengths]     # never the eos id
+
+
+def check_greedy(name, dtype, prompts, outs):
+    """Every generated token is the plain argmax given the same prefix (bfloat16: or within the
+    rounding error of the logits of it)."""
+    plain = P.PlainModel(model_dir(name))
+    for p, o in zip(prompts, outs):
+        toks = list(p)
+        for t in o.token_ids:
+            logits = plain.logits(toks)[-1]
+            slack = 1e-4 if dtype == "float32" else 0.05 * float(logits.std())
+            assert float(logits[t]) >= float(logits.max()) - slack, (name, dtype, len(p), o.token_ids)
+            toks.append(t)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tiny_a_workload_greedy(dtype):
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("A", [5, 11, 23])
+    outs = llm("A", dtype).generate(prompts, SamplingParams(max_new_tokens=8, temperature=0.0, ignore_eos=True))
+    assert [len(o.token_ids) for o in outs] == [8, 8, 8] and all(o.finish_reason == "length" for o in outs)
+    check_greedy("A", dtype, prompts, outs)
+    if dtype == "float32":
+        plain = P.PlainModel(model_dir("A"))
+        assert [o.token_ids for o in outs] == [plain.greedy(p, 8) for p in prompts]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tiny_b_workload_chunks_of_13_temperature(dtype):
+    """4 requests, prompts 1/7/19/40, prefilled in portions of at most 13 tokens mixed with decoding,
+    10 tokens each at temperature 0.8 with a fixed seed."""
+    from pico_vllm_amd import SamplingParams
+    from pico_vllm_amd.sampling.sampler import uniform
+    prompts = prompts_for("B", [1, 7, 19, 40], seed=1)
+    sp = [SamplingParams(max_new_tokens=10, temperature=0.8, seed=100 + i, ignore_eos=True) for i in range(4)]
+    eng = llm("B", dtype, max_num_batched_tokens=13)
+    outs = eng.generate(prompts, sp)
+    assert eng.engine.stats["steps"] > 10 + 3            # prompts were cut: 67 prompt tokens at <= 13 a step
+    again = llm("B", dtype, max_num_batched_tokens=64).generate(prompts, sp)
+    plain = P.PlainModel(model_dir("B"))
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert len(o.token_ids) == 10
+        toks = list(p)
+        for k, t in enumerate(o.token_ids):
+            probs = P.temperature_probs(plain.logits(toks)[-1], 0.8)
+            u = uniform(100 + i, k)
+            want = P.inverse_cdf(probs, u)
+            if t != want:        # only where u falls within the engine's rounding of a CDF boundary
+                cum = torch.cumsum(probs, 0)
+                edge = float(cum[min(t, want)])
+                assert abs(edge - u) < (1e-4 if dtype == "float32" else 2e-2), (dtype, i, k, t, want, u, edge)
+            toks.append(t)
+        if dtype == "float32":
+            assert o.token_ids == again[i].token_ids     # same seed, other batching: same tokens
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_top_p_and_eos(dtype):
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("B", [9, 9], seed=2)
+    outs = llm("B", dtype).generate(prompts, [SamplingParams(max_new_tokens=12, temperature=1.0, top_p=0.5, seed=7),
+                                               SamplingParams(max_new_tokens=12, temperature=0.0)])
+    plain = P.PlainModel(model_dir("B"))
+    toks = list(prompts[0])
+    for t in outs[0].token_ids:                         # every draw lies in the nucleus of the plain rule
+        p = P.top_p_probs(plain.logits(toks)[-1], 1.0, 0.5 if dtype == "float32" else 0.55)
+        assert float(p[t]) > 0
+        toks.append(t)
+    eos = CONFIGS["B"]["eos_token_id"]
+    for o in outs:
+        assert (o.finish_reason == "eos") == (o.token_ids[-1] == eos and len(o.token_ids) <= 12)
+        assert eos not in o.token_ids[:-1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_replayed_from_a_graph_give_the_same_tokens(dtype):
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("A", [5, 11, 23, 40, 3], seed=3)
+    sp = SamplingParams(max_new_tokens=40, temperature=0.0, ignore_eos=True)
+    eager = llm("A", dtype, num_gpu_blocks=128).generate(prompts, sp)
+    graph_llm = llm("A", dtype, num_gpu_blocks=128, use_cuda_graph=True, max_batch_size=4)
+    graphed = graph_llm.generate(prompts, sp)
+    assert graph_llm.engine.runner._graphs, "no decode step went through a graph"
+    if dtype == "float32":
+        assert [o.token_ids for o in graphed] == [o.token_ids for o in eager]
+    check_greedy("A", dtype, prompts, graphed)
+    # a second batch on the same engine replays the graphs captured by the first
+    more = graph_llm.generate(prompts[:2], sp)
+    check_greedy("A", dtype, prompts[:2], more)
+
+
+def test_running_out_of_pages_preempts_and_recomputes_to_the_same_tokens():
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("A", [30, 30, 30], seed=4)
+    sp = SamplingParams(max_new_tokens=40, temperature=0.0, ignore_eos=True)
+    roomy = llm("A", "float32", num_gpu_blocks=64).generate(prompts, sp)
+    tight_llm = llm("A", "float32", num_gpu_blocks=8)               # 8 pages of 16: three requests of 70 do not fit
+    tight = tight_llm.generate(prompts, sp)
+    assert tight_llm.engine.stats["preemptions"] > 0 and sum(o.num_preemptions for o in tight) > 0
+    assert tight[0].num_preemptions == 0                             # the oldest request is never the victim
+    assert [o.token_ids for o in tight] == [o.token_ids for o in roomy]
+    m = tight_llm.engine.runner.manager
+    m.check()
+    assert m.groups[0].pool.num_free == 8 and m.groups[0].pool.reuse_count > 0
+
+
+def test_submit_step_is_done_in_the_reference_manner():
+    from pico_vllm_amd import EngineArgs
+    from pico_vllm_amd.engine.llm import LLMEngine
+    eng = LLMEngine(EngineArgs(model=model_dir("A"), dtype="float32", num_gpu_blocks=32, max_seq_len=128,
+                               use_cuda_graph=False))
+    a = eng.submit([1, 2, 3], max_new_tokens=1, temperature=0, top_p=1.0)
+    b = eng.submit([4, 5, 6, 7], max_new_tokens=3, temperature=0, top_p=1.0, ignore_eos=True)
+    done = []
+    steps = 0
+    while not eng.is_done():
+        done += eng.step()
+        steps += 1
+    # a request that finishes in its prefill step is reported once and not decoded again
+    assert [o.request_id for o in done] == [a, b] and steps == 3
+    assert len(done[0].token_ids) == 1 and len(done[1].token_ids) == 3
+    with pytest.raises(ValueError):
+        eng.submit([1] * 200, max_new_tokens=10)
+    with pytest.raises(ValueError):
+        eng.submit([999], max_new_tokens=1)

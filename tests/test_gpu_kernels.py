@@ -1,0 +1,272 @@
+"""Each HIP kernel alone against a plain float32 reference of the same op, at sizes other than
+the engine's (odd widths, head sizes in steps of 16, page sizes 8..64)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_qwen2 as P
+from gpu_util import DEV, DTYPES, flat_batch, paged_cache, tol
+from test_plain import REFERENCE_CASES
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from pico_vllm_amd.ops import kernels
+    return kernels
+
+
+def close(a, b, dtype, scale=1.0):
+    rtol, atol = tol(dtype)
+    a, b = a.float().cpu(), b.float().cpu()
+    assert a.shape == b.shape
+    err = (a - b).abs()
+    bound = atol * scale + rtol * b.abs()
+    assert bool((err <= bound).all()), f"max err {float(err.max()):.3e} (bound {float(bound.min()):.3e}..)"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(K, dtype):
+    table = torch.randn(301, 136).to(dtype)
+    ids = torch.tensor([0, 300, 5, 5, 17], dtype=torch.int32)
+    out = K.embedding(table.to(DEV), ids.to(DEV))
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [64, 136, 1536, 5000])
+def test_add_rmsnorm(K, dtype, H):
+    T, eps = 7, 1e-5
+    resid = torch.randn(T, H) * 3
+    delta = (torch.randn(T, H)).to(dtype)
+    w = 1 + 0.1 * torch.randn(H)
+    want_sum = resid + delta.float()
+    r = resid.clone().to(DEV)
+    out = K.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, dtype)
+    close(r, want_sum, torch.float32)                                   # the residual stream is float32
+    close(out, P.rms_norm(want_sum, w, eps), dtype)
+    # no delta: the stream is untouched
+    r2 = resid.clone().to(DEV)
+    out = K.add_rmsnorm(r2, None, w.to(DEV), eps, dtype)
+    assert torch.equal(r2.cpu(), resid)
+    close(out, P.rms_norm(resid, w, eps), dtype)
+    # wanted rows only: the stream is untouched, rows are gathered
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    r3 = resid.clone().to(DEV)
+    out = K.add_rmsnorm(r3, delta.to(DEV), w.to(DEV), eps, dtype, rows=rows.to(DEV))
+    assert torch.equal(r3.cpu(), resid)
+    close(out, P.rms_norm(want_sum[rows.long()], w, eps), dtype)
+
+
+def test_rmsnorm_eps_is_inside_the_root(K):
+    x = torch.full((1, 64), 1e-4)
+    out = K.add_rmsnorm(x.to(DEV), None, torch.ones(64, device=DEV), 1e-2, torch.float32)
+    close(out, x / math.sqrt(1e-8 + 1e-2), torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(K, dtype):
+    gu = (torch.randn(5, 2 * 172) * 2).to(dtype)
+    close(K.swiglu(gu.to(DEV)), P.swiglu(gu), dtype)
+    g = gu[:, :172].float()
+    close(K.swiglu(torch.cat([gu[:, :172], torch.ones(5, 172).to(dtype)], -1).to(DEV)), F.silu(g), dtype)
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 301, 136), (5, 64, 172), (70, 130, 64), (130, 17, 33)])
+def test_gemm_f32(K, M, N, K_):
+    a, w, b = torch.randn(M, K_), torch.randn(N, K_), torch.randn(N)
+    out = K.gemm_f32(a.to(DEV), w.to(DEV), b.to(DEV))
+    want = a.double() @ w.double().T + b.double()
+    assert torch.allclose(out.cpu().double(), want, rtol=1e-5, atol=1e-4)
+    # a row's result does not depend on the other rows of the call: bitwise
+    one = K.gemm_f32(a[M // 2:M // 2 + 1].to(DEV), w.to(DEV), b.to(DEV))
+    assert torch.equal(one.cpu()[0], out.cpu()[M // 2])
+    # strided rows (a view into a wider buffer), bfloat16 activations
+    wide = torch.randn(M, K_ + 24).to(DEV)
+    out2 = K.gemm_f32(wide[:, 8:8 + K_], w.to(DEV))
+    assert torch.allclose(out2.cpu().double(), wide[:, 8:8 + K_].cpu().double() @ w.double().T, rtol=1e-5, atol=1e-4)
+    ab = a.to(torch.bfloat16)
+    out3 = K.gemm_f32(ab.to(DEV), w.to(DEV))
+    assert torch.allclose(out3.cpu().double(), ab.double() @ w.double().T, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 301, 136), (3, 256, 64), (8, 384, 192), (33, 130, 172), (64, 1000, 1536),
+                                   (100, 77, 40)])
+@pytest.mark.parametrize("out_dtype", DTYPES)
+def test_gemm_bf16(K, M, N, K_, out_dtype):
+    a, w, b = torch.randn(M, K_).bfloat16(), torch.randn(N, K_).bfloat16(), torch.randn(N)
+    out = K.gemm_bf16(a.to(DEV), w.to(DEV), b.to(DEV), out_dtype)
+    want = a.double() @ w.double().T + b.double()
+    assert out.dtype == out_dtype
+    if out_dtype == torch.float32:       # exact products, float32 accumulation
+        assert torch.allclose(out.cpu().double(), want, rtol=1e-4, atol=1e-3 * math.sqrt(K_))
+    else:
+        assert torch.allclose(out.cpu().double(), want, rtol=1e-2, atol=1e-2 * math.sqrt(K_))
+    out_nb = K.gemm_bf16(a.to(DEV), w.to(DEV), None, torch.float32)
+    assert torch.allclose(out_nb.cpu().double(), a.double() @ w.double().T, rtol=1e-4, atol=1e-3 * math.sqrt(K_))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rot,Pg", [(4, 1, 16, 16, 16), (6, 3, 32, 32, 8), (5, 5, 48, 48, 16), (2, 2, 64, 32, 32),
+                                            (12, 2, 128, 128, 16)])
+def test_rope_and_cache_store(K, dtype, nq, nkv, d, rot, Pg):
+    theta = 10000.0
+    new_lens, prefix_lens = [5, 1, 9], [14, 33, 0]          # 14..18 crosses a page edge of 16 (store_kvcache.py:107-118)
+    pos, seq = flat_batch(new_lens, prefix_lens)
+    T = int(pos.numel())
+    qkv = torch.randn(T, (nq + 2 * nkv) * d).to(dtype)
+    num_pages = 12 * 16 // Pg
+    kc = torch.full((num_pages, nkv, Pg, d), 7.0, dtype=dtype, device=DEV)
+    vc = torch.full((num_pages, nkv, d, Pg), 7.0, dtype=dtype, device=DEV)
+    g = torch.Generator().manual_seed(0)
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    maxp = max(-(-(n + p) // Pg) for n, p in zip(new_lens, prefix_lens))
+    bt = torch.full((3, maxp), -1, dtype=torch.int32)
+    for b, (n, p) in enumerate(zip(new_lens, prefix_lens)):
+        for j in range(-(-(n + p) // Pg)):
+            bt[b, j] = perm.pop()
+    inv = (1.0 / (theta ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    x = qkv.clone().to(DEV)
+    K.rope_kv_store(x, pos, seq, bt.to(DEV), inv, kc, vc, nq, nkv, d, rot)
+    # reference
+    q, k, v = P.split_qkv(qkv.float(), nq, nkv, d)
+    cos, sin = P.rope_tables(pos.cpu(), rot, theta)
+
+    def rot_part(t):
+        return torch.cat([P.apply_rope(t[..., :rot], cos, sin), t[..., rot:]], dim=-1)
+    qr, kr = rot_part(q), rot_part(k)
+    close(x[:, :nq * d].reshape(T, nq, d), qr, dtype, scale=3)
+    assert torch.equal(x[:, nq * d:].cpu(), qkv[:, nq * d:])          # k and v in the activation buffer are untouched
+    want_k = torch.full((num_pages, nkv, Pg, d), 7.0)
+    want_v = torch.full((num_pages, nkv, d, Pg), 7.0)
+    for t in range(T):
+        b, p = int(seq[t]), int(pos[t])
+        page, off = int(bt[b, p // Pg]), p % Pg
+        want_k[page, :, off, :] = kr[t]
+        want_v[page, :, :, off] = v[t]
+    close(kc, want_k, dtype, scale=3)          # also: every slot that no token owns still holds 7
+    close(vc, want_v, dtype, scale=3)
+
+
+def _attn_case(K, dtype, new_lens, prefix_lens, nq, nkv, d, Pg, window=0, seed=0, boost=None):
+    g = torch.Generator().manual_seed(seed)
+    totals = [n + p for n, p in zip(new_lens, prefix_lens)]
+    ks = [(torch.randn(N, nkv, d, generator=g)).to(dtype).float() for N in totals]
+    vs = [(torch.randn(N, nkv, d, generator=g)).to(dtype).float() for N in totals]
+    qs = [(torch.randn(n, nq, d, generator=g)).to(dtype).float() for n in new_lens]
+    if boost is not None:
+        boost(qs, ks, vs)
+    num_pages = sum(-(-N // Pg) for N in totals) + 3
+    kc, vc, bt = paged_cache(ks, vs, Pg, num_pages, dtype, seed)
+    pos, seq = flat_batch(new_lens, prefix_lens)
+    q = torch.cat(qs, 0).reshape(-1, nq * d).to(DEV, dtype)
+    out = K.paged_attention_ref(q, kc, vc, bt, pos, seq, nq, nkv, d, 1.0 / math.sqrt(d), window)
+    want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n), window=window)
+                      for qb, kb, vb, n, p in zip(qs, ks, vs, new_lens, prefix_lens)], 0)
+    return out.reshape(-1, nq, d), want
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", range(len(REFERENCE_CASES)))
+def test_plain_attention_kernel_on_the_reference_cases(K, dtype, case):
+    new_lens, prefix_lens = REFERENCE_CASES[case]
+    out, want = _attn_case(K, dtype, new_lens, prefix_lens, 12, 2, 128, 16, seed=case)
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(4, 1, 16, 16), (6, 3, 32, 8), (5, 5, 48, 16), (3, 1, 80, 32), (8, 2, 256, 64),
+                                        (2, 2, 112, 8)])
+def test_plain_attention_kernel_other_sizes(K, dtype, nq, nkv, d, Pg):
+    out, want = _attn_case(K, dtype, [7, 1, 30, 2], [0, 70, 45, 129], nq, nkv, d, Pg, seed=3)
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key_among_hundreds(K, dtype):
+    # one key far back gets a large score; its value dominates the output.  A kernel that drops a
+    # block of keys, a page or a boundary position fails here, whereas with random scores the loss
+    # of one key among 600 would hide under the tolerance.
+    for far in (0, 15, 16, 63, 64, 200, 511):
+        def boost(qs, ks, vs, far=far):
+            ks[0][far] = qs[0][-1, 0:1, :] * 2.0          # same direction as the last query of head 0
+            vs[0][far] = 100.0
+        out, want = _attn_case(K, dtype, [3], [597], 2, 1, 64, 16, seed=far, boost=boost)
+        assert float(want[-1, 0].mean()) > 50
+        close(out, want, dtype, scale=100)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 64, 100])
+def test_attention_window_edge(K, dtype, window):
+    # the key just outside the window carries a huge value: reading it would show at once
+    def boost(qs, ks, vs):
+        n = ks[0].shape[0]
+        last = n - 1
+        if last - window >= 0:
+            vs[0][last - window] = 1000.0
+    out, want = _attn_case(K, dtype, [4, 1], [126, 40], 4, 2, 32, 16, window=window, seed=window, boost=boost)
+    assert float(want[3].abs().max()) < 50
+    close(out, want, dtype)
+
+
+def test_sampling_greedy_and_ties(K):
+    logits = torch.randn(5, 1000)
+    logits[1, 7] = logits[1, 900] = 50.0            # tie: the lower index wins
+    logits[2, 999] = 60.0
+    z = torch.zeros(5)
+    out = K.sample(logits.to(DEV), z.to(DEV), torch.ones(5, device=DEV), z.to(DEV))
+    want = [P.sample_greedy(l) for l in logits]
+    assert out.tolist() == want and want[1] == 7 and want[2] == 999
+
+
+@pytest.mark.parametrize("V", [301, 5000, 151936])
+def test_sampling_temperature_follows_the_inverse_cdf(K, V):
+    g = torch.Generator().manual_seed(V)
+    R = 64
+    logits = torch.randn(R, V, generator=g) * 3
+    temps = torch.rand(R, generator=g) * 1.5 + 0.2
+    us = torch.rand(R, generator=g)
+    out = K.sample(logits.to(DEV), temps.to(DEV), torch.ones(R, device=DEV), us.to(DEV)).tolist()
+    agree = 0
+    for r in range(R):
+        p = P.temperature_probs(logits[r], float(temps[r]))
+        want = P.inverse_cdf(p, float(us[r]))
+        cum = torch.cumsum(p, 0)
+        # equal, or u falls within float32 rounding of a boundary of the CDF
+        if out[r] == want:
+            agree += 1
+        else:
+            lo, hi = sorted((out[r], want))
+            assert hi - lo <= 2 and abs(float(cum[lo]) - float(us[r])) < 1e-5, (r, out[r], want)
+    assert agree >= R - 3
+
+
+def test_sampling_top_p(K):
+    probs = torch.tensor([[0.05, 0.5, 0.15, 0.3]])
+    logits = torch.log(probs)
+    for top_p, kept in ((0.81, {1, 3, 2}), (0.79, {1, 3}), (0.2, {1})):
+        seen = set()
+        for i in range(200):
+            u = torch.tensor([(i + 0.5) / 200])
+            tok = K.sample(logits.to(DEV), torch.ones(1, device=DEV), torch.tensor([top_p], device=DEV), u.to(DEV))
+            seen.add(int(tok[0]))
+            want = P.inverse_cdf(P.top_p_probs(logits[0], 1.0, top_p), float(u))
+            p_kept = P.top_p_probs(logits[0], 1.0, top_p)
+            cum = torch.cumsum(p_kept, 0)
+            assert int(tok[0]) == want or min(abs(float(c) - float(u)) for c in cum) < 1e-5
+        assert seen == kept
+    # a large vocabulary with random logits: every draw lies in the kept set of the plain rule
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(16, 5000, generator=g) * 4
+    us = torch.rand(16, generator=g)
+    out = K.sample(logits.to(DEV), torch.full((16,), 0.7, device=DEV), torch.full((16,), 0.9, device=DEV), us.to(DEV))
+    for r in range(16):
+        p = P.top_p_probs(logits[r], 0.7, 0.9)
+        assert float(p[int(out[r])]) > 0
+        want = P.inverse_cdf(p, float(us[r]))
+        assert abs(int(out[r]) - want) <= 0 or abs(float(torch.cumsum(p, 0)[min(int(out[r]), want)]) - float(us[r])) < 1e-4

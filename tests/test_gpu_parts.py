@@ -1,0 +1,277 @@
+"""Each part alone against the plain function of the same part, a model whose run order names a
+layer twice, and a toy mixer with state of its own that the test registers without touching the
+framework."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen2 as P
+from gpu_util import DEV, DTYPES, tol
+from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
+
+pytestmark = pytest.mark.gpu
+
+
+def close(a, b, dtype, scale=1.0):
+    rtol, atol = tol(dtype)
+    if dtype == torch.float32:
+        rtol, atol = 1e-4, 1e-4         # several chained kernels
+    a, b = a.float().cpu(), b.float().cpu()
+    err = (a - b).abs()
+    assert bool((err <= atol * scale + rtol * b.abs()).all()), f"max err {float(err.max()):.3e}"
+
+
+def close_to_plain(got, exact, rounded, dtype):
+    """float32: summation order only.  bfloat16: within twice the error that rounding every
+    activation to bfloat16 causes in the plain computation of the same thing (``rounded``)."""
+    got, exact = got.float().cpu(), exact.float()
+    err = (got - exact).abs()
+    if dtype == torch.float32:
+        assert float(err.max()) <= 1e-4 * max(1.0, float(exact.abs().max())), f"max err {float(err.max()):.3e}"
+    else:
+        noise = (rounded.float() - exact).abs()
+        assert float(err.max()) <= 2.0 * float(noise.max()), f"max {float(err.max()):.3e} vs noise {float(noise.max()):.3e}"
+        assert float((err ** 2).mean().sqrt()) <= 1.5 * float((noise ** 2).mean().sqrt())
+
+
+def one_seq_context(n_new, n_cached, runner, req="r"):
+    """A StepContext for one request bringing n_new tokens after n_cached cached ones."""
+    from pico_vllm_amd.engine.batch import SeqStep, build_context
+    m = runner.manager
+    if req not in m.requests:
+        m.add_request(req)
+    m.advance(req, n_cached)
+    assert m.grow(req, n_cached + n_new)
+    seq = SeqStep(req, [0] * n_new, [])
+    return build_context([seq], m, runner.buffers, runner.model.dtype, runner.model.spec.vocab_size)
+
+
+def runner_for(name, dtype):
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import load_model
+    model = load_model(model_dir(name), "float32" if dtype == torch.float32 else "bfloat16", DEV)
+    return ModelRunner(model, PAGE_SIZE[name], 64, 4, 256, 256)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_attention_and_mlp_and_block_parts(name, dtype):
+    r = runner_for(name, dtype)
+    plain = P.PlainModel(model_dir(name))
+    cfg = plain.cfg
+    H, S = cfg.hidden_size, 37
+    blk = r.model.layers[0]
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(S, H, generator=g)
+    h = x.to(dtype)
+    pos = torch.arange(S)
+    # mixer alone: whole sequence in one step, then the same in two portions through the cache
+    ctx = one_seq_context(S, 0, r)
+    out = blk.mixer.forward(h.to(DEV), ctx, r.storage.layer(0))
+    want = P.attention_layer(h.float(), plain.w, "model.layers.0", cfg, pos)
+    rounded = P.attention_layer(h.float(), plain.w, "model.layers.0", cfg, pos, rnd=P.to_bf16)
+    close_to_plain(out, want, rounded, dtype)
+    r.manager.free_request("r")
+    ctx = one_seq_context(20, 0, r)
+    first = blk.mixer.forward(h[:20].to(DEV), ctx, r.storage.layer(0))
+    ctx = one_seq_context(S - 20, 20, r)
+    second = blk.mixer.forward(h[20:].to(DEV), ctx, r.storage.layer(0))
+    close_to_plain(torch.cat([first, second]), want, rounded, dtype)
+    # feed-forward alone
+    f = blk.parts["ff"].forward(h.to(DEV), ctx)
+    wantf = P.mlp_layer(h.float(), plain.w, "model.layers.0")
+    close_to_plain(f, wantf, P.mlp_layer(h.float(), plain.w, "model.layers.0", rnd=P.to_bf16), dtype)
+    # norm alone (the part, with the fused add)
+    delta = torch.randn(S, H, generator=g).to(dtype)
+    resid = x.clone().to(DEV)
+    n = blk.parts["norm1"].add_norm(resid, delta.to(DEV))
+    close(n, P.rms_norm(x + delta.float(), plain.w["model.layers.0.input_layernorm.weight"], cfg.rms_norm_eps), dtype, 3)
+    # the whole block: pending delta in, pending delta out
+    r.manager.free_request("r")
+    ctx = one_seq_context(S, 0, r)
+    resid = x.clone().to(DEV)
+    resid2, pending = blk.forward(resid, None, ctx, r.storage.layer(0))
+    wantb = P.block(x, plain.w, 0, cfg, pos)
+    close_to_plain(resid2 + pending.float(), wantb, P.block(x, plain.w, 0, cfg, pos, rnd=P.to_bf16), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part_with_a_window(dtype):
+    """The same mixer class with window = 24: its cache group gives pages back, and the result is
+    the plain windowed attention."""
+    from pico_vllm_amd.cache.manager import CacheManager
+    from pico_vllm_amd.cache.storage import CacheStorage
+    from pico_vllm_amd.engine.batch import BatchBuffers, SeqStep, build_context
+    from pico_vllm_amd.parts.registry import build_part
+    from pico_vllm_amd.parts.spec import PartSpec
+    H, nq, nkv, d, W, Pg = 96, 6, 2, 16, 24, 8
+    spec = PartSpec("gqa_attention", dict(hidden_size=H, num_heads=nq, num_kv_heads=nkv, head_dim=d, qkv_bias=True,
+                                          window=W, position=PartSpec("rotary_half", {"rotary_dim": d, "theta": 1e4})))
+    mixer = build_part("mixer", spec, act_dtype=dtype)
+    g = torch.Generator().manual_seed(1)
+    w = {p.name: (torch.randn(p.shape, generator=g) * (0.3 if p.role == "matrix" else 0.1)).to(torch.bfloat16)
+         for p in mixer.param_specs()}
+    mixer.load({k: v.to(dtype) for k, v in w.items()}, torch.device(DEV), dtype)
+    mgr = CacheManager({0: mixer.cache_spec()}, Pg, 8, 1)          # 8 pages of 8: a 100-token request only fits
+    store = CacheStorage(mgr, {0: mixer.cache_spec()}, dtype, torch.device(DEV))   # because the window frees pages
+    buf = BatchBuffers(torch.device(DEV), 64, 1, 16, 1)
+    S = 100
+    x = torch.randn(S, H, generator=g).to(dtype)
+    mgr.add_request("r")
+    outs, i = [], 0
+    for n in [13, 2, 30, 1, 1, 17, 36]:
+        assert mgr.grow("r", i + n)
+        ctx = build_context([SeqStep("r", [0] * n, [])], mgr, buf, dtype, 10)
+        outs.append(mixer.forward(x[i:i + n].to(DEV), ctx, store.layer(0)))
+        i += n
+        mgr.advance("r", i)
+        mgr.check()
+    assert i == S and mgr.groups[0].pool.reuse_count > 0
+    # plain: same projections, windowed attention
+    wf = {k: v.float() for k, v in w.items()}
+    qkv = x.float() @ torch.cat([wf["q_proj.weight"], wf["k_proj.weight"], wf["v_proj.weight"]]).T \
+        + torch.cat([wf["q_proj.bias"], wf["k_proj.bias"], wf["v_proj.bias"]])
+    q, k, v = P.split_qkv(qkv, nq, nkv, d)
+    cos, sin = P.rope_tables(torch.arange(S), d, 1e4)
+    o = P.causal_attention(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v, window=W)
+    want = o.reshape(S, nq * d) @ wf["o_proj.weight"].T
+    close(torch.cat(outs), want, dtype, scale=float(want.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_run_order_may_name_a_layer_twice(dtype):
+    """Layers run in the order [0, 1, 0]: layer 0's weights twice, each run with a cache of its own."""
+    import dataclasses
+    from pico_vllm_amd.config.registry import load_model_description
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import DecoderModel
+    from pico_vllm_amd.parts.spec import RunEntry
+    from pico_vllm_amd.weights.loader import load_checkpoint
+    d = model_dir("A")
+    _, cfg, spec = load_model_description(d)
+    spec = dataclasses.replace(spec, run_order=[RunEntry(0), RunEntry(1), RunEntry(0)])
+    model = DecoderModel(spec, dtype, torch.device(DEV))
+    model.load(load_checkpoint(d, model.param_specs(), dtype))
+    assert sorted(model.cache_specs()) == [0, 1, 2]
+    r = ModelRunner(model, 16, 32, 2, 128, 128)
+    plain = P.PlainModel(d)
+    toks = torch.randint(0, 255, (45,), generator=torch.Generator().manual_seed(2)).tolist()
+    x = plain.w["model.embed_tokens.weight"][toks].float()
+    pos = torch.arange(len(toks))
+    for i in (0, 1, 0):
+        x = P.block(x, plain.w, i, plain.cfg, pos)
+    want = P.rms_norm(x, plain.w["model.norm.weight"], plain.cfg.rms_norm_eps) @ plain.w["model.embed_tokens.weight"].T
+    xr = plain.w["model.embed_tokens.weight"][toks].float()
+    for i in (0, 1, 0):
+        xr = P.block(xr, plain.w, i, plain.cfg, pos, rnd=P.to_bf16)
+    rounded = P.to_bf16(P.rms_norm(xr, plain.w["model.norm.weight"], plain.cfg.rms_norm_eps)) \
+        @ plain.w["model.embed_tokens.weight"].T
+    r.manager.add_request("r")
+    got, i = [], 0
+    for n in (20, 3, 1, 21):
+        assert r.manager.grow("r", i + n)
+        seq = [SeqStep("r", toks[i:i + n], list(range(n)))]
+        got.append(r.step(seq))
+        r.advance(seq)
+        i += n
+    close_to_plain(torch.cat(got), want, rounded, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_toy_mixer_with_state_of_its_own_registers_builds_and_steps(dtype):
+    """A mixer that keeps a running mean of its inputs per request (a fixed-size state, no pages)
+    is defined here, registered, put into a new architecture together with the framework's norm
+    and feed-forward, loaded from a random-weights folder and stepped in portions; the framework's
+    files are not changed for it."""
+    import tempfile
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.base import Mixer
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import CacheSpec, LayerSpec, ModelSpec, ParamSpec, PartSpec, RunEntry
+    from pico_vllm_amd.weights.random_init import write_random_model
+
+    @register_part("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """y_t = W * mean(x_0 .. x_t); state per request: [sum (H values), count]."""
+
+        def __init__(self, hidden_size, act_dtype=torch.bfloat16):
+            self.H, self.act_dtype = hidden_size, act_dtype
+
+        def cache_spec(self):
+            return CacheSpec("state", state_shape=(self.H + 1,), state_dtype="float32")
+
+        def param_specs(self):
+            return [ParamSpec("mix.weight", (self.H, self.H), std=0.2)]
+
+        def load(self, tensors, device, dtype):
+            self.w = tensors["mix.weight"].to(device).float()
+
+        def forward(self, x, ctx, cache):
+            out = torch.empty_like(x)
+            cu = ctx.host["cu_seqlens"]
+            slots = ctx.state_slots.tolist()
+            ctxl = ctx.host["context_lens"]
+            for b in range(ctx.num_seqs):
+                lo, hi = int(cu[b]), int(cu[b + 1])
+                st = cache.state[slots[b]]
+                if int(ctxl[b]) - (hi - lo) == 0:
+                    st.zero_()                                  # a new request starts from empty state
+                xs = x[lo:hi].float()
+                sums = st[:self.H] + torch.cumsum(xs, 0)
+                counts = st[self.H] + torch.arange(1, hi - lo + 1, device=x.device)
+                out[lo:hi] = ((sums / counts[:, None]) @ self.w.T).to(x.dtype)
+                st[:self.H] = sums[-1]
+                st[self.H] = counts[-1]
+            return out
+
+    def toy_spec(cfg):
+        H = cfg["hidden_size"]
+        norm = PartSpec("rms_norm", {"size": H, "eps": 1e-5})
+        layers = [LayerSpec(f"toy.layers.{i}", "prenorm", {
+            "norm1": ("ln1", norm), "mixer": ("mixer", PartSpec("toy_running_mean", {"hidden_size": H})),
+            "norm2": ("ln2", norm), "ff": ("mlp", PartSpec("swiglu_mlp", {"hidden_size": H, "intermediate_size": 2 * H}))})
+            for i in range(cfg["num_hidden_layers"])]
+        return ModelSpec(H, cfg["vocab_size"], "toy.embed.weight", layers, [RunEntry(i) for i in range(len(layers))],
+                         norm, "toy.norm", None)
+
+    register_architecture("ToyRunningMeanLM", lambda raw: raw, toy_spec)
+    cfg = {"architectures": ["ToyRunningMeanLM"], "hidden_size": 48, "vocab_size": 100, "num_hidden_layers": 2}
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=0, std_overrides={"mlp": 0.2, "embed": 0.5})
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        r = ModelRunner(model, 16, 4, 3, 64, 64)
+        assert r.manager.state_layers == [0, 1] and not r.manager.groups
+        toks = {"a": list(range(1, 30)), "b": list(range(50, 61))}
+        # whole
+        whole = {}
+        for rid, t in toks.items():
+            r.manager.add_request(rid)
+            s = [SeqStep(rid, t, list(range(len(t))))]
+            whole[rid] = r.step(s)
+            r.manager.free_request(rid)
+        # in portions, both requests in the same steps, state carried between steps in their slots
+        for rid in toks:
+            r.manager.add_request(rid)
+        got = {rid: [] for rid in toks}
+        cuts = {"a": [5, 1, 10, 13], "b": [2, 7, 1, 1]}
+        fed = {rid: 0 for rid in toks}
+        for k in range(4):
+            seqs = []
+            for rid in toks:
+                n = cuts[rid][k]
+                seqs.append(SeqStep(rid, toks[rid][fed[rid]:fed[rid] + n], list(range(n))))
+            out = r.step(seqs)
+            r.advance(seqs)
+            o = 0
+            for s in seqs:
+                got[s.req].append(out[o:o + len(s.tokens)])
+                o += len(s.tokens)
+                fed[s.req] += len(s.tokens)
+        for rid in toks:
+            close(torch.cat(got[rid]), whole[rid], dtype, scale=float(whole[rid].std()) * 3)
+        assert whole["a"].shape == (29, 100) and float(whole["a"].std()) > 0.01

@@ -1,0 +1,292 @@
+"""Trace replay against the plain implementation: the same requests whole, with the last 32
+tokens one by one, in portions of changing size, and mixed with other requests in a pool so small
+that pages are used again; in 32-bit and in bfloat16."""
+import io
+import json
+import os
+import random
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen2 as P
+from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# float32: the engine and the plain implementation differ in summation order only; errors are
+# measured against the spread (standard deviation) of the request's logits.
+# bfloat16: the yardstick is the plain implementation itself with every activation between the
+# parts rounded to bfloat16 (plain_qwen2.to_bf16): how far that moves the logits of this request
+# is the rounding noise of this model at this length.  The engine must stay within a small
+# multiple of it; a fault larger than the rounding noise fails, whatever the model's sensitivity.
+F32_REL_MAX, F32_REL_MEAN = 2e-5, 4e-6
+BF16_RMS_FACTOR, BF16_MAX_FACTOR = 1.5, 2.0
+# The engine stores bfloat16 at the same places where the rounded plain computation rounds (give or
+# take a stage that a fused kernel keeps in registers), so it follows THAT computation much more
+# closely than the exact one: measured 0.00x-0.38x of the rounding noise.
+BF16_VS_ROUNDED_FACTOR = 0.6
+
+
+def make_requests(name, lengths, seed=0):
+    V = CONFIGS[name]["vocab_size"]
+    rng = random.Random(seed)
+    return {f"r{i}": [rng.randrange(V) for _ in range(n)] for i, n in enumerate(lengths)}
+
+
+_plain_cache = {}
+
+
+def plain_logits(name, tokens):
+    key = (name, tuple(tokens))
+    if key not in _plain_cache:
+        if name not in _plain_cache:
+            _plain_cache[name] = P.PlainModel(model_dir(name))
+        _plain_cache[key] = _plain_cache[name].logits(tokens).numpy()
+    return _plain_cache[key]
+
+
+def roundup(n, m=64):
+    return -(-n // m) * m
+
+
+class Trace:
+    """Steps plus the bookkeeping of which (request, position) each output row is."""
+
+    def __init__(self):
+        self.steps, self.rows, self.fed, self.live_peak = [], {}, {}, 0
+
+    def add(self, entries, end=()):
+        """entries: list of (id, tokens, want)."""
+        k = len(self.steps)
+        rows = []
+        for rid, toks, want in entries:
+            base = self.fed.get(rid, 0)
+            rows += [(rid, base + w) for w in want]
+            self.fed[rid] = base + len(toks)
+        self.live_peak = max(self.live_peak, sum(roundup(n) for n in self.fed.values()))
+        self.steps.append({"step": k, "entries": [{"id": r, "tokens": t, "want": list(w)} for r, t, w in entries],
+                           "end": list(end)})
+        self.rows[k] = rows
+        for rid in end:
+            del self.fed[rid]
+
+
+def whole(reqs):
+    t = Trace()
+    for rid, toks in reqs.items():
+        t.add([(rid, toks, range(len(toks)))], end=[rid])
+    return t
+
+
+def tail_one_by_one(reqs, tail=32):
+    t = Trace()
+    for rid, toks in reqs.items():
+        n = max(1, len(toks) - tail)
+        t.add([(rid, toks[:n], range(n))])
+        for i in range(n, len(toks)):
+            t.add([(rid, toks[i:i + 1], [0])], end=[rid] if i == len(toks) - 1 else [])
+        if n == len(toks):
+            t.add([], end=[rid])
+    return t
+
+
+def portions(reqs, sizes=(13, 2, 7, 2, 5, 3, 16, 2, 17, 4, 31, 2, 8)):
+    t = Trace()
+    for rid, toks in reqs.items():
+        i, k = 0, 0
+        while i < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - i)
+            k += 1
+            t.add([(rid, toks[i:i + n], range(n))], end=[rid] if i + n == len(toks) else [])
+            i += n
+    return t
+
+
+def mixed(reqs, seed=0, max_live=4, tail=32):
+    """Up to four live requests; prompt portions of some beside single tokens of others; a request
+    may sit a step out; finished requests end and later ones take their pages."""
+    rng = random.Random(seed)
+    t = Trace()
+    waiting = list(reqs.items())
+    live = {}                                   # id -> [tokens, fed]
+    while waiting or live:
+        while waiting and len(live) < max_live and rng.random() < 0.7:
+            rid, toks = waiting.pop(0)
+            live[rid] = [toks, 0]
+        entries, end = [], []
+        for rid, (toks, fed) in list(live.items()):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                        # left out of this step
+            left = len(toks) - fed
+            n = 1 if left <= tail else min(left - tail, rng.choice([2, 3, 5, 8, 13, 16, 17, 29]))
+            if left - n == 1 and left > tail:
+                n += 1
+            entries.append((rid, toks[fed:fed + n], range(n)))
+            live[rid][1] += n
+            if live[rid][1] == len(toks):
+                end.append(rid)
+                del live[rid]
+        if entries:
+            t.add(entries, end)
+    return t
+
+
+def replay(name, dtype, trace, max_tokens=None):
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    rp = TraceReplayer(model_dir(name), dtype, max_tokens or trace.live_peak, PAGE_SIZE[name])
+    got = {}
+    for step in trace.steps:
+        out = rp.run_step(step)
+        rows = trace.rows[step["step"]]
+        assert (out is None) == (len(rows) == 0)
+        if out is not None:
+            assert out.shape == (len(rows), CONFIGS[name]["vocab_size"]) and out.dtype == np.float32
+            for row, key in zip(out, rows):
+                assert key not in got
+                got[key] = row
+    rp.runner.manager.check()
+    pool = rp.runner.manager.groups[0].pool
+    assert pool.num_free == pool.num_pages and not rp.live
+    return got, pool
+
+
+_noise_cache = {}
+
+
+def bf16_noise(name, tokens):
+    """(rms, max) of the logit error that bfloat16 storage of activations causes in the plain
+    implementation for this request."""
+    key = (name, tuple(tokens))
+    if key not in _noise_cache:
+        plain_logits(name, tokens)
+        rounded = _plain_cache[name].logits(tokens, rnd=P.to_bf16).numpy()
+        err = np.abs(rounded - plain_logits(name, tokens))
+        _noise_cache[key] = (float(np.sqrt((err ** 2).mean())), float(err.max()), rounded)
+    return _noise_cache[key]
+
+
+def compare(name, dtype, reqs, got, label):
+    worst = 0.0
+    for rid, toks in reqs.items():
+        ref = plain_logits(name, toks)
+        spread = float(ref.std())
+        mine = np.stack([got[(rid, p)] for p in range(len(toks))])
+        assert np.isfinite(mine).all()
+        err = np.abs(mine - ref)
+        if dtype == "float32":
+            rel = err.max(axis=1) / spread
+            worst = max(worst, float(rel.max()))
+            assert rel.max() <= F32_REL_MAX, (f"{label} {name} {dtype}: request {rid} first wrong position "
+                                              f"{int(np.argmax(rel > F32_REL_MAX))}, worst {rel.max():.3e} at {int(rel.argmax())}")
+            assert err.mean() / spread <= F32_REL_MEAN, f"{label} {name}: mean error {err.mean() / spread:.3e}"
+        else:
+            noise_rms, noise_max, rounded = bf16_noise(name, toks)
+            rms = float(np.sqrt((err ** 2).mean()))
+            per_pos = np.sqrt((err ** 2).mean(axis=1))
+            worst = max(worst, rms / noise_rms)
+            print(f"[replay] {label} {name} bf16 {rid}: rms {rms / noise_rms:.2f}x max {err.max() / noise_max:.2f}x of the "
+                  f"rounding noise (rms {noise_rms / spread:.2e}, max {noise_max / spread:.2e} of the spread); "
+                  f"vs rounded plain: rms {np.sqrt(((mine - rounded) ** 2).mean()) / noise_rms:.2f}x")
+            assert np.sqrt(((mine - rounded) ** 2).mean()) <= BF16_VS_ROUNDED_FACTOR * noise_rms, \
+                f"{label} {name} bf16: request {rid} strays from the bfloat16-rounded plain computation"
+            assert rms <= BF16_RMS_FACTOR * noise_rms, \
+                f"{label} {name} bf16: request {rid}: rms error {rms / noise_rms:.2f}x the rounding noise"
+            assert err.max() <= BF16_MAX_FACTOR * noise_max, \
+                (f"{label} {name} bf16: request {rid}: max error {err.max() / noise_max:.2f}x the rounding noise, "
+                 f"first position above it {int(np.argmax(err.max(axis=1) > BF16_MAX_FACTOR * noise_max))}")
+            # no single position stands out: a fault at a page edge or at the start of a portion would
+            assert per_pos.max() <= 4.0 * BF16_RMS_FACTOR * noise_rms, \
+                f"{label} {name} bf16: request {rid}: position {int(per_pos.argmax())} is {per_pos.max() / noise_rms:.2f}x the noise"
+    print(f"[replay] {label} {name} {dtype}: worst {worst:.3e}")
+
+
+LENGTHS = {"A": [70, 45, 100, 33, 64, 90], "B": [41, 97, 34, 80, 65, 50], "C": [50, 36, 81]}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(name, dtype):
+    reqs = make_requests(name, LENGTHS[name])
+    got, _ = replay(name, dtype, whole(reqs))
+    compare(name, dtype, reqs, got, "whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_32_tokens_one_by_one(name, dtype):
+    reqs = make_requests(name, LENGTHS[name][:3], seed=1)
+    got, _ = replay(name, dtype, tail_one_by_one(reqs))
+    compare(name, dtype, reqs, got, "tail")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(name, dtype):
+    reqs = make_requests(name, LENGTHS[name][:4], seed=2)
+    got, _ = replay(name, dtype, portions(reqs))
+    compare(name, dtype, reqs, got, "portions")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_with_pages_used_again(name, dtype):
+    reqs = make_requests(name, LENGTHS[name] + [57, 38], seed=3)
+    trace = mixed(reqs, seed=4)
+    assert max(len(s["entries"]) for s in trace.steps) >= 3
+    got, pool = replay(name, dtype, trace)
+    assert pool.reuse_count > 0 and pool.peak_used > pool.num_pages // 2      # pages were used again
+    compare(name, dtype, reqs, got, "mixed")
+
+
+def test_float32_does_not_depend_on_the_cut_at_all():
+    # every reduction of the 32-bit path has a fixed order per output element: bitwise equal
+    reqs = make_requests("B", [77, 40], seed=5)
+    a, _ = replay("B", "float32", whole(reqs))
+    b, _ = replay("B", "float32", portions(reqs))
+    c, _ = replay("B", "float32", mixed(reqs, seed=6))
+    for key in a:
+        assert np.array_equal(a[key], b[key]) and np.array_equal(a[key], c[key]), key
+
+
+def test_long_decoding_and_first_tokens():
+    # 300 tokens one by one from the very first token (position 0, a cache of one key) on
+    reqs = make_requests("A", [300], seed=7)
+    toks = reqs["r0"]
+    t = Trace()
+    for i in range(len(toks)):
+        t.add([("r0", toks[i:i + 1], [0])], end=["r0"] if i == len(toks) - 1 else [])
+    for dtype in ("float32", "bfloat16"):
+        got, _ = replay("A", dtype, t)
+        compare("A", dtype, reqs, got, "long decode")
+        first = np.stack([got[("r0", p)] for p in range(4)])
+        ref = plain_logits("A", toks)[:4]
+        bound = F32_REL_MAX * ref.std() if dtype == "float32" else BF16_MAX_FACTOR * bf16_noise("A", toks)[1]
+        assert np.abs(first - ref).max() <= bound
+
+
+def test_the_program_itself_in_a_subprocess():
+    reqs = make_requests("A", [40, 23], seed=8)
+    trace = mixed(reqs, seed=9)
+    with tempfile.TemporaryDirectory() as out:
+        inp = "\n".join(json.dumps(s) for s in trace.steps) + "\n"
+        r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir("A"), "--dtype", "float32",
+                            "--out", out, "--max-tokens", str(trace.live_peak)],
+                           input=inp, capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, r.stderr[-2000:]
+        assert r.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in trace.steps]
+        got = {}
+        for s in trace.steps:
+            rows = trace.rows[s["step"]]
+            path = os.path.join(out, f"{s['step']}.f32")
+            assert os.path.exists(path) == bool(rows)
+            if rows:
+                a = np.fromfile(path, dtype="<f4").reshape(len(rows), -1)
+                for row, key in zip(a, rows):
+                    got[key] = row
+        compare("A", "float32", reqs, got, "program")

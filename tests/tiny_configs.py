@@ -26,11 +26,18 @@ CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 _made = {}
 
 
-# larger q/k/v/o and MLP matrices than N(0, 0.02): attention scores then spread over several units and
-# the layers change the residual stream visibly, so a wrong rotation, mask or page shows in the logits
-STRONG = {"q_proj.weight": 0.25, "k_proj.weight": 0.25, "v_proj.weight": 0.1, "o_proj.weight": 0.1,
-          "gate_proj": 0.1, "up_proj": 0.1, "down_proj": 0.1, "_proj.bias": 0.2, "embed_tokens": 0.1,
-          "lm_head": 0.1}
+def strong(config) -> dict:
+    """Standard deviations larger than N(0, 0.02), so that a fault shows in the logits: with q and k
+    weights of sqrt(3 / hidden) the attention scores have a spread of about 3, which makes attention
+    pick out keys (a wrong rotation, mask or page changes the result) without making the softmax so
+    sharp that rounding is amplified; the other matrices change the residual stream visibly."""
+    qk = (3.0 / config["hidden_size"]) ** 0.5
+    return {"q_proj.weight": qk, "k_proj.weight": qk, "v_proj.weight": 0.1, "o_proj.weight": 0.1,
+            "gate_proj": 0.1, "up_proj": 0.1, "down_proj": 0.1, "_proj.bias": 0.2, "embed_tokens": 0.1,
+            "lm_head": 0.1}
+
+
+STRONG = strong(TINY_B)
 
 
 def model_dir(name: str, seed: int = 0, strong: bool = True) -> str:
@@ -39,6 +46,6 @@ def model_dir(name: str, seed: int = 0, strong: bool = True) -> str:
     key = (name, seed, strong)
     if key not in _made:
         d = tempfile.mkdtemp(prefix=f"pico_tiny_{name}_")
-        write_random_model(d, CONFIGS[name], seed, STRONG if strong else None)
+        write_random_model(d, CONFIGS[name], seed, globals()['strong'](CONFIGS[name]) if strong else None)
         _made[key] = d
     return _made[key]
