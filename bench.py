@@ -68,10 +68,12 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
     eng = make_engine(model_dir, dtype, batch, model)
     V = CONFIG_1P5B["vocab_size"]
     g = torch.Generator().manual_seed(batch)
-    prompt_len = CONTEXT - (warmup + steps) - 1
+    # while later prompts are still being prefilled the earlier requests already decode: leave room for that
+    slack = batch * (-(-CONTEXT // PREFILL_TOKENS)) + 2
+    prompt_len = CONTEXT - (warmup + steps) - 1 - slack
     for i in range(batch):
         ids = torch.randint(0, V, (prompt_len,), generator=g).tolist()
-        eng.submit(ids, max_new_tokens=warmup + steps + 1, temperature=0.0, ignore_eos=True)
+        eng.submit(ids, max_new_tokens=warmup + steps + 1 + slack, temperature=0.0, ignore_eos=True)
     t0 = time.time()
     while any(r.num_uncomputed > 1 or not r.generated_ids for r in eng.requests.values()):
         eng.step()                                   # prompt portions (and the first decodes of early requests)
@@ -92,7 +94,7 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
     ctx_mean = [c + (steps - 1) / 2 + 1 for c in ctx_start]          # keys read per step, averaged over the region
     nbytes = eng.runner.decode_bytes([int(c) for c in ctx_mean])
     ms = dt / steps * 1e3
-    res = {"tok_s": batch * steps / dt, "ms_per_step": ms, "bytes": nbytes, "gbps": nbytes / (dt / steps) / 1e9,
+    res = {"prompt_len": prompt_len, "tok_s": batch * steps / dt, "ms_per_step": ms, "bytes": nbytes, "gbps": nbytes / (dt / steps) / 1e9,
            "context": sum(ctx_mean) / batch}
     model = eng.model
     del eng
@@ -132,13 +134,14 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
     ap.add_argument("--model", default=None, help="reuse a model folder instead of writing random weights")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
         return 2
-    if a.steps + a.warmup >= CONTEXT // 2:
-        print("bench.py: steps + warmup must stay below 2048")
+    if a.steps + a.warmup >= CONTEXT // 2 - 200:
+        print("bench.py: steps + warmup must stay below 1848")
         return 2
     import torch
     from pico_vllm_amd.weights.random_init import write_random_model
@@ -152,6 +155,9 @@ def main() -> int:
         write_random_model(model_dir, CONFIG_1P5B, seed=0)
         log(f"... {time.time() - t0:.0f}s")
     try:
+        if a.prefill_only:
+            print(json.dumps({"prefill": prefill_point(model_dir, None, a.dtype)}), flush=True)
+            return 0
         main_res, model = decode_point(model_dir, None, a.dtype, a.batch, a.steps, a.warmup)
         log(f"decode batch {a.batch}: {main_res['tok_s']:.0f} tok/s, {main_res['ms_per_step']:.3f} ms/step")
         out = {
@@ -163,8 +169,8 @@ def main() -> int:
             "config": {"model": "Qwen2.5-1.5B shape", "global_batch": a.batch, "seq_len": CONTEXT,
                        "parallelism": "single GPU", "layers": 28, "layers_run": 28, "hidden": 1536, "q_heads": 12,
                        "kv_heads": 2, "head_dim": 128, "intermediate": 8960, "vocab": 151936, "tied": True,
-                       "page_size": 16, "prompt_len": CONTEXT - (a.steps + a.warmup) - 1,
-                       "context_in_timed_steps": round(main_res["context"], 1), "hip_graph": True},
+                       "page_size": 16, "prompt_len": int(main_res["prompt_len"]),
+                       "context_in_timed_steps": round(main_res["context"], 1)},
             "roofline": {"bound": "hbm", "achieved": round(main_res["gbps"], 1), "peak": HBM_PEAK / 1e9,
                          "unit": "GB/s", "frac": round(main_res["gbps"] * 1e9 / HBM_PEAK, 4)},
         }

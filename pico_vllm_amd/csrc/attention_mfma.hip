@@ -1,0 +1,386 @@
+// Paged attention on the matrix cores for bfloat16, specialised at compile time for one head
+// size D = PICO_HEAD_DIM (a multiple of 16 up to 256).  Two kernels share the tile code:
+//
+//   prefill / mixed  one workgroup (4 waves) per 128 query tokens of one sequence and one query
+//                    head; each wave owns 32 queries; keys and values of the sequence stream
+//                    through LDS in tiles of BN keys, from position 0 to the causal frontier.
+//                    A decode token is a sequence that brings one query.
+//   decode           one workgroup (2 waves) per (sequence, kv head, split of the context); the
+//                    "queries" are the G query heads that share the kv head, so keys and values
+//                    are read once for the whole group (the reference's kernel re-reads them per
+//                    query head, pico_vllm/kernels/attention.py:96-105); the waves split the keys;
+//                    partial (max, sum, output) per split are merged by a second kernel.
+//
+// Formulas as in pico_vllm/kernels/attention.py:136-213: scores (q.k) * scale, key visible iff its
+// position <= the query's, online softmax in float32, probabilities rounded to bfloat16 for the
+// P.V product, float32 accumulators.
+//
+// Matrix-core layout (v_mfma_f32_32x32x16_bf16, D = A B, A 32x16, B 16x32): lane l supplies
+// A[l % 32][8 (l / 32) + 0..7] and B[8 (l / 32) + 0..7][l % 32]; it receives, in register r,
+// D[8 (r / 4) + 4 (l / 32) + r % 4][l % 32].  Scores are computed TRANSPOSED, S^T = K Q^T, so a
+// query is a column: its 32 scores of a key tile sit in the 16 registers of two lanes (l, l ^ 32)
+// and the softmax needs one exchange across lanes.  The same registers, rounded to bfloat16, ARE
+// the B operand of O^T += V^T P^T if the contraction index runs over the keys in the order in
+// which the registers hold them; V^T is read from LDS in that order.  That is why the cache
+// keeps V transposed inside a page ([head size][slot]).
+#include "common.h"
+
+#ifndef PICO_HEAD_DIM
+#error "compile with -DPICO_HEAD_DIM=<head size>"
+#endif
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int D = PICO_HEAD_DIM;
+static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
+constexpr int DP = (D + 31) / 32 * 32;   // head size padded to whole 32-wide output tiles
+constexpr int KSTEPS = D / 16;           // contraction steps of K Q^T
+constexpr int DT = DP / 32;              // 32-wide tiles of the output's head dimension
+constexpr int BN = D <= 128 ? 64 : 32;   // keys per LDS tile
+constexpr int KROW = D + 8;              // LDS row strides in elements; the pad spreads rows over banks
+constexpr int VROW = BN + 8;
+constexpr int BM = 128;                  // queries per workgroup in the prefill kernel
+
+struct alignas(16) Tiles {
+  alignas(16) bf16_t k[BN * KROW];    // [key][dim]
+  alignas(16) bf16_t vt[DP * VROW];   // [dim][key]
+};
+
+// Load keys [tile_start, tile_start + BN) of one sequence and kv head into LDS; positions at or
+// beyond kv_end read as zero (their pages may not exist).  P % 8 == 0, tile_start % 8 == 0.
+__device__ __forceinline__ void load_tiles(Tiles& t, const bf16_t* __restrict__ k_cache,
+                                           const bf16_t* __restrict__ v_cache, const int* __restrict__ bt, int g,
+                                           int nkv, int P, int num_pages, int tile_start, int kv_end, int nthreads) {
+  constexpr int KCH = D / 8;  // 16-byte chunks per key
+  for (int c = threadIdx.x; c < BN * KCH; c += nthreads) {
+    const int key = c / KCH, dc = c % KCH;
+    const int pos = tile_start + key;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (pos < kv_end) {
+      const int page = min(max(bt[pos / P], 0), num_pages - 1);
+      v = *reinterpret_cast<const uint4*>(k_cache + (((size_t)page * nkv + g) * P + pos % P) * D + dc * 8);
+    }
+    *reinterpret_cast<uint4*>(&t.k[key * KROW + dc * 8]) = v;
+  }
+  constexpr int VCH = BN / 8;  // 16-byte chunks (8 keys) per head dimension
+  for (int c = threadIdx.x; c < D * VCH; c += nthreads) {
+    const int dim = c / VCH, kc = c % VCH;
+    const int pos = tile_start + kc * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (pos < kv_end) {
+      const int page = min(max(bt[pos / P], 0), num_pages - 1);
+      v = *reinterpret_cast<const uint4*>(v_cache + (((size_t)page * nkv + g) * D + dim) * P + pos % P);
+      if (pos + 8 > kv_end) {  // the tail of the last chunk holds whatever the page held before
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (pos + e >= kv_end) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+        v = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
+    *reinterpret_cast<uint4*>(&t.vt[dim * VROW + kc * 8]) = v;
+  }
+}
+
+__device__ __forceinline__ void zero_pad_rows(Tiles& t, int nthreads) {
+  if (DP > D)
+    for (int i = threadIdx.x; i < (DP - D) * VROW; i += nthreads) t.vt[D * VROW + i] = 0;
+}
+
+// State of one wave: 32 query columns; lane l and lane l ^ 32 share column l % 32.
+struct WaveState {
+  float m, l;        // running maximum and sum of the column
+  f32x16 o[DT];      // O^T tiles: rows = head dimension, column = query
+};
+
+__device__ __forceinline__ void init_state(WaveState& st) {
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int t = 0; t < DT; t++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) st.o[t][r] = 0.f;
+}
+
+// One 32-key sub-tile (keys sub * 32 .. + 31 of the LDS tile) against the wave's 32 query columns.
+// q[step] is the B operand of step `step`; key_pos0 the absolute position of the sub-tile's first
+// key; q_pos the absolute position of this lane's query column (keys beyond it are masked).
+__device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf16x8* q, WaveState& st, float scale,
+                                               int key_pos0, int q_pos, bool need_mask) {
+  const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  f32x16 s;
+#pragma unroll
+  for (int r = 0; r < 16; r++) s[r] = 0.f;
+  const bf16_t* krow = &t.k[(sub * 32 + col) * KROW + 8 * h];
+#pragma unroll
+  for (int step = 0; step < KSTEPS; step++) {
+    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + 16 * step));
+    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q[step], s, 0, 0, 0);
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    float v = s[r] * scale;
+    if (need_mask) {
+      const int kpos = key_pos0 + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (kpos > q_pos) v = -INFINITY;
+    }
+    s[r] = v;
+    mx = fmaxf(mx, v);
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(st.m, mx);
+  const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column with nothing visible yet
+  const float alpha = __expf(st.m - m_use);
+  float sum = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const float p = __expf(s[r] - m_use);
+    s[r] = p;
+    sum += p;
+  }
+  sum += __shfl_xor(sum, 32, 64);
+  st.l = st.l * alpha + sum;
+  st.m = m_new;
+#pragma unroll
+  for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) st.o[tt][r] *= alpha;
+  // P^T as B operand: contraction slot kk of half h in product m is key 16 m + 8 (kk / 4) + 4 h + kk % 4,
+  // which is register 8 m + kk of this lane.
+#pragma unroll
+  for (int m = 0; m < 2; m++) {
+    uint32_t pk[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      pk[i] = (uint32_t)f32_to_bf16(s[8 * m + 2 * i]) | ((uint32_t)f32_to_bf16(s[8 * m + 2 * i + 1]) << 16);
+    const bf16x8 b = __builtin_bit_cast(bf16x8, make_uint4(pk[0], pk[1], pk[2], pk[3]));
+#pragma unroll
+    for (int tt = 0; tt < DT; tt++) {
+      const bf16_t* vrow = &t.vt[(tt * 32 + col) * VROW + sub * 32 + 16 * m + 4 * h];
+      const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+      const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
+      const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+      st.o[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, st.o[tt], 0, 0, 0);
+    }
+  }
+}
+
+// Q^T operand of one query row: 8 consecutive head dimensions per step, 16-byte loads.
+__device__ __forceinline__ void load_q(bf16x8* q, const bf16_t* qrow, bool ok) {
+  const int h = (threadIdx.x & 63) >> 5;
+#pragma unroll
+  for (int step = 0; step < KSTEPS; step++) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (ok) v = *reinterpret_cast<const uint4*>(qrow + 16 * step + 8 * h);
+    q[step] = __builtin_bit_cast(bf16x8, v);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// prefill / mixed batches
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void prefill_kernel(const bf16_t* __restrict__ q, int q_stride,
+                                                      const bf16_t* __restrict__ k_cache,
+                                                      const bf16_t* __restrict__ v_cache,
+                                                      const int* __restrict__ block_table, int max_pages,
+                                                      const int* __restrict__ cu_seqlens,
+                                                      const int* __restrict__ context_lens, int num_seqs,
+                                                      bf16_t* __restrict__ out, int nq, int nkv, int P,
+                                                      int num_pages, float scale) {
+  __shared__ Tiles tiles;
+  // which (sequence, query tile) is this workgroup?  heavy (late) tiles of a sequence come first
+  int b = 0, tile = (int)blockIdx.x, ntiles = 0;
+  for (; b < num_seqs; b++) {
+    ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + BM - 1) / BM;
+    if (tile < ntiles) break;
+    tile -= ntiles;
+  }
+  if (b >= num_seqs) return;
+  tile = ntiles - 1 - tile;
+  const int head = blockIdx.y, g = head / (nq / nkv);
+  const int tok0 = cu_seqlens[b], new_len = cu_seqlens[b + 1] - tok0;
+  const int ctx = context_lens[b], prefix = ctx - new_len;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int* bt = block_table + (size_t)b * max_pages;
+
+  const int q_idx = tile * BM + wave * 32 + col;          // index among the sequence's new tokens
+  const bool q_ok = q_idx < new_len;
+  const int q_pos = prefix + q_idx;
+  bf16x8 qf[KSTEPS];
+  load_q(qf, q + (size_t)(tok0 + (q_ok ? q_idx : 0)) * q_stride + (size_t)head * D, q_ok);
+  const int wave_first_pos = prefix + tile * BM + wave * 32;            // lowest query position of the wave
+  const int wave_last_pos = min(wave_first_pos + 31, ctx - 1);          // highest real one
+  const bool wave_active = tile * BM + wave * 32 < new_len;
+  const int kv_end = min(ctx, prefix + min(new_len, (tile + 1) * BM));  // keys beyond the tile's last query are never needed
+
+  WaveState st;
+  init_state(st);
+  zero_pad_rows(tiles, 256);
+  for (int tile_start = 0; tile_start < kv_end; tile_start += BN) {
+    __syncthreads();
+    load_tiles(tiles, k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start, kv_end, 256);
+    __syncthreads();
+    if (!wave_active) continue;
+#pragma unroll
+    for (int sub = 0; sub < BN / 32; sub++) {
+      const int key0 = tile_start + sub * 32;
+      if (key0 > wave_last_pos) break;                        // wholly beyond the causal frontier of this wave
+      attend_subtile(tiles, sub, qf, st, scale, key0, q_pos, key0 + 31 > wave_first_pos);
+    }
+  }
+  if (!q_ok) return;
+  const float inv_l = 1.0f / st.l;
+  bf16_t* orow = out + ((size_t)(tok0 + q_idx) * nq + head) * D;
+#pragma unroll
+  for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      const int dim = tt * 32 + 8 * a + 4 * h;
+      if (dim < D) {
+        uint2 v;
+        v.x = (uint32_t)f32_to_bf16(st.o[tt][4 * a] * inv_l) | ((uint32_t)f32_to_bf16(st.o[tt][4 * a + 1] * inv_l) << 16);
+        v.y = (uint32_t)f32_to_bf16(st.o[tt][4 * a + 2] * inv_l) | ((uint32_t)f32_to_bf16(st.o[tt][4 * a + 3] * inv_l) << 16);
+        *reinterpret_cast<uint2*>(orow + dim) = v;
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// decode: one query token per sequence, the G heads of a kv group as the 32 columns
+// ---------------------------------------------------------------------------
+// partial results per (sequence, query head, split): o [D] unnormalised, then m and l
+__global__ __launch_bounds__(128) void decode_kernel(const bf16_t* __restrict__ q, int q_stride,
+                                                     const bf16_t* __restrict__ k_cache,
+                                                     const bf16_t* __restrict__ v_cache,
+                                                     const int* __restrict__ block_table, int max_pages,
+                                                     const int* __restrict__ context_lens,
+                                                     float* __restrict__ part, int nsplit, int nq, int nkv, int P,
+                                                     int num_pages, float scale) {
+  __shared__ Tiles tiles;
+  const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  const int G = nq / nkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int ctx = context_lens[b];
+  // this split's keys: a whole number of LDS tiles
+  const int per = ((ctx + nsplit - 1) / nsplit + BN - 1) / BN * BN;
+  const int k_begin = split * per, k_end = min(ctx, k_begin + per);
+  const int* bt = block_table + (size_t)b * max_pages;
+  const bool col_ok = col < G;
+  const int head = g * G + (col_ok ? col : 0);
+  bf16x8 qf[KSTEPS];
+  load_q(qf, q + (size_t)b * q_stride + (size_t)head * D, col_ok && ctx > 0);
+
+  WaveState st;
+  init_state(st);
+  zero_pad_rows(tiles, 128);
+  for (int tile_start = k_begin; tile_start < k_end; tile_start += BN) {
+    __syncthreads();
+    load_tiles(tiles, k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start, k_end, 128);
+    __syncthreads();
+    for (int sub = wave; sub < BN / 32; sub += 2) {
+      const int key0 = tile_start + sub * 32;
+      if (key0 >= k_end) break;
+      // every query sits at position ctx - 1: only keys at or beyond k_end need the mask
+      attend_subtile(tiles, sub, qf, st, scale, key0, k_end - 1, key0 + 32 > k_end);
+    }
+  }
+  // merge the two waves through LDS (reusing the tile memory), then write the split's partial result
+  __syncthreads();
+  float* xo = reinterpret_cast<float*>(&tiles);            // [DP][32] output of wave 1
+  float* xm = xo + DP * 32;                                // [32] m, [32] l
+  static_assert(sizeof(Tiles) >= (DP * 32 + 64) * sizeof(float), "LDS tile memory too small for the merge");
+  if (wave == 1) {
+#pragma unroll
+    for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) xo[(tt * 32 + 8 * (r >> 2) + 4 * h + (r & 3)) * 32 + col] = st.o[tt][r];
+    if (h == 0) { xm[col] = st.m; xm[32 + col] = st.l; }
+  }
+  __syncthreads();
+  if (wave != 0 || !col_ok) return;
+  const float m1 = xm[col], l1 = xm[32 + col];
+  const float m = fmaxf(st.m, m1);
+  const float m_use = (m == -INFINITY) ? 0.f : m;
+  const float a0 = __expf(st.m - m_use), a1 = __expf(m1 - m_use);
+  const float l = st.l * a0 + l1 * a1;
+  float* po = part + (((size_t)b * nq + head) * nsplit + split) * (D + 2);
+#pragma unroll
+  for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int dim = tt * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (dim < D) po[dim] = st.o[tt][r] * a0 + xo[dim * 32 + col] * a1;
+    }
+  if (h == 0) { po[D] = m; po[D + 1] = l; }
+}
+
+// out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s
+__global__ void decode_merge_kernel(const float* __restrict__ part, int nsplit, bf16_t* __restrict__ out, int nq) {
+  const int b = blockIdx.x, head = blockIdx.y;
+  const float* p = part + ((size_t)b * nq + head) * nsplit * (D + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; s++) M = fmaxf(M, p[s * (D + 2) + D]);
+  bf16_t* o = out + ((size_t)b * nq + head) * D;
+  if (M == -INFINITY) {   // an empty row (padding of a captured batch)
+    for (int dim = threadIdx.x; dim < D; dim += blockDim.x) o[dim] = 0;
+    return;
+  }
+  float L = 0.f;
+  for (int s = 0; s < nsplit; s++) L += __expf(p[s * (D + 2) + D] - M) * p[s * (D + 2) + D + 1];
+  const float inv = 1.0f / L;
+  for (int dim = threadIdx.x; dim < D; dim += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < nsplit; s++) acc += __expf(p[s * (D + 2) + D] - M) * p[s * (D + 2) + dim];
+    o[dim] = f32_to_bf16(acc * inv);
+  }
+}
+
+static int check_common(const char* who, int nq, int nkv, int d, int P, int max_pages, int num_pages, int q_stride) {
+  PICO_REQUIRE(d == D, "%s: this library is built for head size %d, got %d", who, D, d);
+  PICO_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "%s: %d query heads are not a multiple of %d kv heads", who, nq, nkv);
+  PICO_REQUIRE(P > 0 && P % 8 == 0, "%s: page size %d is not a multiple of 8", who, P);
+  PICO_REQUIRE(max_pages > 0 && num_pages > 0, "%s: empty block table or cache", who);
+  PICO_REQUIRE(q_stride >= nq * D && q_stride % 8 == 0, "%s: query row stride %d must be a multiple of 8 and hold all heads", who, q_stride);
+  return 0;
+}
+
+extern "C" int pico_attn_head_dim() { return D; }
+
+extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                 const int* block_table, int max_pages, const int* cu_seqlens,
+                                 const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
+                                 int d, int P, int num_pages, float scale, hipStream_t stream) {
+  if (check_common("pico_attn_prefill", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
+  PICO_REQUIRE(num_seqs > 0 && num_tokens >= num_seqs, "pico_attn_prefill: bad batch (%d sequences, %d tokens)", num_seqs, num_tokens);
+  PICO_REQUIRE(nq <= 65535, "pico_attn_prefill: too many heads");
+  PICO_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "pico_attn_prefill: misaligned tensors");
+  const int max_tiles = num_tokens / BM + num_seqs;       // >= sum over sequences of ceil(len / BM)
+  dim3 grid(max_tiles, nq);
+  prefill_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                          block_table, max_pages, cu_seqlens, context_lens, num_seqs, (bf16_t*)out,
+                                          nq, nkv, P, num_pages, scale);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// part: float32 workspace of num_seqs * nq * nsplit * (D + 2) entries
+extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                const int* block_table, int max_pages, const int* context_lens, int num_seqs,
+                                void* out, float* part, int nsplit, int nq, int nkv, int d, int P, int num_pages,
+                                float scale, hipStream_t stream) {
+  if (check_common("pico_attn_decode", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
+  PICO_REQUIRE(nq / nkv <= 32, "pico_attn_decode: %d query heads per kv head are more than 32", nq / nkv);
+  PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= 65535 && nkv <= 65535, "pico_attn_decode: bad sizes");
+  PICO_REQUIRE(((uintptr_t)q % 16 == 0), "pico_attn_decode: misaligned queries");
+  dim3 grid(num_seqs, nkv, nsplit);
+  decode_kernel<<<grid, 128, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                         block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
+                                         scale);
+  PICO_LAUNCH_CHECK();
+  dim3 mgrid(num_seqs, nq);
+  decode_merge_kernel<<<mgrid, 64, 0, stream>>>(part, nsplit, (bf16_t*)out, nq);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

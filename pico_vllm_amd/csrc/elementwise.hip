@@ -5,18 +5,6 @@
 // in both engine dtypes.
 #include "common.h"
 
-#include <stdarg.h>
-#include <stdio.h>
-
-static thread_local char g_error[512] = "";
-extern "C" const char* pico_last_error() { return g_error; }
-void pico_set_error(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_error, sizeof(g_error), fmt, ap);
-  va_end(ap);
-}
-
 // ---------------------------------------------------------------------------
 // embedding: out[t, :] = table[ids[t], :] as float32.  An id outside [0, V) gives a
 // row of zeros (the host checks ids before a step; this only keeps the kernel in bounds).

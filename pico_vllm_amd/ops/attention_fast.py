@@ -1,8 +1,97 @@
-"""Choice of the matrix-core attention kernels for the bfloat16 engine."""
+"""The matrix-core attention kernels of the bfloat16 engine and the choice between them."""
 from __future__ import annotations
 
+import ctypes
+from typing import Optional
 
-def choose(nq: int, nkv: int, head_dim: int, window: int):
-    """A callable (qkv, cache, block_table, ctx, scale) -> [T, nq*d], or None when the
-    sizes are outside what the fast kernels take (the plain kernel serves them)."""
-    return None
+import torch
+
+from . import library
+from .kernels import KernelError, _check, _check_cache, _ptr, _stream
+
+c_float = ctypes.c_float
+
+
+def supported(nq: int, nkv: int, head_dim: int, window: int) -> bool:
+    """Head sizes in steps of 16 up to 256, no window; anything else goes to the plain kernel."""
+    return head_dim % 16 == 0 and 16 <= head_dim <= 256 and window == 0 and nq % nkv == 0
+
+
+class FastAttention:
+    def __init__(self, nq: int, nkv: int, head_dim: int):
+        self.nq, self.nkv, self.d = nq, nkv, head_dim
+        self.lib = library.attention_library(head_dim)
+        if self.lib.pico_attn_head_dim() != head_dim:
+            raise KernelError("attention library was built for another head size")
+
+    def num_splits(self, num_seqs: int, max_context: int) -> int:
+        """Enough workgroups to fill the chip (256 CUs, several workgroups each), but no split
+        shorter than 256 keys."""
+        by_fill = max(1, 1024 // max(1, num_seqs * self.nkv))
+        by_len = max(1, -(-max_context // 256))
+        return max(1, min(by_fill, by_len, 64))
+
+    def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
+                scale: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """q [T, >= nq*d] bfloat16 (row stride free); any mixture of portions; returns [T, nq*d]."""
+        nq, nkv, d = self.nq, self.nkv, self.d
+        T = q.shape[0]
+        pages, P = _check_cache(k_cache, v_cache, nkv, d)
+        self._check_q(q, k_cache)
+        self._check_meta(block_table, cu_seqlens, num_seqs + 1, context_lens, num_seqs)
+        if out is None:
+            out = torch.empty(T, nq * d, dtype=torch.bfloat16, device=q.device)
+        _check(self.lib, self.lib.pico_attn_prefill(
+            _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(cu_seqlens), _ptr(context_lens), num_seqs, T, _ptr(out), nq, nkv, d, P, pages, c_float(scale),
+            _stream()))
+        return out
+
+    def decode(self, q: torch.Tensor, k_cache, v_cache, block_table, context_lens, num_seqs: int, scale: float,
+               nsplit: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """One query token per sequence: q [B, >= nq*d]; returns [B, nq*d]."""
+        nq, nkv, d = self.nq, self.nkv, self.d
+        if q.shape[0] != num_seqs:
+            raise KernelError("decode attention wants exactly one query token per sequence")
+        if nq // nkv > 32:
+            raise KernelError("decode attention handles at most 32 query heads per kv head")
+        pages, P = _check_cache(k_cache, v_cache, nkv, d)
+        self._check_q(q, k_cache)
+        self._check_meta(block_table, None, 0, context_lens, num_seqs)
+        if out is None:
+            out = torch.empty(num_seqs, nq * d, dtype=torch.bfloat16, device=q.device)
+        part = torch.empty(num_seqs * nq * nsplit * (d + 2), dtype=torch.float32, device=q.device)
+        _check(self.lib, self.lib.pico_attn_decode(
+            _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(context_lens), num_seqs, _ptr(out), _ptr(part), nsplit, nq, nkv, d, P, pages, c_float(scale),
+            _stream()))
+        return out
+
+    def _check_q(self, q, k_cache):
+        if not q.is_cuda or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
+            raise KernelError("matrix-core attention wants bfloat16 tensors on the GPU")
+        if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < self.nq * self.d:
+            raise KernelError("q must be [T, >= nq*d] with unit stride along the row")
+
+    @staticmethod
+    def _check_meta(block_table, cu_seqlens, n_cu, context_lens, num_seqs):
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous() \
+                or block_table.shape[0] < num_seqs:
+            raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+        for t, n in ((cu_seqlens, n_cu), (context_lens, num_seqs)):
+            if t is not None and (t.dtype != torch.int32 or t.numel() < n or not t.is_contiguous()):
+                raise KernelError("sequence metadata must be contiguous int32")
+
+    def __call__(self, qkv, cache, block_table, ctx, scale):
+        if ctx.all_decode and self.nq // self.nkv <= 32:
+            return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, ctx.num_seqs, scale,
+                               self.num_splits(ctx.num_seqs, ctx.max_context))
+        return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, ctx.num_seqs, scale)
+
+
+def choose(nq: int, nkv: int, head_dim: int, window: int) -> Optional[FastAttention]:
+    """The matrix-core kernels for these sizes, or None when they are outside what the kernels
+    take (the plain kernel then serves them)."""
+    if not supported(nq, nkv, head_dim, window):
+        return None
+    return FastAttention(nq, nkv, head_dim)

@@ -27,7 +27,9 @@ HIP_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
 
-CORE_SOURCES = ("elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_ref.hip", "sampling.hip")
+CORE_SOURCES = ("errors.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_ref.hip", "sampling.hip")
+
+ATTN_SOURCES = ("errors.hip", "attention_mfma.hip")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 
@@ -134,13 +136,13 @@ def core() -> ctypes.CDLL:
 
 def attention_library(head_dim: int) -> ctypes.CDLL:
     """Matrix-core attention kernels specialised for one head size."""
-    return load_library(f"pico_attn_d{head_dim}", ("attention_mfma.hip",), (f"-DPICO_HEAD_DIM={head_dim}",))
+    return load_library(f"pico_attn_d{head_dim}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={head_dim}",))
 
 
-def build_all(head_dims: Iterable[int] = (16, 32, 64, 128), force: bool = True) -> List[str]:
+def build_all(head_dims: Iterable[int] = (16, 32, 48, 64, 80, 128, 256), force: bool = True) -> List[str]:
     """Compile everything (used by the build check); returns the paths."""
     out = [build_library("pico_core", CORE_SOURCES, force=force)]
     if os.path.isfile(os.path.join(CSRC, "attention_mfma.hip")):
         for d in head_dims:
-            out.append(build_library(f"pico_attn_d{d}", ("attention_mfma.hip",), (f"-DPICO_HEAD_DIM={d}",), force=force))
+            out.append(build_library(f"pico_attn_d{d}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={d}",), force=force))
     return out

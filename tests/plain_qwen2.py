@@ -112,7 +112,7 @@ def split_qkv(qkv: torch.Tensor, n_q: int, n_kv: int, d: int):
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                      q_positions: Optional[torch.Tensor] = None,
-                     window: int = 0) -> torch.Tensor:
+                     window: int = 0, rnd_p=None) -> torch.Tensor:
     """q: [M, nq, d]; k, v: [N, nkv, d]; returns [M, nq, d].
 
     Query head h reads KV head h // (nq/nkv) (kernels/attention.py:31,139).
@@ -121,7 +121,9 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     over visible keys; weighted sum of V.  Without q_positions the M queries
     are the last M of the N positions (tests/test_prefill_paged_attn.py:38-44).
     ``window`` > 0 additionally hides keys with n <= p - window (not in the
-    reference; used only for the windowed-attention part test)."""
+    reference; used only for the windowed-attention part test).  ``rnd_p``
+    rounds the probabilities before they multiply V, as the reference's
+    prefill kernel does in bfloat16 (attention.py:206)."""
     M, nq, d = q.shape
     N, nkv, _ = k.shape
     G = nq // nkv
@@ -138,6 +140,8 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         s = (q[:, h, :].float() @ k[:, g, :].float().T) * scale
         s = s.masked_fill(~visible, float("-inf"))
         p = torch.softmax(s, dim=-1)
+        if rnd_p is not None:
+            p = rnd_p(p)
         out[:, h, :] = p @ v[:, g, :].float()
     return out
 
@@ -174,7 +178,7 @@ def attention_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
     q, k, v = split_qkv(qkv, nq, nkv, d)
     cos, sin = rope_tables(positions, d, cfg.rope_theta)
     q, k = rnd(apply_rope(q, cos, sin)), rnd(apply_rope(k, cos, sin))
-    o = rnd(causal_attention(q, k, v, q_positions=positions - positions[0]))
+    o = rnd(causal_attention(q, k, v, q_positions=positions - positions[0], rnd_p=None if rnd is _same else rnd))
     return rnd(o.reshape(h.shape[0], nq * d) @ w[f"{prefix}.self_attn.o_proj.weight"].T)
 
 

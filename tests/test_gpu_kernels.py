@@ -270,3 +270,77 @@ def test_sampling_top_p(K):
         assert float(p[int(out[r])]) > 0
         want = P.inverse_cdf(p, float(us[r]))
         assert abs(int(out[r]) - want) <= 0 or abs(float(torch.cumsum(p, 0)[min(int(out[r]), want)]) - float(us[r])) < 1e-4
+
+
+# ---- matrix-core attention (bfloat16) ----------------------------------------------------------
+def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1):
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(seed)
+    totals = [n + p for n, p in zip(new_lens, prefix_lens)]
+    ks = [torch.randn(N, nkv, d, generator=g).to(dtype).float() for N in totals]
+    vs = [torch.randn(N, nkv, d, generator=g).to(dtype).float() for N in totals]
+    qs = [torch.randn(n, nq, d, generator=g).to(dtype).float() for n in new_lens]
+    if boost is not None:
+        boost(qs, ks, vs)
+    num_pages = sum(-(-N // Pg) for N in totals) + 3
+    kc, vc, bt = paged_cache(ks, vs, Pg, num_pages, dtype, seed)
+    B = len(new_lens)
+    cu = torch.tensor([0] + list(torch.tensor(new_lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    ctxl = torch.tensor(totals, dtype=torch.int32, device=DEV)
+    # queries live inside a wider buffer, as q does inside the qkv activations
+    T = sum(new_lens)
+    wide = torch.zeros(T, (nq + 2 * nkv) * d, dtype=dtype, device=DEV)
+    wide[:, :nq * d] = torch.cat(qs, 0).reshape(T, nq * d).to(DEV, dtype)
+    fa = FastAttention(nq, nkv, d)
+    scale = 1.0 / math.sqrt(d)
+    if decode:
+        out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
+    else:
+        out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale)
+    want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n))
+                      for qb, kb, vb, n, p in zip(qs, ks, vs, new_lens, prefix_lens)], 0)
+    return out.reshape(-1, nq, d), want
+
+
+@pytest.mark.parametrize("case", range(len(REFERENCE_CASES)))
+def test_fast_prefill_on_the_reference_cases(K, case):
+    new_lens, prefix_lens = REFERENCE_CASES[case]
+    out, want = _fast_case(new_lens, prefix_lens, 12, 2, 128, 16, seed=case)
+    close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(4, 1, 16, 16), (6, 3, 32, 8), (5, 5, 48, 16), (3, 1, 80, 32), (8, 2, 256, 64),
+                                        (2, 2, 64, 8), (12, 2, 128, 16)])
+def test_fast_prefill_other_sizes_and_long_portions(K, nq, nkv, d, Pg):
+    # portions longer than one 128-query tile, a decode token, a 2-token portion, long prefixes
+    out, want = _fast_case([7, 1, 300, 2, 129], [0, 70, 45, 129, 500], nq, nkv, d, Pg, seed=3)
+    close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(4, 1, 16, 16), (6, 3, 32, 8), (5, 5, 48, 16), (3, 1, 80, 32), (8, 2, 256, 64),
+                                        (12, 2, 128, 16), (32, 1, 64, 16)])
+@pytest.mark.parametrize("nsplit", [1, 3, 8])
+def test_fast_decode(K, nq, nkv, d, Pg, nsplit):
+    out, want = _fast_case([1, 1, 1, 1, 1], [0, 70, 45, 129, 1000], nq, nkv, d, Pg, seed=4, decode=True, nsplit=nsplit)
+    close(out, want, torch.bfloat16)
+
+
+def test_fast_kernels_find_one_far_key_among_hundreds(K):
+    for far in (0, 15, 16, 31, 32, 63, 64, 127, 128, 200, 511, 596):
+        def boost(qs, ks, vs, far=far):
+            ks[0][far] = qs[0][-1, 0:1, :] * 2.0
+            vs[0][far] = 100.0
+        out, want = _fast_case([3], [597], 2, 1, 64, 16, seed=far, boost=boost)
+        assert float(want[-1, 0].mean()) > 50
+        close(out, want, torch.bfloat16, scale=100)
+        for nsplit in (1, 4):
+            out, want = _fast_case([1], [599], 2, 1, 64, 16, seed=far, boost=boost, decode=True, nsplit=nsplit)
+            assert float(want[-1, 0].mean()) > 50
+            close(out, want, torch.bfloat16, scale=100)
+
+
+def test_fast_kernels_refuse_what_they_cannot_do(K):
+    from pico_vllm_amd.ops.attention_fast import choose, supported
+    assert choose(4, 2, 24, 0) is None and choose(4, 2, 512, 0) is None and choose(4, 2, 64, 16) is None
+    assert supported(12, 2, 128, 0)

@@ -27,10 +27,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # multiple of it; a fault larger than the rounding noise fails, whatever the model's sensitivity.
 F32_REL_MAX, F32_REL_MEAN = 2e-5, 4e-6
 BF16_RMS_FACTOR, BF16_MAX_FACTOR = 1.5, 2.0
-# The engine stores bfloat16 at the same places where the rounded plain computation rounds (give or
-# take a stage that a fused kernel keeps in registers), so it follows THAT computation much more
-# closely than the exact one: measured 0.00x-0.38x of the rounding noise.
-BF16_VS_ROUNDED_FACTOR = 0.6
+# The engine stores bfloat16 where the rounded plain computation rounds (activations between parts,
+# probabilities before P.V), so it follows THAT computation at least as closely as the exact one:
+# where both round the same value the errors cancel (measured 0.0x-0.4x with the plain attention
+# kernel); where the rounded values differ slightly (the matrix-core kernel rounds unnormalised
+# probabilities of an online softmax) the two rounding patterns are independent (measured 0.6x-0.7x).
+BF16_VS_ROUNDED_FACTOR = 1.0
 
 
 def make_requests(name, lengths, seed=0):
