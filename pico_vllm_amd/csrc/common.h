@@ -32,12 +32,12 @@ typedef uint16_t bf16_t;  // raw bfloat16 bits
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round to nearest even; NaN stays NaN
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+// round to nearest even; on gfx950 the cast is one v_cvt_pk_bf16_f32
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
+
+// two floats as two bfloat16 in one 32-bit word (a in the low half)
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
 }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p);

@@ -41,12 +41,14 @@ extern "C" int pico_embedding(const void* table, int table_dtype, const int* ids
 // kernels/fused_add_norm.py:21-36, but does not call it):
 //   rows == nullptr:  resid[t] += delta[t] (if delta);  out[t] = norm(resid[t])
 //   rows != nullptr:  out[i] = norm(resid[rows[i]] + delta[rows[i]]);  resid unchanged
+// delta may come as `slabs` partial sums (slab s at delta + s * slab_stride), which a GEMM that
+// splits its k range over workgroups leaves behind; they are added in slab order.
 // One workgroup per row.  The sum of squares is taken over the float32 sum.
 // ---------------------------------------------------------------------------
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    const float* __restrict__ w, TO* __restrict__ out,
-                                   const int* __restrict__ rows, int H, float eps) {
+                                   const int* __restrict__ rows, int H, float eps, int slabs, size_t slab_stride) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)src * H;
@@ -56,7 +58,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = x[i];
     if (dl) {
-      v += load_f32(dl + i);
+      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
       if (!rows) x[i] = v;
     }
     ss += v * v;
@@ -65,19 +67,22 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   const float r = 1.0f / sqrtf(ss / (float)H + eps);
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = x[i];
-    if (dl && rows) v += load_f32(dl + i);
+    if (dl && rows)
+      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
     store_f32(o + i, v * r * w[i]);
   }
 }
 
-extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype, const float* w, void* out,
-                                int out_dtype, const int* rows, int T, int H, float eps, hipStream_t stream) {
+extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype, int slabs, long long slab_stride,
+                                const float* w, void* out, int out_dtype, const int* rows, int T, int H, float eps,
+                                hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && H > 0, "pico_add_rmsnorm: bad sizes T=%d H=%d", T, H);
+  PICO_REQUIRE(slabs >= 1 && slab_stride >= 0, "pico_add_rmsnorm: bad slabs");
   PICO_REQUIRE(eps > 0.f, "pico_add_rmsnorm: eps must be positive");
   if (T == 0) return 0;
   const int threads = H >= 2048 ? 512 : 256;
 #define LAUNCH(TD, TO) \
-  add_rmsnorm_kernel<TD, TO><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H, eps)
+  add_rmsnorm_kernel<TD, TO><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H, eps, slabs, (size_t)slab_stride)
   if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_F32) LAUNCH(float, float);
   else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_BF16) LAUNCH(float, bf16_t);

@@ -77,15 +77,22 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """rows is None: resid += delta (if given), returns norm(resid).
-    rows given: returns norm(resid[rows] + delta[rows]); resid is left alone."""
+    rows given: returns norm(resid[rows] + delta[rows]); resid is left alone.
+    delta is [T, H], or a float32 stack [S, T, H] of partial sums that are all added."""
     _gpu(resid, delta, weight, rows)
     T, H = resid.shape
     if resid.dtype != torch.float32 or not resid.is_contiguous():
         raise KernelError("the residual stream must be contiguous float32")
     if weight.dtype != torch.float32 or weight.shape != (H,) or not weight.is_contiguous():
         raise KernelError(f"norm weight must be float32 of shape [{H}]")
-    if delta is not None and (delta.shape != resid.shape or not delta.is_contiguous()):
-        raise KernelError("delta must be contiguous and shaped like the residual stream")
+    slabs = 1
+    if delta is not None:
+        if delta.dim() == 3:
+            slabs = delta.shape[0]
+            if delta.dtype != torch.float32:
+                raise KernelError("a stack of partial sums must be float32")
+        if tuple(delta.shape[-2:]) != (T, H) or not delta.is_contiguous():
+            raise KernelError("delta must be contiguous and shaped like the residual stream")
     n = T
     if rows is not None:
         _i32(rows, "rows")
@@ -96,8 +103,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
         raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
     lib = library.core()
     ddt = _dt(delta) if delta is not None else F32
-    _check(lib, lib.pico_add_rmsnorm(_ptr(resid), _ptr(delta), ddt, _ptr(weight), _ptr(out), _DT[out_dtype],
-                                     _ptr(rows), n, H, c_float(eps), _stream()))
+    _check(lib, lib.pico_add_rmsnorm(_ptr(resid), _ptr(delta), ddt, slabs, c_ll(T * H), _ptr(weight), _ptr(out),
+                                     _DT[out_dtype], _ptr(rows), n, H, c_float(eps), _stream()))
     return out
 
 
@@ -171,6 +178,64 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
                                    a.stride(0) if M > 1 else K, w.stride(0), out.stride(0) if M > 1 else N,
                                    _stream()))
     return out
+
+
+EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
+
+
+def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the weight-streaming kernel takes these operands (few rows, 16-byte aligned rows)."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and a.shape[0] <= 64
+            and a.shape[1] % 8 == 0 and a.stride(1) == 1 and w.stride(1) == 1
+            and (a.stride(0) % 8 == 0 or a.shape[0] == 1) and w.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_BF16,
+                k_splits: int = 1) -> torch.Tensor:
+    """a [M <= 64, K] x w [N, K]^T, both bfloat16.  EPI_BF16 -> bf16 [M, N]; EPI_F32 -> float32 [M, N], or with
+    k_splits > 1 a stack [k_splits, M, N] of partial sums (bias in the first); EPI_SWIGLU (w = [gate; up])
+    -> bf16 [M, N / 2] = silu(gate) * up."""
+    _gpu(a, w, bias)
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise KernelError(f"gemm: inner sizes differ ({K} and {K2})")
+    if not skinny_ok(a, w):
+        raise KernelError("gemm_skinny: operands must be bfloat16, at most 64 rows, K a multiple of 8, rows 16-byte aligned")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (N,) or not bias.is_contiguous()):
+        raise KernelError("gemm_skinny: bias must be contiguous float32 [N]")
+    if k_splits > 1 and epilogue != EPI_F32:
+        raise KernelError("gemm_skinny: only the float32 epilogue can leave partial sums")
+    if epilogue == EPI_F32:
+        shape = (M, N) if k_splits == 1 else (k_splits, M, N)
+        out = torch.empty(shape, dtype=torch.float32, device=a.device)
+        ldo = N
+    elif epilogue == EPI_SWIGLU:
+        if N % 2:
+            raise KernelError("gemm_skinny: SwiGLU needs an even number of weight rows")
+        out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=a.device)
+        ldo = N // 2
+    else:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+        ldo = N
+    lib = library.core()
+    _check(lib, lib.pico_gemm_skinny(_ptr(a), a.stride(0) if M > 1 else K, _ptr(w), w.stride(0), _ptr(bias), _ptr(out),
+                                     ldo, c_ll(M * N), epilogue, M, N, K, k_splits, _stream()))
+    return out
+
+
+def skinny_k_splits(N: int, K: int, max_splits: int = 8) -> int:
+    """How many workgroups share the k range of a small matrix: enough workgroups to cover the chip,
+    ranges of whole 256-wide steps, every range non-empty."""
+    tiles = -(-N // 32)
+    want = max(1, min(max_splits, 512 // max(1, tiles), K // 256))
+    while want > 1:
+        per = -(-(-(-K // want)) // 256) * 256
+        if -(-K // per) == want:
+            return want
+        want -= 1
+    return 1
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int):

@@ -27,7 +27,7 @@ HIP_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
 
-CORE_SOURCES = ("errors.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_ref.hip", "sampling.hip")
+CORE_SOURCES = ("errors.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "gemm_skinny.hip", "attention_ref.hip", "sampling.hip")
 
 ATTN_SOURCES = ("errors.hip", "attention_mfma.hip")
 

@@ -1,9 +1,10 @@
 """y = x W^T (+ b) with W stored [out, in] as in the checkpoint.
 
-bfloat16 weights: the library GEMM (hipBLASLt through torch), as the
-reference uses the library for every projection (pico_vllm/model.py:200,225,
-316,318); a float32 result (logits) comes from the matrix-core kernel of this
-package.  float32 weights: this package's plain-FMA kernel, never a library
+bfloat16 weights: with up to 64 rows of activations (decode, small mixed
+steps) the weight-streaming matrix-core kernel of this package, with bias,
+SwiGLU or float32 output as its epilogue; with more rows the library GEMM
+(hipBLASLt through torch), as the reference uses the library for every
+projection (pico_vllm/model.py:200,225,316,318).  float32 weights: this package's plain-FMA kernel, never a library
 call, so the 32-bit engine has no reduced-precision matrix mode anywhere; if
 the activations are bfloat16 (a tensor stored in 32 bit inside a bfloat16
 engine) they are widened on load and the result is rounded once.
@@ -35,8 +36,29 @@ class Linear:
             return y if out_dtype == torch.float32 else y.to(out_dtype)
         if x.dtype != torch.bfloat16:
             raise ValueError("linear: bfloat16 weights need bfloat16 activations")
+        if kernels.skinny_ok(x, self.weight):
+            epi = kernels.EPI_F32 if out_dtype == torch.float32 else kernels.EPI_BF16
+            return kernels.gemm_skinny(x, self.weight, self.bias_f32, epi)
         if out_dtype == torch.float32:
             return kernels.gemm_bf16(x, self.weight, self.bias_f32, torch.float32)
         if self.bias is not None:
             return torch.addmm(self.bias, x, self.weight.t())
         return torch.mm(x, self.weight.t())
+
+    def swiglu(self, x: torch.Tensor) -> torch.Tensor:
+        """silu(gate) * up where [gate; up] = x W^T (W's first half of rows is the gate).  With few
+        rows the activation is the epilogue of the weight-streaming kernel and [gate; up] never
+        reaches memory."""
+        if self.weight.dtype == torch.bfloat16 and self.bias is None and kernels.skinny_ok(x, self.weight):
+            return kernels.gemm_skinny(x, self.weight, None, kernels.EPI_SWIGLU)
+        return kernels.swiglu(self(x))
+
+    def partial(self, x: torch.Tensor) -> torch.Tensor:
+        """x W^T as something a norm's ``add_norm`` takes as delta: [T, N], or, when the matrix is
+        too small to fill the chip with one workgroup per output tile, a float32 stack [S, T, N] of
+        partial sums over S ranges of k, which the norm kernel adds up."""
+        if self.weight.dtype == torch.bfloat16 and self.bias is None and kernels.skinny_ok(x, self.weight):
+            splits = kernels.skinny_k_splits(self.out_features, self.in_features)
+            if splits > 1:
+                return kernels.gemm_skinny(x, self.weight, None, kernels.EPI_F32, splits)
+        return self(x)

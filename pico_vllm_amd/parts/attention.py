@@ -76,4 +76,4 @@ class GQAAttention(Mixer):
         else:
             a = kernels.paged_attention_ref(qkv, cache.k, cache.v, bt, ctx.positions, ctx.token_seq,
                                             nq, nkv, d, self.scale, self.window)
-        return self.o(a)
+        return self.o.partial(a)

@@ -62,7 +62,9 @@ class Norm(Part):
     def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """resid (float32 [T, H]) += delta, returns the normed rows in the activation dtype;
-        with ``rows`` only those rows are produced and resid is left unchanged."""
+        with ``rows`` only those rows are produced and resid is left unchanged.  delta is
+        [T, H] in the activation dtype or float32, or a float32 stack [S, T, H] of partial
+        sums (what ``ops.linear.Linear.partial`` returns), all of which are added."""
         raise NotImplementedError
 
 

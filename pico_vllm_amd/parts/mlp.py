@@ -5,7 +5,6 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ..ops import kernels
 from ..ops.linear import Linear
 from .base import FeedForward, StepContext
 from .registry import register_part
@@ -36,4 +35,4 @@ class SwiGLUMLP(FeedForward):
         self.down = Linear(tensors["down_proj.weight"].to(device))
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return self.down(kernels.swiglu(self.gate_up(x)))
+        return self.down.partial(self.gate_up.swiglu(x))

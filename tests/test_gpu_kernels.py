@@ -344,3 +344,53 @@ def test_fast_kernels_refuse_what_they_cannot_do(K):
     from pico_vllm_amd.ops.attention_fast import choose, supported
     assert choose(4, 2, 24, 0) is None and choose(4, 2, 512, 0) is None and choose(4, 2, 64, 16) is None
     assert supported(12, 2, 128, 0)
+
+
+# ---- weight-streaming GEMM --------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K_", [(1, 2048, 1536), (8, 1536, 1536), (64, 1536, 8960), (33, 301, 136), (5, 384, 192),
+                                   (2, 64, 320), (17, 1000, 264)])
+def test_gemm_skinny_epilogues(K, M, N, K_):
+    g = torch.Generator().manual_seed(M * N)
+    a = torch.randn(M, K_, generator=g).bfloat16()
+    w = (torch.randn(N, K_, generator=g) / math.sqrt(K_)).bfloat16()
+    b = torch.randn(N, generator=g)
+    want = a.double() @ w.double().T
+    out = K.gemm_skinny(a.to(DEV), w.to(DEV), b.to(DEV), K.EPI_F32)
+    assert torch.allclose(out.cpu().double(), want + b.double(), rtol=1e-4, atol=1e-4)
+    out = K.gemm_skinny(a.to(DEV), w.to(DEV), b.to(DEV), K.EPI_BF16)
+    assert out.dtype == torch.bfloat16 and torch.allclose(out.cpu().double(), want + b.double(), rtol=1e-2, atol=1e-2)
+    # partial sums over ranges of k add up to the product; the bias is in the first slab only
+    for splits in range(2, 9):
+        per = -(-(-(-K_ // splits)) // 256) * 256
+        if -(-K_ // per) != splits:
+            continue
+        slabs = K.gemm_skinny(a.to(DEV), w.to(DEV), b.to(DEV), K.EPI_F32, splits)
+        assert slabs.shape == (splits, M, N)
+        assert torch.allclose(slabs.cpu().double().sum(0), want + b.double(), rtol=1e-4, atol=1e-4)
+        assert torch.allclose(slabs[1:].cpu().double().sum(0) + slabs[0].cpu().double(), want + b.double(), rtol=1e-4, atol=1e-4)
+    # the stack goes into the norm kernel as delta
+    if N >= 64:
+        splits = K.skinny_k_splits(N, K_)
+        delta = K.gemm_skinny(a.to(DEV), w.to(DEV), None, K.EPI_F32, splits)
+        resid = torch.randn(M, N, generator=g)
+        r = resid.clone().to(DEV)
+        out = K.add_rmsnorm(r, delta, torch.ones(N, device=DEV), 1e-6, torch.float32)
+        assert torch.allclose(r.cpu().double(), resid.double() + want, rtol=1e-4, atol=1e-4)
+        close(out, P.rms_norm((resid.double() + want).float(), torch.ones(N), 1e-6), torch.float32, scale=10)
+    # SwiGLU epilogue: w = [gate rows; up rows]
+    if N % 2 == 0:
+        out = K.gemm_skinny(a.to(DEV), w.to(DEV), None, K.EPI_SWIGLU)
+        close(out, P.swiglu(want.float()), torch.bfloat16, scale=2)
+    # a row's result does not depend on the other rows of the call
+    one = K.gemm_skinny(a[M // 2:M // 2 + 1].to(DEV), w.to(DEV), b.to(DEV), K.EPI_F32)
+    full = K.gemm_skinny(a.to(DEV), w.to(DEV), b.to(DEV), K.EPI_F32)
+    assert torch.equal(one.cpu()[0], full.cpu()[M // 2])
+
+
+def test_gemm_skinny_refuses_misaligned_operands(K):
+    a = torch.randn(4, 172).bfloat16().to(DEV)          # K = 172 is no multiple of 8
+    w = torch.randn(64, 172).bfloat16().to(DEV)
+    assert not K.skinny_ok(a, w)
+    with pytest.raises(K.KernelError):
+        K.gemm_skinny(a, w)
+    assert not K.skinny_ok(torch.randn(65, 64).bfloat16().to(DEV), torch.randn(64, 64).bfloat16().to(DEV))
