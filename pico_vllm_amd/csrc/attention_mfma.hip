@@ -5,10 +5,11 @@
 //                    head; each wave owns 32 queries; keys and values of the sequence stream
 //                    through LDS in tiles of BN keys, from position 0 to the causal frontier.
 //                    A decode token is a sequence that brings one query.
-//   decode           one workgroup (2 waves) per (sequence, kv head, split of the context); the
+//   decode           one workgroup per (sequence, kv head, split of the context); the
 //                    "queries" are the G query heads that share the kv head, so keys and values
 //                    are read once for the whole group (the reference's kernel re-reads them per
-//                    query head, pico_vllm/kernels/attention.py:96-105); the waves split the keys;
+//                    query head, pico_vllm/kernels/attention.py:96-105); two waves split the keys of a tile
+//                    (the other two only help to move tiles);
 //                    partial (max, sum, output) per split are merged by a second kernel.
 //
 // Formulas as in pico_vllm/kernels/attention.py:136-213: scores (q.k) * scale, key visible iff its
@@ -47,41 +48,70 @@ struct alignas(16) Tiles {
   alignas(16) bf16_t vt[DP * VROW];   // [dim][key]
 };
 
-// Load keys [tile_start, tile_start + BN) of one sequence and kv head into LDS; positions at or
-// beyond kv_end read as zero (their pages may not exist).  P % 8 == 0, tile_start % 8 == 0.
-__device__ __forceinline__ void load_tiles(Tiles& t, const bf16_t* __restrict__ k_cache,
-                                           const bf16_t* __restrict__ v_cache, const int* __restrict__ bt, int g,
-                                           int nkv, int P, int num_pages, int tile_start, int kv_end, int nthreads) {
-  constexpr int KCH = D / 8;  // 16-byte chunks per key
-  for (int c = threadIdx.x; c < BN * KCH; c += nthreads) {
-    const int key = c / KCH, dc = c % KCH;
-    const int pos = tile_start + key;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (pos < kv_end) {
-      const int page = min(max(bt[pos / P], 0), num_pages - 1);
-      v = *reinterpret_cast<const uint4*>(k_cache + (((size_t)page * nkv + g) * P + pos % P) * D + dc * 8);
+// A tile of BN keys travels global -> registers (fetch: every thread issues all its 16-byte loads
+// before it waits for any) -> LDS (commit).  The fetch of the next tile is issued before the
+// current tile is computed, so its latency hides behind the matrix products.
+// Positions at or beyond kv_end read as zero (their pages may not exist).  P % 8 == 0 and
+// tile_start % 8 == 0, so a 16-byte chunk of V^T (8 keys of one head dimension) lies in one page.
+template <int NT>
+struct TileRegs {
+  static constexpr int KCH = D / 8;                        // 16-byte chunks per key
+  static constexpr int VCH = BN / 8;                       // 16-byte chunks (8 keys) per head dimension
+  static constexpr int NK = (BN * KCH + NT - 1) / NT;      // chunks per thread
+  static constexpr int NV = (D * VCH + NT - 1) / NT;
+  uint4 k[NK], v[NV];
+
+  __device__ __forceinline__ void fetch(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                                        const int* __restrict__ bt, int g, int nkv, int P, int num_pages,
+                                        int tile_start, int kv_end) {
+#pragma unroll
+    for (int i = 0; i < NK; i++) {
+      const int c = threadIdx.x + i * NT;
+      const int key = c / KCH, dc = c % KCH;
+      const int pos = tile_start + key;
+      k[i] = make_uint4(0, 0, 0, 0);
+      if (c < BN * KCH && pos < kv_end) {
+        const int page = min(max(bt[pos / P], 0), num_pages - 1);
+        k[i] = *reinterpret_cast<const uint4*>(k_cache + (((size_t)page * nkv + g) * P + pos % P) * D + dc * 8);
+      }
     }
-    *reinterpret_cast<uint4*>(&t.k[key * KROW + dc * 8]) = v;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int c = threadIdx.x + i * NT;
+      const int dim = c / VCH, kc = c % VCH;
+      const int pos = tile_start + kc * 8;
+      v[i] = make_uint4(0, 0, 0, 0);
+      if (c < D * VCH && pos < kv_end) {
+        const int page = min(max(bt[pos / P], 0), num_pages - 1);
+        v[i] = *reinterpret_cast<const uint4*>(v_cache + (((size_t)page * nkv + g) * D + dim) * P + pos % P);
+      }
+    }
   }
-  constexpr int VCH = BN / 8;  // 16-byte chunks (8 keys) per head dimension
-  for (int c = threadIdx.x; c < D * VCH; c += nthreads) {
-    const int dim = c / VCH, kc = c % VCH;
-    const int pos = tile_start + kc * 8;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (pos < kv_end) {
-      const int page = min(max(bt[pos / P], 0), num_pages - 1);
-      v = *reinterpret_cast<const uint4*>(v_cache + (((size_t)page * nkv + g) * D + dim) * P + pos % P);
-      if (pos + 8 > kv_end) {  // the tail of the last chunk holds whatever the page held before
-        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+
+  __device__ __forceinline__ void commit(Tiles& t, int tile_start, int kv_end) const {
+#pragma unroll
+    for (int i = 0; i < NK; i++) {
+      const int c = threadIdx.x + i * NT;
+      if (c < BN * KCH) *reinterpret_cast<uint4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int c = threadIdx.x + i * NT;
+      if (c >= D * VCH) continue;
+      const int dim = c / VCH, kc = c % VCH;
+      const int pos = tile_start + kc * 8;
+      uint4 x = v[i];
+      if (pos < kv_end && pos + 8 > kv_end) {   // the tail of the last chunk holds whatever the page held before
+        uint32_t w[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
         for (int e = 0; e < 8; e++)
           if (pos + e >= kv_end) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
-        v = make_uint4(w[0], w[1], w[2], w[3]);
+        x = make_uint4(w[0], w[1], w[2], w[3]);
       }
+      *reinterpret_cast<uint4*>(&t.vt[dim * VROW + kc * 8]) = x;
     }
-    *reinterpret_cast<uint4*>(&t.vt[dim * VROW + kc * 8]) = v;
   }
-}
+};
 
 __device__ __forceinline__ void zero_pad_rows(Tiles& t, int nthreads) {
   if (DP > D)
@@ -154,7 +184,7 @@ __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf
     uint32_t pk[4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      pk[i] = (uint32_t)f32_to_bf16(s[8 * m + 2 * i]) | ((uint32_t)f32_to_bf16(s[8 * m + 2 * i + 1]) << 16);
+      pk[i] = pack2_bf16(s[8 * m + 2 * i], s[8 * m + 2 * i + 1]);
     const bf16x8 b = __builtin_bit_cast(bf16x8, make_uint4(pk[0], pk[1], pk[2], pk[3]));
 #pragma unroll
     for (int tt = 0; tt < DT; tt++) {
@@ -181,7 +211,7 @@ __device__ __forceinline__ void load_q(bf16x8* q, const bf16_t* qrow, bool ok) {
 // ---------------------------------------------------------------------------
 // prefill / mixed batches
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void prefill_kernel(const bf16_t* __restrict__ q, int q_stride,
+__global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16_t* __restrict__ q, int q_stride,
                                                       const bf16_t* __restrict__ k_cache,
                                                       const bf16_t* __restrict__ v_cache,
                                                       const int* __restrict__ block_table, int max_pages,
@@ -218,10 +248,13 @@ __global__ __launch_bounds__(256) void prefill_kernel(const bf16_t* __restrict__
   WaveState st;
   init_state(st);
   zero_pad_rows(tiles, 256);
+  TileRegs<256> regs;
+  regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, 0, kv_end);
   for (int tile_start = 0; tile_start < kv_end; tile_start += BN) {
+    __syncthreads();                                          // everyone is done with the previous tile
+    regs.commit(tiles, tile_start, kv_end);
     __syncthreads();
-    load_tiles(tiles, k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start, kv_end, 256);
-    __syncthreads();
+    if (tile_start + BN < kv_end) regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start + BN, kv_end);
     if (!wave_active) continue;
 #pragma unroll
     for (int sub = 0; sub < BN / 32; sub++) {
@@ -240,8 +273,8 @@ __global__ __launch_bounds__(256) void prefill_kernel(const bf16_t* __restrict__
       const int dim = tt * 32 + 8 * a + 4 * h;
       if (dim < D) {
         uint2 v;
-        v.x = (uint32_t)f32_to_bf16(st.o[tt][4 * a] * inv_l) | ((uint32_t)f32_to_bf16(st.o[tt][4 * a + 1] * inv_l) << 16);
-        v.y = (uint32_t)f32_to_bf16(st.o[tt][4 * a + 2] * inv_l) | ((uint32_t)f32_to_bf16(st.o[tt][4 * a + 3] * inv_l) << 16);
+        v.x = pack2_bf16(st.o[tt][4 * a] * inv_l, st.o[tt][4 * a + 1] * inv_l);
+        v.y = pack2_bf16(st.o[tt][4 * a + 2] * inv_l, st.o[tt][4 * a + 3] * inv_l);
         *reinterpret_cast<uint2*>(orow + dim) = v;
       }
     }
@@ -251,7 +284,7 @@ __global__ __launch_bounds__(256) void prefill_kernel(const bf16_t* __restrict__
 // decode: one query token per sequence, the G heads of a kv group as the 32 columns
 // ---------------------------------------------------------------------------
 // partial results per (sequence, query head, split): o [D] unnormalised, then m and l
-__global__ __launch_bounds__(128) void decode_kernel(const bf16_t* __restrict__ q, int q_stride,
+__global__ __launch_bounds__(256, 2) void decode_kernel(const bf16_t* __restrict__ q, int q_stride,
                                                      const bf16_t* __restrict__ k_cache,
                                                      const bf16_t* __restrict__ v_cache,
                                                      const int* __restrict__ block_table, int max_pages,
@@ -274,12 +307,15 @@ __global__ __launch_bounds__(128) void decode_kernel(const bf16_t* __restrict__ 
 
   WaveState st;
   init_state(st);
-  zero_pad_rows(tiles, 128);
+  zero_pad_rows(tiles, 256);
+  TileRegs<256> regs;
+  if (k_begin < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, k_begin, k_end);
   for (int tile_start = k_begin; tile_start < k_end; tile_start += BN) {
     __syncthreads();
-    load_tiles(tiles, k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start, k_end, 128);
+    regs.commit(tiles, tile_start, k_end);
     __syncthreads();
-    for (int sub = wave; sub < BN / 32; sub += 2) {
+    if (tile_start + BN < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start + BN, k_end);
+    for (int sub = wave; sub < BN / 32 && wave < 2; sub += 2) {   // waves 2 and 3 only help to move the tiles
       const int key0 = tile_start + sub * 32;
       if (key0 >= k_end) break;
       // every query sits at position ctx - 1: only keys at or beyond k_end need the mask
@@ -316,23 +352,31 @@ __global__ __launch_bounds__(128) void decode_kernel(const bf16_t* __restrict__ 
   if (h == 0) { po[D] = m; po[D + 1] = l; }
 }
 
-// out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s
-__global__ void decode_merge_kernel(const float* __restrict__ part, int nsplit, bf16_t* __restrict__ out, int nq) {
-  const int b = blockIdx.x, head = blockIdx.y;
+// out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s; one wave per (sequence, head);
+// lane s weighs split s, then every lane sums its head dimensions over the splits.
+__global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
+                                                          bf16_t* __restrict__ out, int nq) {
+  __shared__ float w[64];
+  const int b = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const float* p = part + ((size_t)b * nq + head) * nsplit * (D + 2);
-  float M = -INFINITY;
-  for (int s = 0; s < nsplit; s++) M = fmaxf(M, p[s * (D + 2) + D]);
+  const bool mine = lane < nsplit;                         // nsplit <= 64
+  const float m = mine ? p[lane * (D + 2) + D] : -INFINITY;
+  const float l = mine ? p[lane * (D + 2) + D + 1] : 0.f;
+  const float M = wave_max(m);
   bf16_t* o = out + ((size_t)b * nq + head) * D;
   if (M == -INFINITY) {   // an empty row (padding of a captured batch)
-    for (int dim = threadIdx.x; dim < D; dim += blockDim.x) o[dim] = 0;
+    for (int dim = lane; dim < D; dim += 64) o[dim] = 0;
     return;
   }
-  float L = 0.f;
-  for (int s = 0; s < nsplit; s++) L += __expf(p[s * (D + 2) + D] - M) * p[s * (D + 2) + D + 1];
+  const float wt = mine ? __expf(m - M) : 0.f;
+  const float L = wave_sum(wt * l);
+  w[lane] = wt;
+  __syncthreads();
   const float inv = 1.0f / L;
-  for (int dim = threadIdx.x; dim < D; dim += blockDim.x) {
+  for (int dim = lane; dim < D; dim += 64) {
     float acc = 0.f;
-    for (int s = 0; s < nsplit; s++) acc += __expf(p[s * (D + 2) + D] - M) * p[s * (D + 2) + dim];
+#pragma unroll 8
+    for (int s = 0; s < nsplit; s++) acc += w[s] * p[s * (D + 2) + dim];
     o[dim] = f32_to_bf16(acc * inv);
   }
 }
@@ -372,10 +416,10 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
                                 float scale, hipStream_t stream) {
   if (check_common("pico_attn_decode", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
   PICO_REQUIRE(nq / nkv <= 32, "pico_attn_decode: %d query heads per kv head are more than 32", nq / nkv);
-  PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= 65535 && nkv <= 65535, "pico_attn_decode: bad sizes");
+  PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= 64 && nkv <= 65535, "pico_attn_decode: bad sizes (1 to 64 splits)");
   PICO_REQUIRE(((uintptr_t)q % 16 == 0), "pico_attn_decode: misaligned queries");
   dim3 grid(num_seqs, nkv, nsplit);
-  decode_kernel<<<grid, 128, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+  decode_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                          block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
                                          scale);
   PICO_LAUNCH_CHECK();

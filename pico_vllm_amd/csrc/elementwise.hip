@@ -45,7 +45,24 @@ extern "C" int pico_embedding(const void* table, int table_dtype, const int* ids
 // splits its k range over workgroups leaves behind; they are added in slab order.
 // One workgroup per row.  The sum of squares is taken over the float32 sum.
 // ---------------------------------------------------------------------------
-template <typename TD, typename TO>
+#define MAX_SLABS 8
+
+template <typename TD> __device__ __forceinline__ float4 load4_f32(const TD* p);
+template <> __device__ __forceinline__ float4 load4_f32<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 load4_f32<bf16_t>(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                     __uint_as_float(u.y & 0xffff0000u));
+}
+template <typename TO> __device__ __forceinline__ void store4_f32(TO* p, float4 v);
+template <> __device__ __forceinline__ void store4_f32<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void store4_f32<bf16_t>(bf16_t* p, float4 v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v.x, v.y), pack2_bf16(v.z, v.w));
+}
+
+// VEC: rows are handled four elements at a time (H % 4 == 0, so every row starts on 16 bytes).
+// All loads of an element group (the stream and up to MAX_SLABS slabs) are issued together.
+template <typename TD, typename TO, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    const float* __restrict__ w, TO* __restrict__ out,
                                    const int* __restrict__ rows, int H, float eps, int slabs, size_t slab_stride) {
@@ -55,21 +72,53 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   const TD* dl = delta ? delta + (size_t)src * H : nullptr;
   TO* o = out + (size_t)blockIdx.x * H;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = x[i];
-    if (dl) {
-      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
-      if (!rows) x[i] = v;
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (dl) {
+        float4 d[MAX_SLABS];
+#pragma unroll
+        for (int s = 0; s < MAX_SLABS; s++)
+          d[s] = s < slabs ? load4_f32(dl + s * slab_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int s = 0; s < MAX_SLABS; s++) { v.x += d[s].x; v.y += d[s].y; v.z += d[s].z; v.w += d[s].w; }
+        if (!rows) *reinterpret_cast<float4*>(x + i) = v;
+      }
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
-    ss += v * v;
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      float v = x[i];
+      if (dl) {
+        for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
+        if (!rows) x[i] = v;
+      }
+      ss += v * v;
+    }
   }
   ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)H + eps);
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = x[i];
-    if (dl && rows)
-      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
-    store_f32(o + i, v * r * w[i]);
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (dl && rows) {
+        float4 d[MAX_SLABS];
+#pragma unroll
+        for (int s = 0; s < MAX_SLABS; s++)
+          d[s] = s < slabs ? load4_f32(dl + s * slab_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int s = 0; s < MAX_SLABS; s++) { v.x += d[s].x; v.y += d[s].y; v.z += d[s].z; v.w += d[s].w; }
+      }
+      const float4 g = *reinterpret_cast<const float4*>(w + i);
+      store4_f32(o + i, make_float4(v.x * r * g.x, v.y * r * g.y, v.z * r * g.z, v.w * r * g.w));
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      float v = x[i];
+      if (dl && rows)
+        for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
+      store_f32(o + i, v * r * w[i]);
+    }
   }
 }
 
@@ -77,12 +126,21 @@ extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype
                                 const float* w, void* out, int out_dtype, const int* rows, int T, int H, float eps,
                                 hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && H > 0, "pico_add_rmsnorm: bad sizes T=%d H=%d", T, H);
-  PICO_REQUIRE(slabs >= 1 && slab_stride >= 0, "pico_add_rmsnorm: bad slabs");
+  PICO_REQUIRE(slabs >= 1 && slabs <= MAX_SLABS && slab_stride >= 0, "pico_add_rmsnorm: 1 to %d slabs, got %d", MAX_SLABS, slabs);
+  const bool vec = H % 4 == 0 && (uintptr_t)resid % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+                   (uintptr_t)delta % 16 == 0 && slab_stride % 4 == 0;
   PICO_REQUIRE(eps > 0.f, "pico_add_rmsnorm: eps must be positive");
   if (T == 0) return 0;
-  const int threads = H >= 2048 ? 512 : 256;
-#define LAUNCH(TD, TO) \
-  add_rmsnorm_kernel<TD, TO><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H, eps, slabs, (size_t)slab_stride)
+  const int threads = H >= 4096 ? 512 : (H >= 1024 ? 256 : 128);
+#define LAUNCH(TD, TO)                                                                                                \
+  do {                                                                                                                \
+    if (vec)                                                                                                          \
+      add_rmsnorm_kernel<TD, TO, true><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H, eps, \
+                                                                  slabs, (size_t)slab_stride);                       \
+    else                                                                                                              \
+      add_rmsnorm_kernel<TD, TO, false><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H,    \
+                                                                   eps, slabs, (size_t)slab_stride);                 \
+  } while (0)
   if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_F32) LAUNCH(float, float);
   else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_BF16) LAUNCH(float, bf16_t);

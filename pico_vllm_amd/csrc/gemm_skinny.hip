@@ -24,7 +24,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
 
-template <int MT, int EPI>
+template <int MT, int EPI, bool TAIL>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias, void* __restrict__ out,
@@ -45,15 +45,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
     wrow = tile * 32 + col;
     w_ok = wrow < N;
   }
-  const bf16_t* wp = W + (size_t)(w_ok ? wrow : 0) * ldw + 32 * h;
-  const bf16_t* xp[MT];
-  bool x_ok[MT];
+  // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
+  // Only a k tail must read as zero, because it is summed into outputs that are stored.
+  const int n_rows = N;
+  const bf16_t* wrow0 = W + (size_t)min(wrow, n_rows - 1) * ldw;
+  const bf16_t* xrow0[MT];
 #pragma unroll
-  for (int t = 0; t < MT; t++) {
-    const int m = m0 + 32 * t + col;
-    x_ok[t] = m < M;
-    xp[t] = X + (size_t)(x_ok[t] ? m : 0) * ldx + 32 * h;
-  }
+  for (int t = 0; t < MT; t++) xrow0[t] = X + (size_t)min(m0 + 32 * t + col, M - 1) * ldx;
   f32x16 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; t++)
@@ -61,25 +59,69 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
     for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
 
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  // this wave's 64-wide slices: k_begin + 64 (wave + 4 i)
-#pragma unroll 2
-  for (int k0 = k_begin + 64 * wave; k0 < k_end; k0 += 256) {
-    uint4 wv[4], xv[MT][4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const int k = k0 + 32 * h + 8 * s;          // 8 consecutive k; K % 8 == 0, so all or nothing
-      const bool k_ok = k < k_end;
-      wv[s] = (w_ok && k_ok) ? *reinterpret_cast<const uint4*>(wp + k0 + 8 * s) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < MT; t++)
-        xv[t][s] = (x_ok[t] && k_ok) ? *reinterpret_cast<const uint4*>(xp[t] + k0 + 8 * s) : make_uint4(0, 0, 0, 0);
-    }
+  struct Stage {
+    uint4 w[4], x[MT][4];
+  };
+  auto multiply = [&](const Stage& st) {
 #pragma unroll
     for (int s = 0; s < 4; s++)
 #pragma unroll
       for (int t = 0; t < MT; t++)
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv[s]),
-                                                         __builtin_bit_cast(bf16x8, xv[t][s]), acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, st.w[s]),
+                                                         __builtin_bit_cast(bf16x8, st.x[t][s]), acc[t], 0, 0, 0);
+  };
+  // this wave's slices start at k_begin + 64 (wave + 4 i)
+  const int first = k_begin + 64 * wave;
+  if (!TAIL) {
+    // K % 64 == 0: every slice is whole.  Straight-line code with two stages in flight: the loads of
+    // the next slice are always issued (the last iteration re-reads its own slice, which is cached)
+    // so that no branch stands between a load and the wait for the stage before it.
+    auto load_stage = [&](Stage& st, int k0) {
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        st.w[s] = *reinterpret_cast<const uint4*>(wrow0 + k0 + 32 * h + 8 * s);
+#pragma unroll
+        for (int t = 0; t < MT; t++) st.x[t][s] = *reinterpret_cast<const uint4*>(xrow0[t] + k0 + 32 * h + 8 * s);
+      }
+    };
+    if (first < k_end) {
+      const int last = first + (k_end - 1 - first) / 256 * 256;     // start of this wave's last slice
+      Stage sa, sb;
+      load_stage(sa, first);
+      // the scheduling barriers keep the compiler from sinking the loads next to their use, which
+      // would leave only two of them in flight
+      for (int k0 = first;;) {
+        load_stage(sb, min(k0 + 256, last));
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(sa);
+        __builtin_amdgcn_sched_barrier(0);
+        k0 += 256;
+        if (k0 > last) break;
+        load_stage(sa, min(k0 + 256, last));
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(sb);
+        __builtin_amdgcn_sched_barrier(0);
+        k0 += 256;
+        if (k0 > last) break;
+      }
+    }
+  } else {
+    for (int k0 = first; k0 < k_end; k0 += 256) {
+      Stage st;
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        const int k = k0 + 32 * h + 8 * s;          // 8 consecutive k; K % 8 == 0, so all or nothing
+        const bool ok = k < k_end;
+        const uint4 wv = *reinterpret_cast<const uint4*>(wrow0 + (ok ? k : 0));
+        st.w[s] = ok ? wv : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+          const uint4 xv = *reinterpret_cast<const uint4*>(xrow0[t] + (ok ? k : 0));
+          st.x[t][s] = ok ? xv : make_uint4(0, 0, 0, 0);
+        }
+      }
+      multiply(st);
+    }
   }
 #pragma unroll
   for (int t = 0; t < MT; t++)
@@ -158,11 +200,14 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   dim3 grid(tiles, ky, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535 && grid.y <= 65535, "pico_gemm_skinny: too many blocks");
   const float* b0 = bias;
-#define LAUNCH(MT, EPI) \
-  gemm_skinny_kernel<MT, EPI><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+  const bool tail = K % 64 != 0;
+#define LAUNCH2(MT, EPI, TAIL) \
+  gemm_skinny_kernel<MT, EPI, TAIL><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+#define LAUNCH(MT, EPI) do { if (tail) LAUNCH2(MT, EPI, true); else LAUNCH2(MT, EPI, false); } while (0)
   if (epilogue == EPI_BF16) { if (mt == 1) LAUNCH(1, EPI_BF16); else LAUNCH(2, EPI_BF16); }
   else if (epilogue == EPI_F32) { if (mt == 1) LAUNCH(1, EPI_F32); else LAUNCH(2, EPI_F32); }
   else { if (mt == 1) LAUNCH(1, EPI_SWIGLU); else LAUNCH(2, EPI_SWIGLU); }
+#undef LAUNCH2
 #undef LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;
