@@ -352,6 +352,188 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(const bf16_t* __restrict
   if (h == 0) { po[D] = m; po[D + 1] = l; }
 }
 
+// ---------------------------------------------------------------------------
+// decode without LDS staging, for up to 16 query heads per kv head and D % 32 == 0
+// ---------------------------------------------------------------------------
+// v_mfma_f32_16x16x32_bf16 (A 16x32, B 32x16): lane l supplies A[l % 16][8 (l / 16) + 0..7] and
+// B[8 (l / 16) + 0..7][l % 16] and receives D[4 (l / 16) + r][l % 16] in register r.  A wave owns
+// blocks of 32 keys: two 16-key tiles of S^T = K Q^T (the 16 columns are the query heads of the
+// group), then O^T += V^T P^T with the 32 keys as the contraction; as in the other kernels the
+// contraction order is the order in which the registers hold the keys, so P never moves.
+// Operands come straight from the pages: lane (key, kq) reads the 64 contiguous bytes
+// K[key][32 kq ..] (the contraction over the head dimension runs in that permuted order for K
+// and Q alike), and lane (dim, kq) reads the 8 bytes V^T[dim][4 kq .. 4 kq + 3] of each tile.
+// The loads of a wave's next block are issued while the current block is computed.
+#if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int KS16 = D / 32;   // contraction steps of a 16-key tile
+constexpr int DT16 = D / 16;   // 16-wide tiles of the output's head dimension
+
+__global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restrict__ q, int q_stride,
+                                                          const bf16_t* __restrict__ k_cache,
+                                                          const bf16_t* __restrict__ v_cache,
+                                                          const int* __restrict__ block_table, int max_pages,
+                                                          const int* __restrict__ context_lens,
+                                                          float* __restrict__ part, int nsplit, int nq, int nkv, int P,
+                                                          int num_pages, float scale) {
+  __shared__ float xo[3][D][16];     // outputs of waves 1..3 for the final merge
+  __shared__ float xml[3][2][16];
+  const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  const int G = nq / nkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
+  const int ctx = context_lens[b];
+  const int per = ((ctx + nsplit - 1) / nsplit + 31) / 32 * 32;
+  const int k_begin = split * per, k_end = min(ctx, k_begin + per);
+  const int* bt = block_table + (size_t)b * max_pages;
+  const bool col_ok = col < G;
+  const int head = g * G + (col_ok ? col : 0);
+
+  bf16x8 qf[KS16];
+  {
+    const bf16_t* qrow = q + (size_t)b * q_stride + (size_t)head * D + (D / 4) * kq;
+#pragma unroll
+    for (int st = 0; st < KS16; st++) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (col_ok) v = *reinterpret_cast<const uint4*>(qrow + 8 * st);
+      qf[st] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[DT16];
+#pragma unroll
+  for (int tt = 0; tt < DT16; tt++) o[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int first = k_begin + 32 * wave;
+  if (first < k_end) {
+    const int last = first + (k_end - 1 - first) / 128 * 128;   // this wave's last block
+    const int last_key = k_end - 1, last_group = last_key / 4 * 4;
+    uint4 kr[2][KS16];
+    uint2 vr[DT16][2];
+    // positions beyond the split are clamped to its last key (group): the pages exist, the scores are masked
+    auto load_k = [&](int key0) {
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const int pos = min(key0 + 16 * t + col, last_key);
+        const int page = min(max(bt[pos / P], 0), num_pages - 1);
+        const bf16_t* kp = k_cache + (((size_t)page * nkv + g) * P + pos % P) * D + (D / 4) * kq;
+#pragma unroll
+        for (int st = 0; st < KS16; st++) kr[t][st] = *reinterpret_cast<const uint4*>(kp + 8 * st);
+      }
+    };
+    auto load_v = [&](int key0) {
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const int pos = min(key0 + 16 * t + 4 * kq, last_group);
+        const int page = min(max(bt[pos / P], 0), num_pages - 1);
+        const bf16_t* vp = v_cache + (((size_t)page * nkv + g) * D + col) * P + pos % P;
+#pragma unroll
+        for (int tt = 0; tt < DT16; tt++) vr[tt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)tt * 16 * P);
+      }
+    };
+    load_k(first);
+    __builtin_amdgcn_sched_barrier(0);       // keys before values, as in the loop, so the waits there stay partial
+    load_v(first);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int key0 = first;; key0 += 128) {
+      const int next = min(key0 + 128, last);
+      f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+      for (int st = 0; st < KS16; st++) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kr[0][st]), qf[st], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kr[1][st]), qf[st], s1, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      load_k(next);
+      __builtin_amdgcn_sched_barrier(0);
+      const bool tail = key0 + 32 > k_end;                     // the same for the whole wave
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 8; r++) {
+        float v = (r < 4 ? s0[r & 3] : s1[r & 3]) * scale;
+        if (tail && key0 + 16 * (r >> 2) + 4 * kq + (r & 3) >= k_end) v = -INFINITY;
+        sv[r] = v;
+        mx = fmaxf(mx, v);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);                        // finite: the block holds at least one key < k_end
+      const float alpha = __expf(m - m_new);
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 8; r++) {
+        sv[r] = __expf(sv[r] - m_new);
+        sum += sv[r];
+      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l = l * alpha + sum;
+      m = m_new;
+      const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack2_bf16(sv[0], sv[1]), pack2_bf16(sv[2], sv[3]),
+                                                               pack2_bf16(sv[4], sv[5]), pack2_bf16(sv[6], sv[7])));
+      if (tail) {   // values of keys beyond the split hold whatever the page held before: make them zero
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int pos = key0 + 16 * t + 4 * kq;
+#pragma unroll
+          for (int tt = 0; tt < DT16; tt++) {
+            if (pos >= k_end) vr[tt][t] = make_uint2(0, 0);
+            else {
+              if (pos + 1 >= k_end) vr[tt][t].x &= 0x0000ffffu;
+              if (pos + 2 >= k_end) vr[tt][t].y = 0;
+              else if (pos + 3 >= k_end) vr[tt][t].y &= 0x0000ffffu;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int tt = 0; tt < DT16; tt++) {
+        o[tt] *= alpha;
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vr[tt][0].x, vr[tt][0].y, vr[tt][1].x, vr[tt][1].y));
+        o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[tt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (key0 >= last) break;
+      load_v(next);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // merge the four waves; lane (col, kq) of wave 0 holds head dimensions 16 tt + 4 kq + r of head `col`
+  if (wave > 0) {
+#pragma unroll
+    for (int tt = 0; tt < DT16; tt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) xo[wave - 1][16 * tt + 4 * kq + r][col] = o[tt][r];
+    if (kq == 0) { xml[wave - 1][0][col] = m; xml[wave - 1][1][col] = l; }
+  }
+  __syncthreads();
+  if (wave != 0 || !col_ok) return;
+  float M = m;
+#pragma unroll
+  for (int w = 0; w < 3; w++) M = fmaxf(M, xml[w][0][col]);
+  const float m_use = (M == -INFINITY) ? 0.f : M;
+  const float a0 = __expf(m - m_use);
+  float aw[3], L = l * a0;
+#pragma unroll
+  for (int w = 0; w < 3; w++) {
+    aw[w] = __expf(xml[w][0][col] - m_use);
+    L += xml[w][1][col] * aw[w];
+  }
+  float* po = part + (((size_t)b * nq + head) * nsplit + split) * (D + 2);
+#pragma unroll
+  for (int tt = 0; tt < DT16; tt++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int dim = 16 * tt + 4 * kq + r;
+      float acc = o[tt][r] * a0;
+#pragma unroll
+      for (int w = 0; w < 3; w++) acc += xo[w][dim][col] * aw[w];
+      po[dim] = acc;
+    }
+  if (kq == 0) { po[D] = M; po[D + 1] = L; }
+}
+#endif
+
 // out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s; one wave per (sequence, head);
 // lane s weighs split s, then every lane sums its head dimensions over the splits.
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
@@ -419,9 +601,18 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
   PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= 64 && nkv <= 65535, "pico_attn_decode: bad sizes (1 to 64 splits)");
   PICO_REQUIRE(((uintptr_t)q % 16 == 0), "pico_attn_decode: misaligned queries");
   dim3 grid(num_seqs, nkv, nsplit);
-  decode_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
-                                         block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
-                                         scale);
+  bool direct = false;
+#if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
+  direct = nq / nkv <= 16 && P % 4 == 0;
+  if (direct)
+    decode16_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+                                             (const bf16_t*)v_cache, block_table, max_pages, context_lens, part,
+                                             nsplit, nq, nkv, P, num_pages, scale);
+#endif
+  if (!direct)
+    decode_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                           block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
+                                           scale);
   PICO_LAUNCH_CHECK();
   dim3 mgrid(num_seqs, nq);
   decode_merge_kernel<<<mgrid, 64, 0, stream>>>(part, nsplit, (bf16_t*)out, nq);
