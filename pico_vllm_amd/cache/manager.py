@@ -17,6 +17,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
+
 from ..parts.spec import CacheSpec
 from .page_pool import PagePool, PagePoolError, StateSlots
 
@@ -38,6 +40,17 @@ class RequestCache:
     tables: List[List[int]]                  # one per group
     num_computed: int = 0                    # tokens whose keys/state are in the cache
     first_live: List[int] = field(default_factory=list)   # per group: first page index still held
+    arrays: List[np.ndarray] = field(default_factory=list)  # per group: the table again as int32 array, for packing
+
+
+def _mirror(rc: RequestCache, gi: int) -> None:
+    """Bring the int32 copy of table ``gi`` up to date after the list changed."""
+    table = rc.tables[gi]
+    arr = rc.arrays[gi]
+    if len(table) > arr.shape[0]:
+        arr = np.full(max(2 * arr.shape[0], len(table), 16), -1, dtype=np.int32)
+        rc.arrays[gi] = arr
+    arr[:len(table)] = table
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -76,7 +89,8 @@ class CacheManager:
         slot = self.slots.acquire()
         if slot is None:
             return False
-        self.requests[req] = RequestCache(slot, [[] for _ in self.groups], 0, [0] * len(self.groups))
+        self.requests[req] = RequestCache(slot, [[] for _ in self.groups], 0, [0] * len(self.groups),
+                                          [np.full(16, -1, dtype=np.int32) for _ in self.groups])
         return True
 
     def free_request(self, req: Hashable) -> None:
@@ -101,8 +115,10 @@ class CacheManager:
         if any(n > g.pool.num_free for n, g in zip(need, self.groups)):
             return False
         rc = self.requests[req]
-        for n, g, table in zip(need, self.groups, rc.tables):
-            table.extend(g.pool.allocate(n))
+        for gi, (n, g, table) in enumerate(zip(need, self.groups, rc.tables)):
+            if n:
+                table.extend(g.pool.allocate(n))
+                _mirror(rc, gi)
         return True
 
     def advance(self, req: Hashable, num_computed: int) -> None:
@@ -123,6 +139,7 @@ class CacheManager:
                 rc.tables[gi][j] = -1
             if gone:
                 g.pool.release(gone)
+                _mirror(rc, gi)
             rc.first_live[gi] = max(rc.first_live[gi], dead_upto)
 
     def fork_prefix(self, src: Hashable, dst: Hashable, num_tokens: int) -> None:
@@ -144,11 +161,20 @@ class CacheManager:
                 raise PagePoolError("a page of the prefix was already given back by its window")
             g.pool.share(pages)
             dt.extend(pages)
+        for gi in range(len(self.groups)):
+            _mirror(d, gi)
         d.num_computed = num_tokens
 
     # ---- views ----------------------------------------------------------
     def block_table(self, req: Hashable, group: int = 0) -> List[int]:
         return self.requests[req].tables[group]
+
+    def block_table_array(self, req: Hashable, group: int, n: int) -> np.ndarray:
+        """The first ``n`` entries of the table as an int32 array (a view; do not write)."""
+        rc = self.requests[req]
+        if n > len(rc.tables[group]):
+            raise PagePoolError(f"request {req!r}: {n} pages are needed, {len(rc.tables[group])} are allocated")
+        return rc.arrays[group][:n]
 
     def slot(self, req: Hashable) -> int:
         return self.requests[req].slot

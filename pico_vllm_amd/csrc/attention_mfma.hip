@@ -534,12 +534,14 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 }
 #endif
 
-// out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s; one wave per (sequence, head);
-// lane s weighs split s, then every lane sums its head dimensions over the splits.
-__global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
-                                                          bf16_t* __restrict__ out, int nq) {
-  __shared__ float w[64];
-  const int b = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+// out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s; one workgroup per (sequence,
+// head).  Every wave weighs all splits (lane s holds split s) and sums a quarter of them for all
+// head dimensions, all loads issued together; wave 0 adds the four quarters.
+__global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
+                                                           bf16_t* __restrict__ out, int nq) {
+  constexpr int DPL = (D + 63) / 64;                        // head dimensions per lane
+  __shared__ float quarter[3][DPL * 64];
+  const int b = blockIdx.x, head = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float* p = part + ((size_t)b * nq + head) * nsplit * (D + 2);
   const bool mine = lane < nsplit;                         // nsplit <= 64
   const float m = mine ? p[lane * (D + 2) + D] : -INFINITY;
@@ -547,19 +549,44 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   const float M = wave_max(m);
   bf16_t* o = out + ((size_t)b * nq + head) * D;
   if (M == -INFINITY) {   // an empty row (padding of a captured batch)
-    for (int dim = lane; dim < D; dim += 64) o[dim] = 0;
+    if (wave == 0)
+      for (int dim = lane; dim < D; dim += 64) o[dim] = 0;
     return;
   }
   const float wt = mine ? __expf(m - M) : 0.f;
   const float L = wave_sum(wt * l);
-  w[lane] = wt;
+  float acc[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; i++) acc[i] = 0.f;
+  const int s0 = wave * 16;
+  float v[16][DPL];
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const int s = min(s0 + j, nsplit - 1);
+#pragma unroll
+    for (int i = 0; i < DPL; i++) {
+      const int dim = lane + 64 * i;
+      v[j][i] = dim < D ? p[s * (D + 2) + dim] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const float ws = (s0 + j < nsplit) ? __shfl(wt, s0 + j, 64) : 0.f;
+#pragma unroll
+    for (int i = 0; i < DPL; i++) acc[i] += ws * v[j][i];
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < DPL; i++) quarter[wave - 1][lane + 64 * i] = acc[i];
+  }
   __syncthreads();
+  if (wave != 0) return;
   const float inv = 1.0f / L;
-  for (int dim = lane; dim < D; dim += 64) {
-    float acc = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < nsplit; s++) acc += w[s] * p[s * (D + 2) + dim];
-    o[dim] = f32_to_bf16(acc * inv);
+#pragma unroll
+  for (int i = 0; i < DPL; i++) {
+    const int dim = lane + 64 * i;
+    if (dim < D)
+      o[dim] = f32_to_bf16((acc[i] + quarter[0][dim] + quarter[1][dim] + quarter[2][dim]) * inv);
   }
 }
 
@@ -615,7 +642,7 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
                                            scale);
   PICO_LAUNCH_CHECK();
   dim3 mgrid(num_seqs, nq);
-  decode_merge_kernel<<<mgrid, 64, 0, stream>>>(part, nsplit, (bf16_t*)out, nq);
+  decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq);
   PICO_LAUNCH_CHECK();
   return 0;
 }

@@ -85,6 +85,25 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
     for b, s in enumerate(seqs):
         n = lens[b]
         cached = manager.num_computed(s.req)
+        if n == 1:
+            tok = s.tokens[0]
+            if not 0 <= tok < vocab_size:
+                raise BatchError(f"request {s.req!r}: token id outside [0, {vocab_size})")
+            h_tok[t] = tok
+            h_pos[t] = cached
+            h_seq[t] = b
+            for w in s.want:
+                if w != 0:
+                    raise BatchError(f"request {s.req!r}: wanted place {w} is outside its 1 tokens")
+                h_want[r] = t
+                r += 1
+            t += 1
+            h_cu[b + 1] = t
+            h_ctx[b] = cached + 1
+            h_slot[b] = manager.slot(s.req)
+            max_ctx = max(max_ctx, cached + 1)
+            need_pages = max(need_pages, -(-(cached + 1) // P))
+            continue
         toks = np.asarray(s.tokens, dtype=np.int64)
         if toks.min() < 0 or toks.max() >= vocab_size:
             raise BatchError(f"request {s.req!r}: token id outside [0, {vocab_size})")
@@ -117,10 +136,7 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
     for b, s in enumerate(seqs):
         need = -(-int(h_ctx[b]) // P)
         for g in range(G):
-            table = manager.block_table(s.req, g)
-            if len(table) < need:
-                raise BatchError(f"request {s.req!r}: {need} pages are needed, {len(table)} are allocated")
-            tables[g, b, :need] = table[:need]
+            tables[g, b, :need] = manager.block_table_array(s.req, g, need)
     used = bt_off + G * rows * width
     buf.dev[:used].copy_(buf.host[:used], non_blocking=True)
     if buf.copied is not None:

@@ -25,9 +25,9 @@ class FastAttention:
             raise KernelError("attention library was built for another head size")
 
     def num_splits(self, num_seqs: int, max_context: int) -> int:
-        """Enough workgroups to fill the chip (256 CUs, a few workgroups each), no split shorter
+        """Enough workgroups to fill the chip (256 CUs, two workgroups each), no split shorter
         than one 64-key tile, at most 64 splits (one lane of the merging wave each)."""
-        by_fill = max(1, 1024 // max(1, num_seqs * self.nkv))
+        by_fill = max(1, 512 // max(1, num_seqs * self.nkv))
         by_len = max(1, -(-max_context // 64))
         return max(1, min(by_fill, by_len, 64))
 

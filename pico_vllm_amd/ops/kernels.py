@@ -39,8 +39,29 @@ def _ptr(t: Optional[torch.Tensor]):
     return c_void_p(t.data_ptr() if t is not None else 0)
 
 
+_bound_stream = None
+
+
 def _stream():
+    if _bound_stream is not None:
+        return _bound_stream
     return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class stream_scope:
+    """Look torch's current stream up once for all launches inside the scope (the lookup costs
+    more than a launch).  The scope must not span a change of the current stream."""
+
+    def __enter__(self):
+        global _bound_stream
+        self._outer = _bound_stream
+        _bound_stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+        return self
+
+    def __exit__(self, *exc):
+        global _bound_stream
+        _bound_stream = self._outer
+        return False
 
 
 def _check(lib, code: int) -> None:

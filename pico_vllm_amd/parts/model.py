@@ -112,6 +112,10 @@ class DecoderModel:
 
     def forward(self, ctx: StepContext, storage) -> torch.Tensor:
         """Logits float32 [R, V] at ctx.want_rows."""
+        with kernels.stream_scope():
+            return self._forward(ctx, storage)
+
+    def _forward(self, ctx: StepContext, storage) -> torch.Tensor:
         resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens])
         pending = None
         for i, e in enumerate(self.spec.run_order):

@@ -39,6 +39,8 @@ class Sampler:
         self._host = torch.zeros(3, max_rows, dtype=torch.float32, pin_memory=torch.cuda.is_available())
         self._dev = torch.zeros(3, max_rows, dtype=torch.float32, device=device)
         self._out = torch.zeros(max_rows, dtype=torch.int32, device=device)
+        self._host_np = self._host.numpy()
+        self._zeroed = True
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
                seeds: Sequence[int], indices: Sequence[int]) -> List[int]:
@@ -50,11 +52,17 @@ class Sampler:
             raise ValueError(f"{R} rows to sample, the sampler was made for {self.max_rows}")
         if R == 0:
             return []
-        h = self._host
-        for i in range(R):
-            h[0, i] = temperatures[i]
-            h[1, i] = top_ps[i]
-            h[2, i] = uniform(seeds[i], indices[i]) if temperatures[i] > 0 else 0.0
-        self._dev.copy_(h, non_blocking=True)
+        if not any(temperatures):
+            # all rows greedy: temperatures of zero are already on the device, nothing to upload
+            if not self._zeroed:
+                self._dev.zero_()
+                self._zeroed = True
+        else:
+            h = self._host_np
+            h[0, :R] = temperatures
+            h[1, :R] = top_ps
+            h[2, :R] = [uniform(s, i) if t > 0 else 0.0 for s, i, t in zip(seeds, indices, temperatures)]
+            self._dev.copy_(self._host, non_blocking=True)
+            self._zeroed = False
         kernels.sample(logits, self._dev[0], self._dev[1], self._dev[2], self._out)
         return self._out[:R].tolist()      # the one device-to-host sync of a step
