@@ -31,7 +31,7 @@ class EngineArgs:
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
-        if self.block_size < 8 or self.block_size % 8:
-            raise ValueError(f"block_size must be a positive multiple of 8, got {self.block_size}")
+        if self.block_size < 8 or self.block_size & (self.block_size - 1):
+            raise ValueError(f"block_size must be a power of two of at least 8, got {self.block_size}")
         if self.max_num_seqs < 1 or self.max_num_batched_tokens < 1 or self.max_seq_len < 1:
             raise ValueError("max_num_seqs, max_num_batched_tokens and max_seq_len must be positive")

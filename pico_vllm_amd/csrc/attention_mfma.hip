@@ -42,6 +42,11 @@ constexpr int BN = D <= 128 ? 64 : 32;   // keys per LDS tile
 constexpr int KROW = D + 8;              // LDS row strides in elements; the pad spreads rows over banks
 constexpr int VROW = BN + 8;
 constexpr int BM = 128;                  // queries per workgroup in the prefill kernel
+#if PICO_HEAD_DIM > 128
+#define PICO_ATTN_WAVES_PER_SIMD 1       // accumulators of a large head need the whole register file
+#else
+#define PICO_ATTN_WAVES_PER_SIMD 2
+#endif
 
 struct alignas(16) Tiles {
   alignas(16) bf16_t k[BN * KROW];    // [key][dim]
@@ -61,54 +66,60 @@ struct TileRegs {
   static constexpr int NV = (D * VCH + NT - 1) / NT;
   uint4 k[NK], v[NV];
 
+  // No branch stands between the loads: chunks that do not exist (beyond the tile's chunk count or
+  // beyond kv_end) read a clamped, valid address instead.  Keys beyond kv_end need no zeroing, their
+  // scores are masked; values do, which commit() takes care of.
   __device__ __forceinline__ void fetch(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-                                        const int* __restrict__ bt, int g, int nkv, int P, int num_pages,
+                                        const int* __restrict__ bt, int g, int nkv, int pshift, int num_pages,
                                         int tile_start, int kv_end) {
+    const int P = 1 << pshift, last_key = kv_end - 1, last_chunk = last_key & ~7;
 #pragma unroll
     for (int i = 0; i < NK; i++) {
-      const int c = threadIdx.x + i * NT;
-      const int key = c / KCH, dc = c % KCH;
-      const int pos = tile_start + key;
-      k[i] = make_uint4(0, 0, 0, 0);
-      if (c < BN * KCH && pos < kv_end) {
-        const int page = min(max(bt[pos / P], 0), num_pages - 1);
-        k[i] = *reinterpret_cast<const uint4*>(k_cache + (((size_t)page * nkv + g) * P + pos % P) * D + dc * 8);
-      }
+      const int c = min((int)threadIdx.x + i * NT, BN * KCH - 1);
+      const int pos = min(tile_start + c / KCH, last_key);
+      const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
+      k[i] = *reinterpret_cast<const uint4*>(k_cache + ((((size_t)page * nkv + g) << pshift) + (pos & (P - 1))) * D +
+                                             (c % KCH) * 8);
     }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-      const int c = threadIdx.x + i * NT;
-      const int dim = c / VCH, kc = c % VCH;
-      const int pos = tile_start + kc * 8;
-      v[i] = make_uint4(0, 0, 0, 0);
-      if (c < D * VCH && pos < kv_end) {
-        const int page = min(max(bt[pos / P], 0), num_pages - 1);
-        v[i] = *reinterpret_cast<const uint4*>(v_cache + (((size_t)page * nkv + g) * D + dim) * P + pos % P);
-      }
+      const int c = min((int)threadIdx.x + i * NT, D * VCH - 1);
+      const int pos = min(tile_start + (c % VCH) * 8, last_chunk);
+      const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
+      v[i] = *reinterpret_cast<const uint4*>(v_cache + ((((size_t)page * nkv + g) * D + c / VCH) << pshift) + (pos & (P - 1)));
     }
   }
 
+  // LDS layout of V^T: per head dimension a row of BN values in OPERAND order: the 8 values that lane
+  // half h feeds into product m of sub-tile sub (keys 16 m + 4 h + 0..3 and 16 m + 8 + 4 h + 0..3 of the
+  // sub-tile) are contiguous, so the P.V loop reads one 16-byte unit per product.  A chunk from
+  // memory (8 consecutive keys) splits into two 8-byte halves that go to the units of h = 0 and 1.
   __device__ __forceinline__ void commit(Tiles& t, int tile_start, int kv_end) const {
 #pragma unroll
     for (int i = 0; i < NK; i++) {
       const int c = threadIdx.x + i * NT;
       if (c < BN * KCH) *reinterpret_cast<uint4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
     }
+    const bool tail = tile_start + BN > kv_end;              // the same for the whole workgroup
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int c = threadIdx.x + i * NT;
       if (c >= D * VCH) continue;
       const int dim = c / VCH, kc = c % VCH;
-      const int pos = tile_start + kc * 8;
       uint4 x = v[i];
-      if (pos < kv_end && pos + 8 > kv_end) {   // the tail of the last chunk holds whatever the page held before
+      if (tail) {   // values of keys at or beyond kv_end hold whatever the page held before
+        const int pos = tile_start + kc * 8;
         uint32_t w[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
         for (int e = 0; e < 8; e++)
           if (pos + e >= kv_end) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
         x = make_uint4(w[0], w[1], w[2], w[3]);
       }
-      *reinterpret_cast<uint4*>(&t.vt[dim * VROW + kc * 8]) = x;
+      // chunk kc covers keys 8 kc .. 8 kc + 7 of the tile: sub-tile kc / 4, product (kc % 4) / 2,
+      // first or second group of four slots by kc % 2
+      bf16_t* unit = &t.vt[dim * VROW + (kc >> 1) * 16 + (kc & 1) * 4];
+      *reinterpret_cast<uint2*>(unit) = make_uint2(x.x, x.y);          // keys +0..3: half h = 0
+      *reinterpret_cast<uint2*>(unit + 8) = make_uint2(x.z, x.w);      // keys +4..7: half h = 1
     }
   }
 };
@@ -188,11 +199,93 @@ __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf
     const bf16x8 b = __builtin_bit_cast(bf16x8, make_uint4(pk[0], pk[1], pk[2], pk[3]));
 #pragma unroll
     for (int tt = 0; tt < DT; tt++) {
-      const bf16_t* vrow = &t.vt[(tt * 32 + col) * VROW + sub * 32 + 16 * m + 4 * h];
-      const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-      const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
-      const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+      const bf16x8 a = __builtin_bit_cast(
+          bf16x8, *reinterpret_cast<const uint4*>(&t.vt[(tt * 32 + col) * VROW + sub * 32 + 16 * m + 8 * h]));
       st.o[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, st.o[tt], 0, 0, 0);
+    }
+  }
+}
+
+// A whole LDS tile (its first nsub 32-key sub-tiles) against the wave's 32 query columns with ONE
+// softmax update, for the prefill kernel, whose cost is vector instructions rather than matrix ones:
+//   * scores stay raw; p = 2^(s c - m c) with c = scale * log2(e) is one fused multiply-add and
+//     one v_exp_f32 per score;
+//   * the reference maximum m may lag behind the true running maximum by up to 8 in the exponent
+//     (p <= 256, harmless in float32 sums and in bfloat16 P); the accumulators are rescaled only
+//     when some column of the wave outgrows that, which after the first tiles of a row is rare.
+//     Output and sum share the reference, so o / l is unchanged by the lag.
+template <int NS>
+__device__ __forceinline__ void attend_tile(const Tiles& t, int nsub, const bf16x8* q, WaveState& st, float c,
+                                            int key_pos0, int q_pos, bool need_mask) {
+  const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  f32x16 s[NS];
+#pragma unroll
+  for (int sub = 0; sub < NS; sub++) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[sub][r] = 0.f;
+    if (sub < nsub) {
+      const bf16_t* krow = &t.k[(sub * 32 + col) * KROW + 8 * h];
+#pragma unroll
+      for (int step = 0; step < KSTEPS; step++) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + 16 * step));
+        s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q[step], s[sub], 0, 0, 0);
+      }
+    }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int sub = 0; sub < NS; sub++) {
+    if (sub < nsub) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        if (need_mask && key_pos0 + 32 * sub + 8 * (r >> 2) + 4 * h + (r & 3) > q_pos) s[sub][r] = -INFINITY;
+        mx = fmaxf(mx, s[sub][r]);
+      }
+    }
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(st.m, mx);
+  const bool outgrown = (m_new - st.m) * c > 8.0f;          // also true while the reference is -inf
+  if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {          // the same decision for the whole wave
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((st.m - m_use) * c);
+    st.l *= alpha;
+    st.m = m_new;
+#pragma unroll
+    for (int tt = 0; tt < DT; tt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) st.o[tt][r] *= alpha;
+  }
+  const float mc = ((st.m == -INFINITY) ? 0.f : st.m) * c;
+  float sum = 0.f;
+#pragma unroll
+  for (int sub = 0; sub < NS; sub++) {
+    if (sub < nsub) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[sub][r], c, -mc));
+        s[sub][r] = p;
+        sum += p;
+      }
+    }
+  }
+  sum += __shfl_xor(sum, 32, 64);
+  st.l += sum;
+#pragma unroll
+  for (int sub = 0; sub < NS; sub++) {
+    if (sub < nsub) {
+#pragma unroll
+      for (int m = 0; m < 2; m++) {
+        const bf16x8 b = __builtin_bit_cast(
+            bf16x8, make_uint4(pack2_bf16(s[sub][8 * m], s[sub][8 * m + 1]), pack2_bf16(s[sub][8 * m + 2], s[sub][8 * m + 3]),
+                               pack2_bf16(s[sub][8 * m + 4], s[sub][8 * m + 5]), pack2_bf16(s[sub][8 * m + 6], s[sub][8 * m + 7])));
+#pragma unroll
+        for (int tt = 0; tt < DT; tt++) {
+          const bf16x8 a = __builtin_bit_cast(
+              bf16x8, *reinterpret_cast<const uint4*>(&t.vt[(tt * 32 + col) * VROW + sub * 32 + 16 * m + 8 * h]));
+          st.o[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, st.o[tt], 0, 0, 0);
+        }
+      }
     }
   }
 }
@@ -211,7 +304,7 @@ __device__ __forceinline__ void load_q(bf16x8* q, const bf16_t* qrow, bool ok) {
 // ---------------------------------------------------------------------------
 // prefill / mixed batches
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16_t* __restrict__ q, int q_stride,
+__global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void prefill_kernel(const bf16_t* __restrict__ q, int q_stride,
                                                       const bf16_t* __restrict__ k_cache,
                                                       const bf16_t* __restrict__ v_cache,
                                                       const int* __restrict__ block_table, int max_pages,
@@ -245,23 +338,22 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16_t* __restric
   const bool wave_active = tile * BM + wave * 32 < new_len;
   const int kv_end = min(ctx, prefix + min(new_len, (tile + 1) * BM));  // keys beyond the tile's last query are never needed
 
+  const float c = scale * 1.4426950408889634f;               // scores go through 2^x
+  const int pshift = 31 - __clz(P);                          // page sizes are powers of two
   WaveState st;
   init_state(st);
   zero_pad_rows(tiles, 256);
   TileRegs<256> regs;
-  regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, 0, kv_end);
+  regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, 0, kv_end);
   for (int tile_start = 0; tile_start < kv_end; tile_start += BN) {
     __syncthreads();                                          // everyone is done with the previous tile
     regs.commit(tiles, tile_start, kv_end);
     __syncthreads();
-    if (tile_start + BN < kv_end) regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start + BN, kv_end);
-    if (!wave_active) continue;
-#pragma unroll
-    for (int sub = 0; sub < BN / 32; sub++) {
-      const int key0 = tile_start + sub * 32;
-      if (key0 > wave_last_pos) break;                        // wholly beyond the causal frontier of this wave
-      attend_subtile(tiles, sub, qf, st, scale, key0, q_pos, key0 + 31 > wave_first_pos);
-    }
+    if (tile_start + BN < kv_end) regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, tile_start + BN, kv_end);
+    if (!wave_active || tile_start > wave_last_pos) continue;
+    // sub-tiles wholly beyond the causal frontier of this wave are left out
+    const int nsub = min(BN / 32, (wave_last_pos - tile_start) / 32 + 1);
+    attend_tile<BN / 32>(tiles, nsub, qf, st, c, tile_start, q_pos, tile_start + 32 * nsub - 1 > wave_first_pos);
   }
   if (!q_ok) return;
   const float inv_l = 1.0f / st.l;
@@ -284,7 +376,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16_t* __restric
 // decode: one query token per sequence, the G heads of a kv group as the 32 columns
 // ---------------------------------------------------------------------------
 // partial results per (sequence, query head, split): o [D] unnormalised, then m and l
-__global__ __launch_bounds__(256, 2) void decode_kernel(const bf16_t* __restrict__ q, int q_stride,
+__global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(const bf16_t* __restrict__ q, int q_stride,
                                                      const bf16_t* __restrict__ k_cache,
                                                      const bf16_t* __restrict__ v_cache,
                                                      const int* __restrict__ block_table, int max_pages,
@@ -302,6 +394,7 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(const bf16_t* __restrict
   const int* bt = block_table + (size_t)b * max_pages;
   const bool col_ok = col < G;
   const int head = g * G + (col_ok ? col : 0);
+  const int pshift = 31 - __clz(P);
   bf16x8 qf[KSTEPS];
   load_q(qf, q + (size_t)b * q_stride + (size_t)head * D, col_ok && ctx > 0);
 
@@ -309,12 +402,12 @@ __global__ __launch_bounds__(256, 2) void decode_kernel(const bf16_t* __restrict
   init_state(st);
   zero_pad_rows(tiles, 256);
   TileRegs<256> regs;
-  if (k_begin < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, k_begin, k_end);
+  if (k_begin < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, k_begin, k_end);
   for (int tile_start = k_begin; tile_start < k_end; tile_start += BN) {
     __syncthreads();
     regs.commit(tiles, tile_start, k_end);
     __syncthreads();
-    if (tile_start + BN < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, P, num_pages, tile_start + BN, k_end);
+    if (tile_start + BN < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, tile_start + BN, k_end);
     for (int sub = wave; sub < BN / 32 && wave < 2; sub += 2) {   // waves 2 and 3 only help to move the tiles
       const int key0 = tile_start + sub * 32;
       if (key0 >= k_end) break;
@@ -404,6 +497,7 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
   for (int tt = 0; tt < DT16; tt++) o[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int first = k_begin + 32 * wave;
+  const int pshift = 31 - __clz(P);                             // page sizes are powers of two
   if (first < k_end) {
     const int last = first + (k_end - 1 - first) / 128 * 128;   // this wave's last block
     const int last_key = k_end - 1, last_group = last_key / 4 * 4;
@@ -414,8 +508,8 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int pos = min(key0 + 16 * t + col, last_key);
-        const int page = min(max(bt[pos / P], 0), num_pages - 1);
-        const bf16_t* kp = k_cache + (((size_t)page * nkv + g) * P + pos % P) * D + (D / 4) * kq;
+        const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
+        const bf16_t* kp = k_cache + ((((size_t)page * nkv + g) << pshift) + (pos & (P - 1))) * D + (D / 4) * kq;
 #pragma unroll
         for (int st = 0; st < KS16; st++) kr[t][st] = *reinterpret_cast<const uint4*>(kp + 8 * st);
       }
@@ -424,10 +518,10 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int pos = min(key0 + 16 * t + 4 * kq, last_group);
-        const int page = min(max(bt[pos / P], 0), num_pages - 1);
-        const bf16_t* vp = v_cache + (((size_t)page * nkv + g) * D + col) * P + pos % P;
+        const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
+        const bf16_t* vp = v_cache + ((((size_t)page * nkv + g) * D + col) << pshift) + (pos & (P - 1));
 #pragma unroll
-        for (int tt = 0; tt < DT16; tt++) vr[tt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)tt * 16 * P);
+        for (int tt = 0; tt < DT16; tt++) vr[tt][t] = *reinterpret_cast<const uint2*>(vp + ((size_t)tt * 16 << pshift));
       }
     };
     load_k(first);
@@ -593,7 +687,7 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restri
 static int check_common(const char* who, int nq, int nkv, int d, int P, int max_pages, int num_pages, int q_stride) {
   PICO_REQUIRE(d == D, "%s: this library is built for head size %d, got %d", who, D, d);
   PICO_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "%s: %d query heads are not a multiple of %d kv heads", who, nq, nkv);
-  PICO_REQUIRE(P > 0 && P % 8 == 0, "%s: page size %d is not a multiple of 8", who, P);
+  PICO_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "%s: page size %d is not a power of two of at least 8", who, P);
   PICO_REQUIRE(max_pages > 0 && num_pages > 0, "%s: empty block table or cache", who);
   PICO_REQUIRE(q_stride >= nq * D && q_stride % 8 == 0, "%s: query row stride %d must be a multiple of 8 and hold all heads", who, q_stride);
   return 0;
@@ -630,7 +724,7 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
   dim3 grid(num_seqs, nkv, nsplit);
   bool direct = false;
 #if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
-  direct = nq / nkv <= 16 && P % 4 == 0;
+  direct = nq / nkv <= 16;
   if (direct)
     decode16_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                              (const bf16_t*)v_cache, block_table, max_pages, context_lens, part,
