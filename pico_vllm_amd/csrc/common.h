@@ -37,7 +37,9 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_ca
 
 // two floats as two bfloat16 in one 32-bit word (a in the low half)
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
-  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t));
 }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p);

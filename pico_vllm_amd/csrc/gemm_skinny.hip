@@ -73,37 +73,43 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   // this wave's slices start at k_begin + 64 (wave + 4 i)
   const int first = k_begin + 64 * wave;
   if (!TAIL) {
-    // K % 64 == 0: every slice is whole.  Straight-line code with two stages in flight: the loads of
-    // the next slice are always issued (the last iteration re-reads its own slice, which is cached)
-    // so that no branch stands between a load and the wait for the stage before it.
-    auto load_stage = [&](Stage& st, int k0) {
-#pragma unroll
-      for (int s = 0; s < 4; s++) {
-        st.w[s] = *reinterpret_cast<const uint4*>(wrow0 + k0 + 32 * h + 8 * s);
-#pragma unroll
-        for (int t = 0; t < MT; t++) st.x[t][s] = *reinterpret_cast<const uint4*>(xrow0[t] + k0 + 32 * h + 8 * s);
-      }
-    };
+    // K % 64 == 0: every slice is whole.  DEPTH slices are in flight per wave.  The slices are
+    // taken in rounds of DEPTH: inside a round there is no branch (a branch between a load and the
+    // wait for an older one makes the compiler wait for everything); every step of a round
+    // multiplies one stage and refills it with the slice DEPTH ahead (beyond the wave's last
+    // slice the last one is read again and not used); the last round, the only one that can be
+    // partial, does not refill and multiplies only the slices that exist.
+    constexpr int DEPTH = MT == 1 ? 3 : 2;
     if (first < k_end) {
-      const int last = first + (k_end - 1 - first) / 256 * 256;     // start of this wave's last slice
-      Stage sa, sb;
-      load_stage(sa, first);
-      // the scheduling barriers keep the compiler from sinking the loads next to their use, which
-      // would leave only two of them in flight
-      for (int k0 = first;;) {
-        load_stage(sb, min(k0 + 256, last));
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(sa);
-        __builtin_amdgcn_sched_barrier(0);
-        k0 += 256;
-        if (k0 > last) break;
-        load_stage(sa, min(k0 + 256, last));
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(sb);
-        __builtin_amdgcn_sched_barrier(0);
-        k0 += 256;
-        if (k0 > last) break;
+      const int n_slices = (k_end - first + 255) / 256;
+      const int rounds = (n_slices + DEPTH - 1) / DEPTH;
+      const int last = first + (n_slices - 1) * 256;
+      auto load_stage = [&](Stage& st, int slice) {
+        const int k0 = min(first + 256 * slice, last);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          st.w[s] = *reinterpret_cast<const uint4*>(wrow0 + k0 + 32 * h + 8 * s);
+#pragma unroll
+          for (int t = 0; t < MT; t++) st.x[t][s] = *reinterpret_cast<const uint4*>(xrow0[t] + k0 + 32 * h + 8 * s);
+        }
+      };
+      Stage st[DEPTH];
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++) load_stage(st[d], d);
+      __builtin_amdgcn_sched_barrier(0);
+      for (int r = 0; r + 1 < rounds; r++) {      // every slice of these rounds exists
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+          multiply(st[d]);
+          __builtin_amdgcn_sched_barrier(0);     // keeps the refill from sinking next to its use
+          load_stage(st[d], (r + 1) * DEPTH + d);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+      const int left = n_slices - (rounds - 1) * DEPTH;           // 1..DEPTH slices in the last round
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++)
+        if (d < left) multiply(st[d]);
     }
   } else {
     for (int k0 = first; k0 < k_end; k0 += 256) {
