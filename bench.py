@@ -135,6 +135,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--write-model", metavar="DIR", default=None,
+                    help="only write the random-weights model folder to DIR (to reuse with --model) and exit")
     ap.add_argument("--model", default=None, help="reuse a model folder instead of writing random weights")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -145,6 +147,10 @@ def main() -> int:
         return 2
     import torch
     from pico_vllm_amd.weights.random_init import write_random_model
+    if a.write_model:
+        write_random_model(a.write_model, CONFIG_1P5B, seed=0)
+        print(f"wrote {a.write_model}")
+        return 0
     tmp = None
     model_dir = a.model
     if model_dir is None:

@@ -73,7 +73,15 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   TO* o = out + (size_t)blockIdx.x * H;
   float ss = 0.f;
   if (VEC) {
-    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+    // up to VPT groups of four elements per thread stay in registers from the sum of squares to
+    // the scaling; a longer row is read again for the second pass
+    constexpr int VPT = 4;
+    const int stride = blockDim.x * 4;
+    const bool in_regs = H <= VPT * stride;
+    float4 keep[VPT];
+#pragma unroll
+    for (int j = 0; j < VPT; j++) keep[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = threadIdx.x * 4, j = 0; i < H; i += stride, j++) {
       float4 v = *reinterpret_cast<const float4*>(x + i);
       if (dl) {
         float4 d[MAX_SLABS];
@@ -85,40 +93,50 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
         if (!rows) *reinterpret_cast<float4*>(x + i) = v;
       }
       ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-    }
-  } else {
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-      float v = x[i];
-      if (dl) {
-        for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
-        if (!rows) x[i] = v;
+      if (in_regs) {
+#pragma unroll
+        for (int jj = 0; jj < VPT; jj++)
+          if (jj == j) keep[jj] = v;
       }
-      ss += v * v;
     }
-  }
-  ss = block_sum(ss, scratch);
-  const float r = 1.0f / sqrtf(ss / (float)H + eps);
-  if (VEC) {
-    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
-      float4 v = *reinterpret_cast<const float4*>(x + i);
-      if (dl && rows) {
-        float4 d[MAX_SLABS];
+    ss = block_sum(ss, scratch);
+    const float r = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x * 4, j = 0; i < H; i += stride, j++) {
+      float4 v;
+      if (in_regs) {
+        v = keep[0];
 #pragma unroll
-        for (int s = 0; s < MAX_SLABS; s++)
-          d[s] = s < slabs ? load4_f32(dl + s * slab_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int s = 0; s < MAX_SLABS; s++) { v.x += d[s].x; v.y += d[s].y; v.z += d[s].z; v.w += d[s].w; }
+        for (int jj = 1; jj < VPT; jj++)
+          if (jj == j) v = keep[jj];
+      } else {
+        v = *reinterpret_cast<const float4*>(x + i);
+        if (dl && rows) {
+          for (int s = 0; s < slabs; s++) {
+            const float4 d = load4_f32(dl + s * slab_stride + i);
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+          }
+        }
       }
       const float4 g = *reinterpret_cast<const float4*>(w + i);
       store4_f32(o + i, make_float4(v.x * r * g.x, v.y * r * g.y, v.z * r * g.z, v.w * r * g.w));
     }
-  } else {
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-      float v = x[i];
-      if (dl && rows)
-        for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
-      store_f32(o + i, v * r * w[i]);
+    return;
+  }
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (dl) {
+      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
+      if (!rows) x[i] = v;
     }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (dl && rows)
+      for (int s = 0; s < slabs; s++) v += load_f32(dl + s * slab_stride + i);
+    store_f32(o + i, v * r * w[i]);
   }
 }
 
@@ -213,15 +231,16 @@ extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, h
 // qkv: [T, (nq + 2 nkv) * d], rows [q heads | k heads | v heads]; q is rotated in place.
 // Cache of one layer: K pages [page][kv head][slot in page][d],
 //                     V pages [page][kv head][d][slot in page]  (slot contiguous).
-// A token at position p of sequence s goes to page block_table[s][p / P], slot p % P.
+// slots[t] = page * P + position % P says where token t's key and value go (the host computes it
+// from the block table, as the reference does, pico_vllm/cache.py:143-156); a negative slot means
+// "store nothing" (padding rows of a captured batch).
 // Grid (T, nq + nkv); block 64.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
-                                  const int* __restrict__ token_seq, const int* __restrict__ block_table,
-                                  int max_pages, const float* __restrict__ inv_freq, T* __restrict__ k_cache,
-                                  T* __restrict__ v_cache, int nq, int nkv, int d, int rot, int P,
-                                  int num_pages) {
+                                  const int* __restrict__ slots, const float* __restrict__ inv_freq,
+                                  T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv, int d, int rot,
+                                  int P, int num_pages) {
   const int t = blockIdx.x, head = blockIdx.y;
   const int pos = positions[t];
   T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
@@ -238,9 +257,9 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
     return;
   }
   const int g = head - nq;
-  const int page = block_table[(size_t)token_seq[t] * max_pages + pos / P];
-  if (page < 0 || page >= num_pages) return;  // the host has checked; stay in bounds regardless
-  const int off = pos % P;
+  const int slot = slots[t];
+  const int page = slot / P, off = slot % P;
+  if (slot < 0 || page >= num_pages) return;  // padding row; the host has checked the rest
   const T* k = row + (size_t)(nq + g) * d;
   const T* v = row + (size_t)(nq + nkv + g) * d;
   T* kc = k_cache + (((size_t)page * nkv + g) * P + off) * d;
@@ -256,23 +275,19 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
   for (int j = threadIdx.x; j < d; j += blockDim.x) vc[(size_t)j * P] = v[j];
 }
 
-extern "C" int pico_rope_kv_store(void* qkv, int dtype, const int* positions, const int* token_seq,
-                                  const int* block_table, int max_pages, const float* inv_freq, void* k_cache,
-                                  void* v_cache, int T, int nq, int nkv, int d, int rot, int P, int num_pages,
-                                  hipStream_t stream) {
-  PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && d > 0 && P > 0 && max_pages > 0 && num_pages > 0,
-               "pico_rope_kv_store: bad sizes");
+extern "C" int pico_rope_kv_store(void* qkv, int dtype, const int* positions, const int* slots,
+                                  const float* inv_freq, void* k_cache, void* v_cache, int T, int nq, int nkv, int d,
+                                  int rot, int P, int num_pages, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && d > 0 && P > 0 && num_pages > 0, "pico_rope_kv_store: bad sizes");
   PICO_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "pico_rope_kv_store: rotary size %d does not fit head size %d", rot, d);
   if (T == 0) return 0;
   dim3 grid(T, nq + nkv);
   if (dtype == PICO_DTYPE_F32)
-    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, positions, token_seq, block_table, max_pages,
-                                                      inv_freq, (float*)k_cache, (float*)v_cache, nq, nkv, d, rot,
-                                                      P, num_pages);
+    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, positions, slots, inv_freq, (float*)k_cache,
+                                                      (float*)v_cache, nq, nkv, d, rot, P, num_pages);
   else if (dtype == PICO_DTYPE_BF16)
-    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, positions, token_seq, block_table, max_pages,
-                                                       inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, nq, nkv, d,
-                                                       rot, P, num_pages);
+    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, positions, slots, inv_freq, (bf16_t*)k_cache,
+                                                       (bf16_t*)v_cache, nq, nkv, d, rot, P, num_pages);
   else
     PICO_REQUIRE(false, "pico_rope_kv_store: unknown dtype %d", dtype);
   PICO_LAUNCH_CHECK();

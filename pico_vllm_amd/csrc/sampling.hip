@@ -17,9 +17,18 @@
 __device__ __forceinline__ float masked_sum(const float* __restrict__ x, int V, float mx, float inv_t, float thr,
                                             bool inclusive, float* scratch) {
   float s = 0.f;
-  for (int i = threadIdx.x; i < V; i += SAMPLE_THREADS) {
-    const float e = expf((x[i] - mx) * inv_t);
-    if (inclusive ? (e >= thr) : (e > thr)) s += e;
+  for (int i0 = threadIdx.x; i0 < V; i0 += 8 * SAMPLE_THREADS) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int i = i0 + j * SAMPLE_THREADS;
+      v[j] = i < V ? x[i] : -INFINITY;           // exp(-inf) = 0 adds nothing
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float e = expf((v[j] - mx) * inv_t);
+      if (inclusive ? (e >= thr) : (e > thr)) s += e;
+    }
   }
   return block_sum(s, scratch);
 }
@@ -41,9 +50,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   // max and its first index
   float mx = -INFINITY;
   int mi = 0x7fffffff;
-  for (int i = tid; i < V; i += SAMPLE_THREADS) {
-    const float v = x[i];
-    if (v > mx || (v == mx && i < mi)) { mx = v; mi = i; }
+  // eight loads in flight per thread; indices rise within a thread, so ">" keeps the first maximum
+  for (int i0 = tid; i0 < V; i0 += 8 * SAMPLE_THREADS) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int i = i0 + j * SAMPLE_THREADS;
+      v[j] = i < V ? x[i] : -INFINITY;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (v[j] > mx) { mx = v[j]; mi = i0 + j * SAMPLE_THREADS; }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {

@@ -39,7 +39,8 @@ class BatchBuffers:
         self.device = device
         self.max_tokens, self.max_seqs, self.max_pages, self.num_groups = max_tokens, max_seqs, max_pages, num_groups
         self.max_want = max_want if max_want is not None else max_tokens
-        n = 3 * max_tokens + (max_seqs + 1) + 2 * max_seqs + self.max_want + num_groups * max_seqs * max_pages
+        n = (3 + num_groups) * max_tokens + (max_seqs + 1) + 2 * max_seqs + self.max_want \
+            + num_groups * max_seqs * max_pages
         self.host = torch.zeros(n, dtype=torch.int32, pin_memory=torch.cuda.is_available())
         self.dev = torch.zeros(n, dtype=torch.int32, device=device)
         self.copied = torch.cuda.Event() if torch.cuda.is_available() else None
@@ -71,7 +72,8 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         buf.copied.synchronize()          # the previous step's copy has left the pinned buffer
     h = buf.host.numpy()
     h_tok, h_pos, h_seq = h[0:T], h[buf.max_tokens:buf.max_tokens + T], h[2 * buf.max_tokens:2 * buf.max_tokens + T]
-    o = 3 * buf.max_tokens
+    h_slots = [h[(3 + g) * buf.max_tokens:(3 + g) * buf.max_tokens + T] for g in range(G)]
+    o = (3 + G) * buf.max_tokens
     h_cu = h[o:o + rows + 1]; o += buf.max_seqs + 1
     h_ctx = h[o:o + rows]; o += buf.max_seqs
     h_slot = h[o:o + rows]; o += buf.max_seqs
@@ -135,14 +137,20 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
     tables[:] = -1
     for b, s in enumerate(seqs):
         need = -(-int(h_ctx[b]) // P)
+        lo, hi = int(h_cu[b]), int(h_cu[b + 1])
         for g in range(G):
-            tables[g, b, :need] = manager.block_table_array(s.req, g, need)
+            table = manager.block_table_array(s.req, g, need)
+            tables[g, b, :need] = table
+            pos = h_pos[lo:hi]
+            h_slots[g][lo:hi] = table[pos // P] * P + pos % P          # pico_vllm/cache.py:143-156
+    for g in range(G):
+        h_slots[g][int(h_cu[B]):T] = -1                               # padding rows store nothing
     used = bt_off + G * rows * width
     buf.dev[:used].copy_(buf.host[:used], non_blocking=True)
     if buf.copied is not None:
         buf.copied.record()
     d = buf.dev
-    o = 3 * buf.max_tokens
+    o = (3 + G) * buf.max_tokens
     ctx = StepContext(
         num_tokens=T, num_seqs=rows,
         token_ids=d[0:T], positions=d[buf.max_tokens:buf.max_tokens + T],
@@ -152,6 +160,7 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         state_slots=d[o + 2 * buf.max_seqs + 1:o + 2 * buf.max_seqs + 1 + rows],
         want_rows=d[o + 3 * buf.max_seqs + 1:o + 3 * buf.max_seqs + 1 + R],
         block_tables=[d[bt_off + g * rows * width:bt_off + (g + 1) * rows * width].view(rows, width) for g in range(G)],
+        slot_mapping=[d[(3 + g) * buf.max_tokens:(3 + g) * buf.max_tokens + T] for g in range(G)],
         act_dtype=act_dtype,
         max_new_tokens=max(lens), max_context=max_ctx, all_decode=max(lens) == 1,
         host={"cu_seqlens": h_cu.copy(), "context_lens": h_ctx.copy()},

@@ -270,11 +270,11 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int)
     return pages, P
 
 
-def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
-                  inv_freq: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, nq: int, nkv: int, d: int,
-                  rotary_dim: int) -> None:
-    """Rotate q (in place) and k, write k and v of every token into its page."""
-    _gpu(qkv, positions, token_seq, block_table, inv_freq, k_cache, v_cache)
+def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, inv_freq: torch.Tensor,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, nq: int, nkv: int, d: int, rotary_dim: int) -> None:
+    """Rotate q (in place) and k, write k and v of token t to slot ``slots[t]`` (page * page size +
+    offset in the page; negative: nothing is stored)."""
+    _gpu(qkv, positions, slots, inv_freq, k_cache, v_cache)
     T = qkv.shape[0]
     if qkv.shape != (T, (nq + 2 * nkv) * d) or not qkv.is_contiguous():
         raise KernelError(f"qkv must be contiguous [T, {(nq + 2 * nkv) * d}], got {tuple(qkv.shape)}")
@@ -282,15 +282,12 @@ def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, token_seq: torch.T
     if k_cache.dtype != qkv.dtype:
         raise KernelError("cache and activations differ in dtype")
     _i32(positions, "positions", T)
-    _i32(token_seq, "token_seq", T)
-    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
-        raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+    _i32(slots, "slots", T)
     if inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2 or not inv_freq.is_contiguous():
         raise KernelError("inv_freq must be float32 of rotary_dim / 2 entries")
     lib = library.core()
-    _check(lib, lib.pico_rope_kv_store(_ptr(qkv), _dt(qkv), _ptr(positions), _ptr(token_seq), _ptr(block_table),
-                                       block_table.shape[1], _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), T, nq,
-                                       nkv, d, rotary_dim, P, pages, _stream()))
+    _check(lib, lib.pico_rope_kv_store(_ptr(qkv), _dt(qkv), _ptr(positions), _ptr(slots), _ptr(inv_freq),
+                                       _ptr(k_cache), _ptr(v_cache), T, nq, nkv, d, rotary_dim, P, pages, _stream()))
 
 
 def paged_attention_ref(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

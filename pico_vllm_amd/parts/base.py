@@ -39,6 +39,7 @@ class StepContext:
     context_lens: torch.Tensor       # int32 [B]   cached + new tokens
     state_slots: torch.Tensor        # int32 [B]   slot of fixed-size state
     block_tables: List[torch.Tensor]  # per cache group: int32 [B, max_pages]
+    slot_mapping: List[torch.Tensor]  # per cache group: int32 [T], page * page size + offset of each token (-1: none)
     want_rows: torch.Tensor          # int32 [R]   flat token indices whose logits are wanted
     act_dtype: torch.dtype
     # host-side facts for choosing kernels (fixed at capture time under a graph)

@@ -28,7 +28,7 @@ class RotaryHalf(PositionEncoding):
         self.inv_freq = inv.to(device).contiguous()
 
     def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
-        kernels.rope_kv_store(qkv, ctx.positions, ctx.token_seq, block_table, self.inv_freq,
+        kernels.rope_kv_store(qkv, ctx.positions, ctx.slot_mapping[kv.group], self.inv_freq,
                               kv.k, kv.v, nq, nkv, d, self.rotary_dim)
 
 
@@ -43,5 +43,5 @@ class NoPosition(PositionEncoding):
         self._empty = torch.zeros(0, dtype=torch.float32, device=device)
 
     def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
-        kernels.rope_kv_store(qkv, ctx.positions, ctx.token_seq, block_table, self._empty,
+        kernels.rope_kv_store(qkv, ctx.positions, ctx.slot_mapping[kv.group], self._empty,
                               kv.k, kv.v, nq, nkv, d, 0)

@@ -131,7 +131,9 @@ def test_rope_and_cache_store(K, dtype, nq, nkv, d, rot, Pg):
             bt[b, j] = perm.pop()
     inv = (1.0 / (theta ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
     x = qkv.clone().to(DEV)
-    K.rope_kv_store(x, pos, seq, bt.to(DEV), inv, kc, vc, nq, nkv, d, rot)
+    slots = torch.tensor([int(bt[int(b), int(p) // Pg]) * Pg + int(p) % Pg for b, p in zip(seq, pos)],
+                         dtype=torch.int32, device=DEV)
+    K.rope_kv_store(x, pos, slots, inv, kc, vc, nq, nkv, d, rot)
     # reference
     q, k, v = P.split_qkv(qkv.float(), nq, nkv, d)
     cos, sin = P.rope_tables(pos.cpu(), rot, theta)
