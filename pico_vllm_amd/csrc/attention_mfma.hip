@@ -32,6 +32,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int D = PICO_HEAD_DIM;
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
@@ -64,7 +65,8 @@ struct TileRegs {
   static constexpr int VCH = BN / 8;                       // 16-byte chunks (8 keys) per head dimension
   static constexpr int NK = (BN * KCH + NT - 1) / NT;      // chunks per thread
   static constexpr int NV = (D * VCH + NT - 1) / NT;
-  uint4 k[NK], v[NV];
+  u32x4 k[NK];                              // plain vectors: a struct copy would go through memory
+  uint4 v[NV];
 
   // No branch stands between the loads: chunks that do not exist (beyond the tile's chunk count or
   // beyond kv_end) read a clamped, valid address instead.  Keys beyond kv_end need no zeroing, their
@@ -78,7 +80,7 @@ struct TileRegs {
       const int c = min((int)threadIdx.x + i * NT, BN * KCH - 1);
       const int pos = min(tile_start + c / KCH, last_key);
       const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
-      k[i] = *reinterpret_cast<const uint4*>(k_cache + ((((size_t)page * nkv + g) << pshift) + (pos & (P - 1))) * D +
+      k[i] = *reinterpret_cast<const u32x4*>(k_cache + ((((size_t)page * nkv + g) << pshift) + (pos & (P - 1))) * D +
                                              (c % KCH) * 8);
     }
 #pragma unroll
@@ -98,7 +100,7 @@ struct TileRegs {
 #pragma unroll
     for (int i = 0; i < NK; i++) {
       const int c = threadIdx.x + i * NT;
-      if (c < BN * KCH) *reinterpret_cast<uint4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
+      if (c < BN * KCH) *reinterpret_cast<u32x4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
     }
     const bool tail = tile_start + BN > kv_end;              // the same for the whole workgroup
 #pragma unroll
@@ -371,6 +373,308 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void prefill_kernel(
       }
     }
 }
+
+// ---------------------------------------------------------------------------
+// prefill / mixed batches for head sizes that are multiples of 32: 16 queries per wave
+// ---------------------------------------------------------------------------
+// v_mfma_f32_16x16x32_bf16 (A 16x32, B 32x16): lane l = (c, kq) = (l % 16, l / 16) supplies
+// A[c][8 kq + 0..7] and B[8 kq + 0..7][c] and receives D[4 kq + r][c] in register r.
+// A workgroup owns 64 queries of one sequence and one head.  Its waves form KT teams of four;
+// the four waves of a team own 16 queries each, and team t works on keys 64 t .. 64 t + 63 of every
+// LDS tile of 64 KT keys, so the long key loop of a late query tile is shared by KT waves per
+// SIMD whose softmax and matrix products overlap; the teams' results are merged through LDS at the
+// end.  A wave's accumulators (O^T: D x 16) take D / 4 registers.  Per 64 keys the scores are four
+// 16 x 16 blocks of S^T = K Q^T.  Which key is row a of block j is free; it is key
+// 32 (j / 2) + 8 (a / 4) + 4 (j % 2) + a % 4, so that the registers of lane quarter kq in the pair
+// of blocks (2 m, 2 m + 1) hold the eight consecutive keys 32 m + 8 kq + 0..7.  Rounded to bfloat16
+// they are the B operand of O^T += V^T P^T with contraction slot 8 kq + i = key 32 m + 8 kq + i,
+// and the A operand is 16 contiguous bytes of V^T as the pages hold it.
+// Offsets into the cache are 32-bit byte offsets: the host checks that K and V are below 4 GiB.
+#if PICO_HEAD_DIM % 32 == 0
+typedef float f32x4p __attribute__((ext_vector_type(4)));
+constexpr int PF_BM = 64;                         // queries per workgroup
+constexpr int PF_KT_MAX = D <= 128 ? 2 : 1;       // teams of four waves: one or two
+constexpr int PF_KS = D / 32;                     // contraction steps of a 16-key block
+constexpr int PF_DT = D / 16;                     // 16-wide tiles of the output's head dimension
+
+template <int KT>
+struct alignas(16) PfTiles {
+  static constexpr int TK = 64 * KT;        // keys per LDS tile
+  static constexpr int VROW = TK + 8;
+  alignas(16) bf16_t k[TK * KROW];          // [key][dim]
+  alignas(16) bf16_t vt[D * VROW];          // [dim][key]
+};
+
+// mask of a 32-bit word that holds two bfloat16 of which the first `left` exist
+__device__ __forceinline__ uint32_t pair_mask(int left) { return left >= 2 ? 0xffffffffu : (left == 1 ? 0x0000ffffu : 0u); }
+
+// Global -> registers -> LDS, as TileRegs, with the page numbers of a tile read one tile before
+// its keys and values so that no load waits for another.  D % 32 == 0 makes the chunk counts whole.
+template <int KT>
+struct PfFetch {
+  static constexpr int PF_NT = 256 * KT, PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
+  static constexpr int KCH = D / 8;         // 16-byte chunks per key
+  static constexpr int VCH = PF_TK / 8;     // 16-byte chunks (8 keys) per head dimension
+  static constexpr int N = D / 32;          // chunks of K and of V^T per thread
+  u32x4 k[N], v[N];                         // plain vectors: a struct copy would go through memory
+  int page_k[N], page_v;
+
+  // chunk i of this thread: K chunk c = tid + PF_NT i is key c / KCH, part c % KCH; V^T chunk c is
+  // head dimension c / VCH, keys 8 (c % VCH) .. + 7, and c % VCH = tid % VCH for every i.
+  __device__ __forceinline__ void load_pages(const int* __restrict__ bt, int pshift, int num_pages, int tile_start,
+                                             int kv_end) {
+    const int last_key = kv_end - 1;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int pos = min(tile_start + ((int)threadIdx.x + PF_NT * i) / KCH, last_key);
+      page_k[i] = min(max(bt[pos >> pshift], 0), num_pages - 1);
+    }
+    const int pos = min(tile_start + 8 * ((int)threadIdx.x % VCH), last_key & ~7);
+    page_v = min(max(bt[pos >> pshift], 0), num_pages - 1);
+  }
+
+  // positions at or beyond kv_end read a clamped, valid address: their scores are masked and
+  // commit() makes their values zero
+  __device__ __forceinline__ void fetch(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int g,
+                                        int nkv, int pshift, int tile_start, int kv_end) {
+    const int P = 1 << pshift, last_key = kv_end - 1;
+    const char* kb = reinterpret_cast<const char*>(k_cache);
+    const char* vb = reinterpret_cast<const char*>(v_cache);
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int c = (int)threadIdx.x + PF_NT * i;
+      const int pos = min(tile_start + c / KCH, last_key);
+      const uint32_t off = ((((uint32_t)page_k[i] * nkv + g) << pshift) + (pos & (P - 1))) * (2 * D) + (c % KCH) * 16;
+      k[i] = *reinterpret_cast<const u32x4*>(kb + off);
+    }
+    const int pos = min(tile_start + 8 * ((int)threadIdx.x % VCH), last_key & ~7);
+    const uint32_t off0 = (((((uint32_t)page_v * nkv + g) * D + threadIdx.x / VCH) << pshift) + (pos & (P - 1))) * 2;
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      v[i] = *reinterpret_cast<const u32x4*>(vb + (off0 + ((uint32_t)((PF_NT / VCH) * i) << (pshift + 1))));
+  }
+
+  __device__ __forceinline__ void commit(PfTiles<KT>& t, int tile_start, int kv_end) const {
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int c = threadIdx.x + PF_NT * i;
+      *reinterpret_cast<u32x4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
+    }
+    const bool tail = tile_start + PF_TK > kv_end;           // the same for the whole workgroup
+    const int kc = threadIdx.x % VCH;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      u32x4 x = v[i];
+      if (tail) {   // values of keys at or beyond kv_end hold whatever the page held before
+        const int left = kv_end - (tile_start + kc * 8);       // keys of this chunk that exist
+        x[0] &= pair_mask(left);
+        x[1] &= pair_mask(left - 2);
+        x[2] &= pair_mask(left - 4);
+        x[3] &= pair_mask(left - 6);
+      }
+      *reinterpret_cast<u32x4*>(&t.vt[(threadIdx.x / VCH + (PF_NT / VCH) * i) * PF_VROW + kc * 8]) = x;
+    }
+  }
+};
+
+struct PfState {
+  float m, l;          // reference maximum of the column; this lane's part of the column's sum
+  f32x4p o[PF_DT];     // O^T tiles: rows = head dimension, column = query
+};
+
+// The 64 keys of one team (its first NPAIR pairs of 16-key blocks) against the wave's 16 query
+// columns, one softmax update: raw scores, p = 2^(s c - m c) with c = scale * log2(e); the reference
+// maximum may lag behind the running maximum by up to 8 in the exponent and the accumulators are
+// rescaled only when a column of the wave outgrows that (see attend_tile).
+// krow: row 8 (col / 4) + col % 4 of the team's keys in LDS, vrow: row col of V^T at the team's keys,
+// both at this lane quarter's 16 bytes; key_pos0: position of the team's first key.
+template <int NPAIR, bool MASK, int PF_VROW>
+__device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow, const bf16x8* q, PfState& st, float c,
+                                          int key_pos0, int q_pos) {
+  const int kq = (threadIdx.x & 63) >> 4;
+  f32x4p s[2 * NPAIR];
+#pragma unroll
+  for (int j = 0; j < 2 * NPAIR; j++) {
+    s[j] = f32x4p{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int step = 0; step < PF_KS; step++) {
+      const bf16x8 a = __builtin_bit_cast(
+          bf16x8, *reinterpret_cast<const u32x4*>(krow + (32 * (j / 2) + 4 * (j % 2)) * KROW + 32 * step));
+      s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[step], s[j], 0, 0, 0);
+    }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < 2 * NPAIR; j++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      if (MASK && key_pos0 + 32 * (j / 2) + 8 * kq + 4 * (j % 2) + r > q_pos) s[j][r] = -INFINITY;
+      mx = fmaxf(mx, s[j][r]);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(st.m, mx);
+  const bool outgrown = (m_new - st.m) * c > 8.0f;           // also true while the reference is -inf
+  if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {          // the same decision for the whole wave
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((st.m - m_use) * c);
+    st.l *= alpha;
+    st.m = m_new;
+#pragma unroll
+    for (int tt = 0; tt < PF_DT; tt++) st.o[tt] *= alpha;
+  }
+  const float mc = ((st.m == -INFINITY) ? 0.f : st.m) * c;
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2 * NPAIR; j++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[j][r], c, -mc));
+      s[j][r] = p;
+      sum += p;
+    }
+  st.l += sum;
+#pragma unroll
+  for (int m = 0; m < NPAIR; m++) {
+    const bf16x8 b = __builtin_bit_cast(
+        bf16x8, u32x4{pack2_bf16(s[2 * m][0], s[2 * m][1]), pack2_bf16(s[2 * m][2], s[2 * m][3]),
+                      pack2_bf16(s[2 * m + 1][0], s[2 * m + 1][1]), pack2_bf16(s[2 * m + 1][2], s[2 * m + 1][3])});
+#pragma unroll
+    for (int tt = 0; tt < PF_DT; tt++) {
+      const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(vrow + 16 * tt * PF_VROW + 32 * m));
+      st.o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, st.o[tt], 0, 0, 0);
+    }
+  }
+}
+
+// grid: x = query head, y = (sequence, 64-query tile), late (long) tiles first.  One team keeps three
+// workgroups on a compute unit, which serves many long, equal tiles best; two teams halve the key
+// loop of the longest tile, which decides when the tiles are few or unequal (a causal triangle).
+template <int KT>
+__global__ __launch_bounds__(256 * KT, KT == 1 ? 3 : 2) void prefill16_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
+    float scale) {
+  constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
+  __shared__ PfTiles<KT> tiles;
+  int b = 0, tile = (int)blockIdx.y, ntiles = 0;
+  for (; b < num_seqs; b++) {
+    ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
+    if (tile < ntiles) break;
+    tile -= ntiles;
+  }
+  if (b >= num_seqs) return;
+  tile = ntiles - 1 - tile;
+  const int head = blockIdx.x, g = head / (nq / nkv);
+  const int tok0 = cu_seqlens[b], new_len = cu_seqlens[b + 1] - tok0;
+  const int ctx = context_lens[b], prefix = ctx - new_len;
+  const int wave = (threadIdx.x >> 6) & 3, team = threadIdx.x >> 8;
+  const int lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
+  const int* bt = block_table + (size_t)b * max_pages;
+
+  const int q_idx = tile * PF_BM + wave * 16 + col;            // index among the sequence's new tokens
+  const bool q_ok = q_idx < new_len;
+  const int q_pos = prefix + q_idx;
+  bf16x8 qf[PF_KS];
+  {
+    const bf16_t* qrow = q + (size_t)(tok0 + (q_ok ? q_idx : 0)) * q_stride + (size_t)head * D + 8 * kq;
+#pragma unroll
+    for (int step = 0; step < PF_KS; step++) {
+      u32x4 v = u32x4{0, 0, 0, 0};
+      if (q_ok) v = *reinterpret_cast<const u32x4*>(qrow + 32 * step);
+      qf[step] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  const int wave_first_pos = prefix + tile * PF_BM + wave * 16;         // lowest query position of the wave
+  const int wave_last_pos = min(wave_first_pos + 15, ctx - 1);          // highest real one
+  const bool wave_active = tile * PF_BM + wave * 16 < new_len;
+  const int kv_end = min(ctx, prefix + min(new_len, (tile + 1) * PF_BM));  // keys beyond the tile's last query are never needed
+
+  const float c = scale * 1.4426950408889634f;                 // scores go through 2^x
+  const int pshift = 31 - __clz(P);                            // page sizes are powers of two
+  PfState st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int tt = 0; tt < PF_DT; tt++) st.o[tt] = f32x4p{0.f, 0.f, 0.f, 0.f};
+  const bf16_t* krow = &tiles.k[(64 * team + 8 * (col >> 2) + (col & 3)) * KROW + 8 * kq];
+  const bf16_t* vrow = &tiles.vt[col * PF_VROW + 64 * team + 8 * kq];
+  PfFetch<KT> regs;
+  regs.load_pages(bt, pshift, num_pages, 0, kv_end);
+  regs.fetch(k_cache, v_cache, g, nkv, pshift, 0, kv_end);
+  regs.load_pages(bt, pshift, num_pages, PF_TK, kv_end);
+  for (int tile_start = 0; tile_start < kv_end; tile_start += PF_TK) {
+    __syncthreads();                                            // everyone is done with the previous tile
+    regs.commit(tiles, tile_start, kv_end);
+    __syncthreads();
+    // the next tile's keys and values (clamped to the last key if there is no next tile) and the
+    // page numbers of the tile after it; no branch, so no wait is forced here
+    regs.fetch(k_cache, v_cache, g, nkv, pshift, tile_start + PF_TK, kv_end);
+    regs.load_pages(bt, pshift, num_pages, tile_start + 2 * PF_TK, kv_end);
+    const int key0 = tile_start + 64 * team;                    // this team's keys
+    if (!wave_active || key0 > wave_last_pos) continue;
+    if (key0 + 63 <= wave_first_pos) {
+      pf_attend<2, false, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
+    } else if (key0 + 32 <= wave_last_pos) {
+      pf_attend<2, true, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
+    } else {   // the second pair of 16-key blocks lies wholly beyond the causal frontier of this wave
+      pf_attend<1, true, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
+    }
+  }
+  if (KT > 1) {
+    // merge the teams through LDS (reusing the tile memory): lane-wise, the layouts agree
+    __syncthreads();
+    float* xo = reinterpret_cast<float*>(&tiles);              // [team - 1][wave][PF_DT * 4 + 2][64 lanes]
+    constexpr int PER_WAVE = (PF_DT * 4 + 2) * 64;
+    static_assert(sizeof(PfTiles<KT>) >= (size_t)(KT - 1) * 4 * PER_WAVE * sizeof(float) || KT == 1,
+                  "LDS tile memory too small for the merge");
+    if (team > 0) {
+      float* mine = xo + ((team - 1) * 4 + wave) * PER_WAVE + lane;
+#pragma unroll
+      for (int tt = 0; tt < PF_DT; tt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) mine[(4 * tt + r) * 64] = st.o[tt][r];
+      mine[(PF_DT * 4) * 64] = st.m;
+      mine[(PF_DT * 4 + 1) * 64] = st.l;
+    }
+    __syncthreads();
+    if (team > 0) return;
+    float M = st.m;
+#pragma unroll
+    for (int t = 1; t < KT; t++) M = fmaxf(M, xo[((t - 1) * 4 + wave) * PER_WAVE + (PF_DT * 4) * 64 + lane]);
+    const float m_use = (M == -INFINITY) ? 0.f : M;
+    const float a0 = __builtin_amdgcn_exp2f((st.m - m_use) * c);
+    st.l *= a0;
+#pragma unroll
+    for (int tt = 0; tt < PF_DT; tt++) st.o[tt] *= a0;
+#pragma unroll
+    for (int t = 1; t < KT; t++) {
+      const float* theirs = xo + ((t - 1) * 4 + wave) * PER_WAVE + lane;
+      const float at = __builtin_amdgcn_exp2f((theirs[(PF_DT * 4) * 64] - m_use) * c);
+      st.l += at * theirs[(PF_DT * 4 + 1) * 64];
+#pragma unroll
+      for (int tt = 0; tt < PF_DT; tt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) st.o[tt][r] += at * theirs[(4 * tt + r) * 64];
+    }
+  }
+  if (!q_ok) return;
+  float l = st.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  const float inv_l = 1.0f / l;
+  bf16_t* orow = out + ((size_t)(tok0 + q_idx) * nq + head) * D + 4 * kq;
+#pragma unroll
+  for (int tt = 0; tt < PF_DT; tt++) {
+    uint2 v;
+    v.x = pack2_bf16(st.o[tt][0] * inv_l, st.o[tt][1] * inv_l);
+    v.y = pack2_bf16(st.o[tt][2] * inv_l, st.o[tt][3] * inv_l);
+    *reinterpret_cast<uint2*>(orow + 16 * tt) = v;
+  }
+}
+#endif
+
 
 // ---------------------------------------------------------------------------
 // decode: one query token per sequence, the G heads of a kv group as the 32 columns
@@ -695,14 +999,34 @@ static int check_common(const char* who, int nq, int nkv, int d, int P, int max_
 
 extern "C" int pico_attn_head_dim() { return D; }
 
+// teams: 1 or 2 waves per SIMD share the key loop of a query tile (0: the default, 2 where the head
+// size allows it); a hint, any value gives the same result up to rounding
 extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int* block_table, int max_pages, const int* cu_seqlens,
                                  const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
-                                 int d, int P, int num_pages, float scale, hipStream_t stream) {
+                                 int d, int P, int num_pages, float scale, int teams, hipStream_t stream) {
   if (check_common("pico_attn_prefill", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
   PICO_REQUIRE(num_seqs > 0 && num_tokens >= num_seqs, "pico_attn_prefill: bad batch (%d sequences, %d tokens)", num_seqs, num_tokens);
   PICO_REQUIRE(nq <= 65535, "pico_attn_prefill: too many heads");
   PICO_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "pico_attn_prefill: misaligned tensors");
+#if PICO_HEAD_DIM % 32 == 0 && !defined(PICO_PF_WIDE)
+  // the 16-query kernel addresses the cache with 32-bit byte offsets
+  if ((uint64_t)num_pages * nkv * P * D * sizeof(bf16_t) < (1ull << 32)) {
+    const int max_tiles = num_tokens / PF_BM + num_seqs;  // >= sum over sequences of ceil(len / PF_BM)
+    PICO_REQUIRE(max_tiles <= 65535, "pico_attn_prefill: %d tokens are too many for one launch", num_tokens);
+    dim3 grid(nq, max_tiles);
+    if (teams == 1 || PF_KT_MAX == 1)
+      prefill16_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+                                                   (const bf16_t*)v_cache, block_table, max_pages, cu_seqlens,
+                                                   context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+    else
+      prefill16_kernel<PF_KT_MAX><<<grid, 256 * PF_KT_MAX, 0, stream>>>(
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
+          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+    PICO_LAUNCH_CHECK();
+    return 0;
+  }
+#endif
   const int max_tiles = num_tokens / BM + num_seqs;       // >= sum over sequences of ceil(len / BM)
   dim3 grid(max_tiles, nq);
   prefill_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,

@@ -31,9 +31,23 @@ class FastAttention:
         by_len = max(1, -(-max_context // 64))
         return max(1, min(by_fill, by_len, 64))
 
+    def prefill_teams(self, new_lens, context_lens) -> int:
+        """How many waves per SIMD share the key loop of a 64-query tile: two halve the longest
+        workgroup's loop, which decides while the work (in 64 x 64 tiles) would not keep 256
+        compute units busy for the time the longest tile takes; one leaves room for three
+        workgroups per unit, which serves many long tiles best."""
+        longest, total = 1, 0
+        for n, c in zip(new_lens, context_lens):
+            n, c = int(n), int(c)
+            tiles = -(-n // 64)
+            longest = max(longest, -(-c // 64))
+            total += tiles * max(1, (2 * c - n) // 128)      # mean key tiles of the portion's query tiles
+        return 1 if total * self.nq >= 256 * longest else 2
+
     def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
-                scale: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """q [T, >= nq*d] bfloat16 (row stride free); any mixture of portions; returns [T, nq*d]."""
+                scale: float, out: Optional[torch.Tensor] = None, teams: int = 0) -> torch.Tensor:
+        """q [T, >= nq*d] bfloat16 (row stride free); any mixture of portions; returns [T, nq*d].
+        teams: 0 lets the kernel choose, else the result of ``prefill_teams``."""
         nq, nkv, d = self.nq, self.nkv, self.d
         T = q.shape[0]
         pages, P = _check_cache(k_cache, v_cache, nkv, d)
@@ -44,7 +58,7 @@ class FastAttention:
         _check(self.lib, self.lib.pico_attn_prefill(
             _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens), _ptr(context_lens), num_seqs, T, _ptr(out), nq, nkv, d, P, pages, c_float(scale),
-            _stream()))
+            teams, _stream()))
         return out
 
     def decode(self, q: torch.Tensor, k_cache, v_cache, block_table, context_lens, num_seqs: int, scale: float,
@@ -86,7 +100,12 @@ class FastAttention:
         if ctx.all_decode and self.nq // self.nkv <= 32:
             return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, ctx.num_seqs, scale,
                                self.num_splits(ctx.num_seqs, ctx.max_context))
-        return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, ctx.num_seqs, scale)
+        teams = 0
+        if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
+            cu = ctx.host["cu_seqlens"]
+            teams = self.prefill_teams(cu[1:ctx.num_seqs + 1] - cu[:ctx.num_seqs], ctx.host["context_lens"][:ctx.num_seqs])
+        return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, ctx.num_seqs, scale,
+                            teams=teams)
 
 
 def choose(nq: int, nkv: int, head_dim: int, window: int) -> Optional[FastAttention]:
