@@ -24,31 +24,13 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
 
-template <int MT, int EPI, bool TAIL>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
-                                                          const bf16_t* __restrict__ W, int ldw,
-                                                          const float* __restrict__ bias, void* __restrict__ out,
-                                                          int ldo, long long slab_stride, int M, int N, int K,
-                                                          int k_per_wg) {
-  __shared__ float red[4][MT][16][64];   // [wave][column block][register][lane]
+// The stream of one output tile: sums over k_begin .. k_end of W[wrow0][k] X[m][k] for the 32 tile rows
+// (wrow0: this lane's row of W) and 32 MT tokens, reduced over the 4 waves' k slices into
+// red[wave][token block][register][lane]; the caller sums the 4 waves after the barrier at the end.
+template <int MT, bool TAIL>
+__device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ wrow0,
+                                              int m0, int M, int k_begin, int k_end, float (*red)[MT][16][64]) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
-  const int tile = blockIdx.x;
-  const int m0 = blockIdx.z * 32 * MT;
-  // the row of W that tile row `col` stands for
-  int wrow;
-  bool w_ok;
-  if (EPI == EPI_SWIGLU) {
-    const int I = N / 2, gi = tile * 16 + (col & 15);
-    w_ok = gi < I;
-    wrow = (col < 16 ? 0 : I) + gi;
-  } else {
-    wrow = tile * 32 + col;
-    w_ok = wrow < N;
-  }
-  // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
-  // Only a k tail must read as zero, because it is summed into outputs that are stored.
-  const int n_rows = N;
-  const bf16_t* wrow0 = W + (size_t)min(wrow, n_rows - 1) * ldw;
   const bf16_t* xrow0[MT];
 #pragma unroll
   for (int t = 0; t < MT; t++) xrow0[t] = X + (size_t)min(m0 + 32 * t + col, M - 1) * ldx;
@@ -57,8 +39,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   for (int t = 0; t < MT; t++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
-
-  const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
   struct Stage {
     uint4 w[4], x[MT][4];
   };
@@ -134,6 +114,34 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
     for (int r = 0; r < 16; r++) red[wave][t][r][lane] = acc[t][r];
   __syncthreads();
+}
+
+template <int MT, int EPI, bool TAIL>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
+                                                          const bf16_t* __restrict__ W, int ldw,
+                                                          const float* __restrict__ bias, void* __restrict__ out,
+                                                          int ldo, long long slab_stride, int M, int N, int K,
+                                                          int k_per_wg) {
+  __shared__ float red[4][MT][16][64];   // [wave][column block][register][lane]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int tile = blockIdx.x;
+  const int m0 = blockIdx.z * 32 * MT;
+  // the row of W that tile row `col` stands for
+  int wrow;
+  bool w_ok;
+  if (EPI == EPI_SWIGLU) {
+    const int I = N / 2, gi = tile * 16 + (col & 15);
+    w_ok = gi < I;
+    wrow = (col < 16 ? 0 : I) + gi;
+  } else {
+    wrow = tile * 32 + col;
+    w_ok = wrow < N;
+  }
+  // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
+  // Only a k tail must read as zero, because it is summed into outputs that are stored.
+  const bf16_t* wrow0 = W + (size_t)min(wrow, N - 1) * ldw;
+  const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
+  skinny_stream<MT, TAIL>(X, ldx, wrow0, m0, M, k_begin, k_end, red);
 
   // thread (a = wave, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col`: sum of the 4 waves
   const int a = wave;
@@ -214,6 +222,121 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   else if (epilogue == EPI_F32) { if (mt == 1) LAUNCH(1, EPI_F32); else LAUNCH(2, EPI_F32); }
   else { if (mt == 1) LAUNCH(1, EPI_SWIGLU); else LAUNCH(2, EPI_SWIGLU); }
 #undef LAUNCH2
+#undef LAUNCH
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The q/k/v projection of a decode step with everything that follows it before attention:
+// bias, rotate-half position encoding of q and k (pico_vllm/kernels/fused_rope_kvcache_store.py:51-101
+// fuses the rotation with the store; here both ride on the projection) and the store of k and v
+// into the paged cache.  W = [q heads | k heads | v heads] x d rows.  A tile of a q or k head
+// holds 16 rows j .. j + 15 of the head and the 16 rows j + d/2 .. they are rotated with, so a pair
+// is local to a lane as gate and up are in the SwiGLU epilogue; a tile of a v head holds 32
+// consecutive rows.  Needs rot == d and d % 32 == 0.
+//   q_out [M, ldq] bfloat16 gets the rotated q heads at columns head * d + dim;
+//   K pages [page][kv head][slot][d], V pages [page][kv head][d][slot], P = 1 << pshift slots;
+//   slots[m] = page * P + slot of token m, negative: store nothing.
+// ---------------------------------------------------------------------------
+template <int MT, bool TAIL>
+__global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
+    const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
+    bf16_t* __restrict__ q_out, int ldq, const int* __restrict__ positions, const int* __restrict__ slots,
+    const float* __restrict__ inv_freq, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
+    int nq, int nkv, int d, int pshift, int num_pages) {
+  __shared__ float red[4][MT][16][64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int tiles_per_head = d >> 5, half = d >> 1;
+  const int head = blockIdx.x / tiles_per_head, tp = blockIdx.x % tiles_per_head;
+  const int m0 = blockIdx.z * 32 * MT;
+  const bool rotated = head < nq + nkv;
+  const int wrow = head * d + (rotated ? 16 * tp + (col & 15) + (col < 16 ? 0 : half) : 32 * tp + col);
+  skinny_stream<MT, TAIL>(X, ldx, W + (size_t)wrow * ldw, m0, M, 0, K, red);
+
+  const int a = wave;
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const int m = m0 + 32 * t + col;
+    if (m >= M) continue;
+    if (rotated) {
+      if (a >= 2) continue;
+      const int j0 = 16 * tp + 8 * a + 4 * h;        // this thread's four pairs (j, j + d/2)
+      const float pos = (float)positions[m];
+      float y1[4], y2[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        float x1 = 0.f, x2 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+          x1 += red[w][t][4 * a + b][lane];
+          x2 += red[w][t][4 * (a + 2) + b][lane];
+        }
+        if (bias) {
+          x1 += bias[head * d + j0 + b];
+          x2 += bias[head * d + j0 + b + half];
+        }
+        // rounded as the projection's output is when it goes through memory, so that a token gets
+        // the same key whether it came in a small step (here) or in a large one
+        x1 = bf16_to_f32(f32_to_bf16(x1));
+        x2 = bf16_to_f32(f32_to_bf16(x2));
+        const float ang = pos * inv_freq[j0 + b];
+        const float c = cosf(ang), s = sinf(ang);
+        y1[b] = x1 * c - x2 * s;
+        y2[b] = x2 * c + x1 * s;
+      }
+      bf16_t* o;
+      if (head < nq) {
+        o = q_out + (size_t)m * ldq + head * d + j0;
+      } else {
+        const int slot = slots[m];
+        const int page = slot >> pshift;
+        if (slot < 0 || page >= num_pages) continue;   // padding row; the host has checked the rest
+        o = k_cache + ((((size_t)page * nkv + (head - nq)) << pshift) + (slot & ((1 << pshift) - 1))) * d + j0;
+      }
+      *reinterpret_cast<uint2*>(o) = make_uint2(pack2_bf16(y1[0], y1[1]), pack2_bf16(y1[2], y1[3]));
+      *reinterpret_cast<uint2*>(o + half) = make_uint2(pack2_bf16(y2[0], y2[1]), pack2_bf16(y2[2], y2[3]));
+    } else {
+      const int slot = slots[m];
+      const int page = slot >> pshift;
+      if (slot < 0 || page >= num_pages) continue;
+      const int n0 = 32 * tp + 8 * a + 4 * h;          // this thread's four head dimensions
+      bf16_t* o = v_cache + ((((size_t)page * nkv + (head - nq - nkv)) * d + n0) << pshift) + (slot & ((1 << pshift) - 1));
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) v += red[w][t][4 * a + b][lane];
+        if (bias) v += bias[head * d + n0 + b];
+        o[(size_t)b << pshift] = f32_to_bf16(v);
+      }
+    }
+  }
+}
+
+extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int ldw, const float* bias, void* q_out,
+                                     int ldq, const int* positions, const int* slots, const float* inv_freq,
+                                     void* k_cache, void* v_cache, int M, int K, int nq, int nkv, int d, int P,
+                                     int num_pages, hipStream_t stream) {
+  PICO_REQUIRE(M > 0 && K > 0 && nq > 0 && nkv > 0 && num_pages > 0, "pico_gemm_skinny_rope: bad sizes");
+  PICO_REQUIRE(d >= 32 && d % 32 == 0, "pico_gemm_skinny_rope: head size %d is not a multiple of 32", d);
+  PICO_REQUIRE(P >= 1 && (P & (P - 1)) == 0, "pico_gemm_skinny_rope: page size %d is not a power of two", P);
+  PICO_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
+               "pico_gemm_skinny_rope: K and the row strides must be multiples of 8 (K=%d ldx=%d ldw=%d)", K, ldx, ldw);
+  PICO_REQUIRE((uintptr_t)X % 16 == 0 && (uintptr_t)W % 16 == 0, "pico_gemm_skinny_rope: operands must be 16-byte aligned");
+  PICO_REQUIRE(ldq >= nq * d && ldq % 4 == 0 && (uintptr_t)q_out % 8 == 0 && (uintptr_t)k_cache % 8 == 0,
+               "pico_gemm_skinny_rope: q and the cache must be 8-byte aligned, the q row stride a multiple of 4");
+  const int mt = M <= 32 ? 1 : 2;
+  int pshift = 0;
+  while ((1 << pshift) < P) pshift++;
+  dim3 grid((nq + 2 * nkv) * (d / 32), 1, (M + 32 * mt - 1) / (32 * mt));
+  PICO_REQUIRE(grid.z <= 65535, "pico_gemm_skinny_rope: too many rows");
+  const bool tail = K % 64 != 0;
+#define LAUNCH(MT, TAIL) \
+  gemm_skinny_rope_kernel<MT, TAIL><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
+      (bf16_t*)q_out, ldq, positions, slots, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
+  if (mt == 1) { if (tail) LAUNCH(1, true); else LAUNCH(1, false); }
+  else { if (tail) LAUNCH(2, true); else LAUNCH(2, false); }
 #undef LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;

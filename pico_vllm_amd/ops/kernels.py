@@ -290,6 +290,37 @@ def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tenso
                                        _ptr(k_cache), _ptr(v_cache), T, nq, nkv, d, rotary_dim, P, pages, _stream()))
 
 
+def gemm_skinny_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                     slots: torch.Tensor, inv_freq: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     nq: int, nkv: int, d: int) -> torch.Tensor:
+    """The q/k/v projection of up to 64 tokens with bias, rotate-half encoding of q and k (over the
+    whole head size) and the store of k and v at ``slots`` in one kernel; returns the encoded queries
+    [M, nq * d].  w: [(nq + 2 nkv) * d, K] bfloat16, rows [q heads | k heads | v heads]."""
+    _gpu(a, w, bias, positions, slots, inv_freq, k_cache, v_cache)
+    M, K = a.shape
+    if w.shape != ((nq + 2 * nkv) * d, K):
+        raise KernelError(f"gemm_skinny_rope: weight {tuple(w.shape)} is not [{(nq + 2 * nkv) * d}, {K}]")
+    if not skinny_ok(a, w):
+        raise KernelError("gemm_skinny_rope: operands must be bfloat16, at most 64 rows, K a multiple of 8, rows 16-byte aligned")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (w.shape[0],) or not bias.is_contiguous()):
+        raise KernelError("gemm_skinny_rope: bias must be contiguous float32 [N]")
+    pages, P = _check_cache(k_cache, v_cache, nkv, d)
+    if k_cache.dtype != torch.bfloat16:
+        raise KernelError("gemm_skinny_rope: the cache must be bfloat16")
+    if d % 32 or P & (P - 1):
+        raise KernelError("gemm_skinny_rope: head size must be a multiple of 32 and the page size a power of two")
+    _i32(positions, "positions", M)
+    _i32(slots, "slots", M)
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != d // 2 or not inv_freq.is_contiguous():
+        raise KernelError("gemm_skinny_rope: inv_freq must be float32 of head size / 2 entries")
+    q = torch.empty(M, nq * d, dtype=torch.bfloat16, device=a.device)
+    lib = library.core()
+    _check(lib, lib.pico_gemm_skinny_rope(_ptr(a), a.stride(0) if M > 1 else K, _ptr(w), w.stride(0), _ptr(bias), _ptr(q),
+                                          nq * d, _ptr(positions), _ptr(slots), _ptr(inv_freq), _ptr(k_cache),
+                                          _ptr(v_cache), M, K, nq, nkv, d, P, pages, _stream()))
+    return q
+
+
 def paged_attention_ref(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                         positions: torch.Tensor, token_seq: torch.Tensor, nq: int, nkv: int, d: int,
                         scale: float, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -69,8 +69,8 @@ class GQAAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         nq, nkv, d = self.nq, self.nkv, self.d
         bt = ctx.block_tables[cache.group]
-        qkv = self.qkv(x)                                         # [T, (nq + 2 nkv) d]
-        self.position.rotate_and_store(qkv, ctx, cache, bt, nq, nkv, d)
+        # [T, >= nq d]: the encoded queries first; keys and values are in the cache after this
+        qkv = self.position.project_rotate_store(x, self.qkv, ctx, cache, bt, nq, nkv, d)
         if self.fast is not None and cache.k.dtype == torch.bfloat16:
             a = self.fast(qkv, cache, bt, ctx, self.scale)
         else:

@@ -75,6 +75,14 @@ class PositionEncoding(Part):
         """Encode positions into q (in place) and k, and write k, v into the pages of ``kv``."""
         raise NotImplementedError
 
+    def project_rotate_store(self, x: torch.Tensor, linear, ctx: StepContext, kv, block_table: torch.Tensor,
+                             nq: int, nkv: int, d: int) -> torch.Tensor:
+        """qkv = linear(x), then ``rotate_and_store``; returns a tensor whose first nq * d columns are
+        the encoded queries.  An encoding may override this to fuse the three steps."""
+        qkv = linear(x)
+        self.rotate_and_store(qkv, ctx, kv, block_table, nq, nkv, d)
+        return qkv
+
 
 class Mixer(Part):
     def cache_spec(self) -> CacheSpec:

@@ -31,6 +31,14 @@ class RotaryHalf(PositionEncoding):
         kernels.rope_kv_store(qkv, ctx.positions, ctx.slot_mapping[kv.group], self.inv_freq,
                               kv.k, kv.v, nq, nkv, d, self.rotary_dim)
 
+    def project_rotate_store(self, x, linear, ctx, kv, block_table, nq, nkv, d) -> torch.Tensor:
+        # few tokens in bfloat16: projection, bias, rotation and cache store are one weight-streaming kernel
+        if (self.rotary_dim == d and d % 32 == 0 and kv.k.dtype == torch.bfloat16
+                and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0 and kernels.skinny_ok(x, linear.weight)):
+            return kernels.gemm_skinny_rope(x, linear.weight, linear.bias_f32, ctx.positions, ctx.slot_mapping[kv.group],
+                                            self.inv_freq, kv.k, kv.v, nq, nkv, d)
+        return super().project_rotate_store(x, linear, ctx, kv, block_table, nq, nkv, d)
+
 
 @register_part("position", "none")
 class NoPosition(PositionEncoding):

@@ -389,6 +389,45 @@ def test_gemm_skinny_epilogues(K, M, N, K_):
     assert torch.equal(one.cpu()[0], full.cpu()[M // 2])
 
 
+@pytest.mark.parametrize("M,nq,nkv,d,H,Pg,bias", [(1, 12, 2, 128, 1536, 16, True), (8, 12, 2, 128, 1536, 16, True),
+                                                  (64, 6, 3, 32, 192, 8, True), (37, 3, 1, 64, 136, 32, False),
+                                                  (5, 2, 2, 96, 264, 16, True)])
+def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias):
+    # projection + bias + rotate-half + store in one kernel against the plain steps one after the other
+    theta = 1e6
+    g = torch.Generator().manual_seed(M + d)
+    x = torch.randn(M, H, generator=g).bfloat16()
+    N = (nq + 2 * nkv) * d
+    w = (torch.randn(N, H, generator=g) / math.sqrt(H)).bfloat16()
+    b = torch.randn(N, generator=g) if bias else None
+    pos = torch.randint(0, 5000, (M,), generator=g, dtype=torch.int32)
+    num_pages = M + 4
+    pages = torch.randperm(num_pages, generator=g)[:M]
+    offs = torch.randint(0, Pg, (M,), generator=g)
+    slots = (pages * Pg + offs).to(torch.int32)
+    if M > 2:
+        slots[M // 2] = -1                                  # a padding row stores nothing
+    kc = torch.full((num_pages, nkv, Pg, d), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((num_pages, nkv, d, Pg), 7.0, dtype=torch.bfloat16, device=DEV)
+    inv = (1.0 / (theta ** (torch.arange(0, d, 2).float() / d))).to(DEV)
+    q_out = K.gemm_skinny_rope(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), pos.to(DEV), slots.to(DEV), inv,
+                               kc, vc, nq, nkv, d)
+    qkv = (x.double() @ w.double().T + (0 if b is None else b.double())).float()
+    q, k, v = P.split_qkv(qkv, nq, nkv, d)
+    cos, sin = P.rope_tables(pos, d, theta)
+    qr, kr = P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin)
+    close(q_out.reshape(M, nq, d), qr, torch.bfloat16, scale=4)
+    want_k = torch.full((num_pages, nkv, Pg, d), 7.0)
+    want_v = torch.full((num_pages, nkv, d, Pg), 7.0)
+    for t in range(M):
+        if int(slots[t]) < 0:
+            continue
+        want_k[int(pages[t]), :, int(offs[t]), :] = kr[t]
+        want_v[int(pages[t]), :, :, int(offs[t])] = v[t]
+    close(kc, want_k, torch.bfloat16, scale=4)             # also: every slot that no token owns still holds 7
+    close(vc, want_v, torch.bfloat16, scale=4)
+
+
 def test_gemm_skinny_refuses_misaligned_operands(K):
     a = torch.randn(4, 172).bfloat16().to(DEV)          # K = 172 is no multiple of 8
     w = torch.randn(64, 172).bfloat16().to(DEV)
