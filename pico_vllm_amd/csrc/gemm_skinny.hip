@@ -11,6 +11,14 @@
 //   * when the matrix is too small to fill the chip (N small), the k range is also split over
 //     workgroups (grid y); each writes a float32 partial slab that the consumer sums.
 //
+//   * few rows (one block of up to 32 tokens, K % 64 == 0): the slices do not go through registers.
+//     Lane (i, h) reading its own row of W makes every load instruction touch 32 cache lines, and the
+//     address unit of the compute unit, not HBM, then bounds the stream.  Instead each slice is
+//     copied global -> LDS by `global_load_lds_dwordx4` in the order of memory (8 lanes share one
+//     128-byte line, 8 lines per instruction) and the matrix-core operands are read back from LDS;
+//     the copy is asynchronous, so DEPTH slices per wave are in flight without holding registers.
+//     Activations take the same way, only the 8-row groups that hold real tokens.
+//
 // Epilogues on the float32 sums: bias; SwiGLU (the tile holds 16 gate rows and the 16 matching up
 // rows, so silu(gate) * up is local to a lane; pico_vllm/kernels/swiglu.py:36-41); float32 or
 // bfloat16 store.  Layout of the 32x32 result tile: lane l holds output column (token) l % 32 and
@@ -19,6 +27,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define EPI_BF16 0     // out bf16 [M, N]
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
@@ -116,32 +125,150 @@ __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int 
   __syncthreads();
 }
 
-template <int MT, int EPI, bool TAIL>
+// ---- the stream through LDS ----------------------------------------------------------------
+// One slice of one wave in LDS: 4 groups of W (8 tile rows x 128 bytes each) and NX groups of X
+// (8 tokens x 128 bytes).  A group is what one load instruction brings: lane l = (rho, pos) =
+// (l / 8, l % 8) writes bytes 16 l .. 16 l + 15 of the group, and fetches chunk pos ^ rho of row
+// rho of the group, so that the rows of a group lie in LDS with their 16-byte chunks xor-swizzled by
+// the row and the operand reads below (32 rows, one chunk each) spread over the banks; groups are
+// 16 bytes further apart than their size for the same reason.
+#define GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+constexpr int SK_GROUP = 1024 + 16;
+template <int NX> constexpr int sk_stage_bytes() { return (4 + NX) * SK_GROUP; }
+template <int NX> constexpr int sk_depth() { return NX == 4 ? 2 : 3; }
+// s_waitcnt for "at most n vector memory operations outstanding", nothing else waited for
+constexpr int sk_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+template <int MT, int NX>
+constexpr int sk_smem_bytes() {
+  constexpr int red = 4 * MT * 16 * 64 * 4;
+  if (NX == 0) return red;
+  constexpr int stages = sk_depth<NX>() * 4 * sk_stage_bytes<NX>();
+  return stages > red ? stages : red;
+}
+
+// Tile rows 0..15 are rows row_a .. of W, tile rows 16..31 rows row_b .. (clamped to n_rows - 1);
+// tokens m0 .. m0 + 8 NX - 1 (clamped to M - 1).  The sums of the 4 waves end up in
+// red[wave][0][register][lane] at the start of smem, as skinny_stream leaves them.
+template <int NX>
+__device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W,
+                                                  int ldw, int row_a, int row_b, int n_rows, int m0, int M, int k_begin,
+                                                  int k_end, char* smem) {
+  constexpr int DEPTH = sk_depth<NX>(), STAGE = sk_stage_bytes<NX>(), LOADS = 4 + NX;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int col = lane & 31, h = lane >> 5, rho = lane >> 3, pos = lane & 7;
+  // sources of this lane's 16 bytes in each group, at k = 0
+  const bf16_t* wsrc[4];
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    const int row = min((g < 2 ? row_a + 8 * g : row_b + 8 * (g - 2)) + rho, n_rows - 1);
+    wsrc[g] = W + (size_t)row * ldw + 8 * (pos ^ rho);
+  }
+  const bf16_t* xsrc[NX];
+#pragma unroll
+  for (int g = 0; g < NX; g++) xsrc[g] = X + (size_t)min(m0 + 8 * g + rho, M - 1) * ldx + 8 * (pos ^ rho);
+  // where lane (col, h) finds chunk 4 h + s of tile row (or token) col, relative to the slice
+  int rd[4];
+#pragma unroll
+  for (int s = 0; s < 4; s++) rd[s] = (col >> 3) * SK_GROUP + (col & 7) * 128 + (((4 * h + s) ^ (col & 7)) << 4);
+  char* mine = smem + wave * STAGE;            // stage d of this wave: mine + d * 4 * STAGE
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+  const int first = k_begin + 64 * wave;       // this wave's slices start at k_begin + 64 (wave + 4 i)
+  if (first < k_end) {
+    const int n_slices = (k_end - first + 255) / 256;
+    const int rounds = (n_slices + DEPTH - 1) / DEPTH;
+    const int last = first + (n_slices - 1) * 256;
+    auto issue = [&](int d, int slice) {       // beyond the wave's last slice the last one is copied again
+      const int k0 = min(first + 256 * slice, last);
+      char* dst = mine + d * 4 * STAGE;
+#pragma unroll
+      for (int g = 0; g < 4; g++) __builtin_amdgcn_global_load_lds(GPTR(wsrc[g] + k0), LPTR(dst + g * SK_GROUP), 16, 0, 0);
+#pragma unroll
+      for (int g = 0; g < NX; g++)
+        __builtin_amdgcn_global_load_lds(GPTR(xsrc[g] + k0), LPTR(dst + (4 + g) * SK_GROUP), 16, 0, 0);
+    };
+    auto multiply = [&](int d) {
+      const char* src = mine + d * 4 * STAGE;
+      u32x4 a[4], b[4];
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        a[s] = *reinterpret_cast<const u32x4*>(src + rd[s]);
+        b[s] = *reinterpret_cast<const u32x4*>(src + 4 * SK_GROUP + rd[s]);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; s++)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[s]), __builtin_bit_cast(bf16x8, b[s]),
+                                                      acc, 0, 0, 0);
+    };
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) issue(d, d);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int r = 0; r + 1 < rounds; r++) {     // every slice of these rounds exists
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++) {
+        // DEPTH stages are in flight, stage d is the oldest: it has landed when at most the loads of
+        // the DEPTH - 1 younger stages are outstanding.  The compiler does not order LDS reads after
+        // these copies by itself.
+        __builtin_amdgcn_s_waitcnt(sk_vmcnt((DEPTH - 1) * LOADS));
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(d);                            // its operand reads are complete when the products have issued
+        __builtin_amdgcn_sched_barrier(0);
+        issue(d, (r + 1) * DEPTH + d);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(sk_vmcnt(0));
+    __builtin_amdgcn_sched_barrier(0);
+    const int left = n_slices - (rounds - 1) * DEPTH;            // 1..DEPTH slices in the last round
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+      if (d < left) multiply(d);
+  }
+  __syncthreads();                             // every wave is done with its stages: the sums take their place
+  float(*red)[1][16][64] = reinterpret_cast<float(*)[1][16][64]>(smem);
+#pragma unroll
+  for (int r = 0; r < 16; r++) red[wave][0][r][lane] = acc[r];
+  __syncthreads();
+}
+
+// The 32 tile rows' sums for this workgroup's tokens, through LDS (NX > 0) or registers (NX == 0).
+template <int MT, bool TAIL, int NX>
+__device__ __forceinline__ float (*skinny_tile(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
+                                               int row_a, int row_b, int n_rows, int m0, int M, int k_begin, int k_end,
+                                               char* smem))[MT][16][64] {
+  float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
+  if constexpr (NX > 0) {
+    static_assert(MT == 1 && !TAIL, "the stream through LDS takes one block of tokens and whole slices");
+    skinny_stream_lds<NX>(X, ldx, W, ldw, row_a, row_b, n_rows, m0, M, k_begin, k_end, smem);
+  } else {
+    const int col = threadIdx.x & 31;
+    const int wrow = col < 16 ? row_a + col : row_b + col - 16;
+    // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
+    // Only a k tail must read as zero, because it is summed into outputs that are stored.
+    skinny_stream<MT, TAIL>(X, ldx, W + (size_t)min(wrow, n_rows - 1) * ldw, m0, M, k_begin, k_end, red);
+  }
+  return red;
+}
+
+template <int MT, int EPI, bool TAIL, int NX>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias, void* __restrict__ out,
                                                           int ldo, long long slab_stride, int M, int N, int K,
                                                           int k_per_wg) {
-  __shared__ float red[4][MT][16][64];   // [wave][column block][register][lane]
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX>()];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int tile = blockIdx.x;
   const int m0 = blockIdx.z * 32 * MT;
-  // the row of W that tile row `col` stands for
-  int wrow;
-  bool w_ok;
-  if (EPI == EPI_SWIGLU) {
-    const int I = N / 2, gi = tile * 16 + (col & 15);
-    w_ok = gi < I;
-    wrow = (col < 16 ? 0 : I) + gi;
-  } else {
-    wrow = tile * 32 + col;
-    w_ok = wrow < N;
-  }
-  // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
-  // Only a k tail must read as zero, because it is summed into outputs that are stored.
-  const bf16_t* wrow0 = W + (size_t)min(wrow, N - 1) * ldw;
+  // the rows of W that tile rows 0..15 and 16..31 stand for
+  const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
+  const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  skinny_stream<MT, TAIL>(X, ldx, wrow0, m0, M, k_begin, k_end, red);
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
 
   // thread (a = wave, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col`: sum of the 4 waves
   const int a = wave;
@@ -215,13 +342,23 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   PICO_REQUIRE(grid.z <= 65535 && grid.y <= 65535, "pico_gemm_skinny: too many blocks");
   const float* b0 = bias;
   const bool tail = K % 64 != 0;
-#define LAUNCH2(MT, EPI, TAIL) \
-  gemm_skinny_kernel<MT, EPI, TAIL><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
-#define LAUNCH(MT, EPI) do { if (tail) LAUNCH2(MT, EPI, true); else LAUNCH2(MT, EPI, false); } while (0)
-  if (epilogue == EPI_BF16) { if (mt == 1) LAUNCH(1, EPI_BF16); else LAUNCH(2, EPI_BF16); }
-  else if (epilogue == EPI_F32) { if (mt == 1) LAUNCH(1, EPI_F32); else LAUNCH(2, EPI_F32); }
-  else { if (mt == 1) LAUNCH(1, EPI_SWIGLU); else LAUNCH(2, EPI_SWIGLU); }
-#undef LAUNCH2
+  // few rows and whole slices: the stream through LDS, with as many 8-token groups as hold tokens
+  const int nx = (mt == 1 && !tail) ? (M <= 8 ? 1 : M <= 16 ? 2 : 4) : 0;
+#define LAUNCH3(MT, EPI, TAIL, NX) \
+  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+#define LAUNCH(EPI)                                               \
+  do {                                                            \
+    if (nx == 1) LAUNCH3(1, EPI, false, 1);                       \
+    else if (nx == 2) LAUNCH3(1, EPI, false, 2);                  \
+    else if (nx == 4) LAUNCH3(1, EPI, false, 4);                  \
+    else if (mt == 1) LAUNCH3(1, EPI, true, 0);                   \
+    else if (tail) LAUNCH3(2, EPI, true, 0);                      \
+    else LAUNCH3(2, EPI, false, 0);                               \
+  } while (0)
+  if (epilogue == EPI_BF16) LAUNCH(EPI_BF16);
+  else if (epilogue == EPI_F32) LAUNCH(EPI_F32);
+  else LAUNCH(EPI_SWIGLU);
+#undef LAUNCH3
 #undef LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;
@@ -239,20 +376,21 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
 //   K pages [page][kv head][slot][d], V pages [page][kv head][d][slot], P = 1 << pshift slots;
 //   slots[m] = page * P + slot of token m, negative: store nothing.
 // ---------------------------------------------------------------------------
-template <int MT, bool TAIL>
+template <int MT, bool TAIL, int NX>
 __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
     const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
     bf16_t* __restrict__ q_out, int ldq, const int* __restrict__ positions, const int* __restrict__ slots,
     const float* __restrict__ inv_freq, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
     int nq, int nkv, int d, int pshift, int num_pages) {
-  __shared__ float red[4][MT][16][64];
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX>()];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int tiles_per_head = d >> 5, half = d >> 1;
   const int head = blockIdx.x / tiles_per_head, tp = blockIdx.x % tiles_per_head;
   const int m0 = blockIdx.z * 32 * MT;
   const bool rotated = head < nq + nkv;
-  const int wrow = head * d + (rotated ? 16 * tp + (col & 15) + (col < 16 ? 0 : half) : 32 * tp + col);
-  skinny_stream<MT, TAIL>(X, ldx, W + (size_t)wrow * ldw, m0, M, 0, K, red);
+  const int row_a = head * d + (rotated ? 16 * tp : 32 * tp);
+  const int row_b = rotated ? row_a + half : row_a + 16;
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX>(X, ldx, W, ldw, row_a, row_b, (nq + 2 * nkv) * d, m0, M, 0, K, smem);
 
   const int a = wave;
 #pragma unroll
@@ -332,11 +470,16 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   dim3 grid((nq + 2 * nkv) * (d / 32), 1, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535, "pico_gemm_skinny_rope: too many rows");
   const bool tail = K % 64 != 0;
-#define LAUNCH(MT, TAIL) \
-  gemm_skinny_rope_kernel<MT, TAIL><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
+  const int nx = (mt == 1 && !tail) ? (M <= 8 ? 1 : M <= 16 ? 2 : 4) : 0;
+#define LAUNCH(MT, TAIL, NX) \
+  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
       (bf16_t*)q_out, ldq, positions, slots, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
-  if (mt == 1) { if (tail) LAUNCH(1, true); else LAUNCH(1, false); }
-  else { if (tail) LAUNCH(2, true); else LAUNCH(2, false); }
+  if (nx == 1) LAUNCH(1, false, 1);
+  else if (nx == 2) LAUNCH(1, false, 2);
+  else if (nx == 4) LAUNCH(1, false, 4);
+  else if (mt == 1) LAUNCH(1, true, 0);
+  else if (tail) LAUNCH(2, true, 0);
+  else LAUNCH(2, false, 0);
 #undef LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;

@@ -350,7 +350,8 @@ def test_fast_kernels_refuse_what_they_cannot_do(K):
 
 # ---- weight-streaming GEMM --------------------------------------------------------------------
 @pytest.mark.parametrize("M,N,K_", [(1, 2048, 1536), (8, 1536, 1536), (64, 1536, 8960), (33, 301, 136), (5, 384, 192),
-                                   (2, 64, 320), (17, 1000, 264)])
+                                   (2, 64, 320), (17, 1000, 264), (12, 1536, 1536), (16, 90, 64), (24, 512, 1024),
+                                   (32, 301, 256), (9, 1000, 8960)])
 def test_gemm_skinny_epilogues(K, M, N, K_):
     g = torch.Generator().manual_seed(M * N)
     a = torch.randn(M, K_, generator=g).bfloat16()
@@ -391,7 +392,8 @@ def test_gemm_skinny_epilogues(K, M, N, K_):
 
 @pytest.mark.parametrize("M,nq,nkv,d,H,Pg,bias", [(1, 12, 2, 128, 1536, 16, True), (8, 12, 2, 128, 1536, 16, True),
                                                   (64, 6, 3, 32, 192, 8, True), (37, 3, 1, 64, 136, 32, False),
-                                                  (5, 2, 2, 96, 264, 16, True)])
+                                                  (5, 2, 2, 96, 264, 16, True), (13, 4, 2, 64, 320, 16, True),
+                                                  (29, 2, 1, 128, 128, 8, False)])
 def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias):
     # projection + bias + rotate-half + store in one kernel against the plain steps one after the other
     theta = 1e6
