@@ -2,22 +2,24 @@
 // out = X W^T with X [M <= 64 per launch block, K] and W [N, K] bfloat16, K contiguous in both.
 // The cost is reading W once from HBM, so the kernel is built around that stream:
 //
-//   * a workgroup owns 32 rows of W (one output tile) and one range of k; its 4 waves take
+//   * a workgroup owns 32 rows of W (one output tile) and one range of k; its waves take
 //     interleaved 64-wide k slices of that range and are summed through LDS in a fixed order,
 //     so the split over k needs no atomics and results are reproducible;
-//   * inside a 64-wide slice lane (i, h) reads the 64 contiguous bytes W[row i][k0 + 32 h ..],
-//     four 16-byte loads that feed four v_mfma_f32_32x32x16_bf16 steps; the activations are read
-//     with the same k order (the contraction does not care about the order of k);
+//   * a slice of a wave (32 rows x 128 bytes of W, and of the activations as many 8-token groups
+//     as hold tokens) does not go through registers.  A lane that reads its own row of W makes
+//     every load instruction touch 32 cache lines, and the address unit of the compute unit, not
+//     HBM, then bounds the stream (measured: 16 us against 13 us for the 55 MB gate/up matrix with
+//     8 tokens, 34 us against 22 us with 64).  Instead `global_load_lds_dwordx4` copies the slice
+//     global -> LDS in the order of memory (8 lanes share one 128-byte line, 8 lines per
+//     instruction) and the v_mfma_f32_32x32x16_bf16 operands are read back from LDS (lane (i, h)
+//     takes chunks 4 h + 0..3 of row i, W and activations alike: the contraction does not care
+//     about the order of k).  The copy is asynchronous: DEPTH slices per wave are in flight
+//     without holding registers;
+//   * up to 32 tokens: 4 waves per workgroup; 33 to 64 tokens: 2 waves, each with both blocks of
+//     32 tokens, so that three workgroups still share the LDS of a compute unit;
 //   * when the matrix is too small to fill the chip (N small), the k range is also split over
-//     workgroups (grid y); each writes a float32 partial slab that the consumer sums.
-//
-//   * few rows (one block of up to 32 tokens, K % 64 == 0): the slices do not go through registers.
-//     Lane (i, h) reading its own row of W makes every load instruction touch 32 cache lines, and the
-//     address unit of the compute unit, not HBM, then bounds the stream.  Instead each slice is
-//     copied global -> LDS by `global_load_lds_dwordx4` in the order of memory (8 lanes share one
-//     128-byte line, 8 lines per instruction) and the matrix-core operands are read back from LDS;
-//     the copy is asynchronous, so DEPTH slices per wave are in flight without holding registers.
-//     Activations take the same way, only the 8-row groups that hold real tokens.
+//     workgroups (grid y); each writes a float32 partial slab that the consumer sums;
+//   * K % 64 != 0 (any multiple of 8): a plain loop with operands in registers.
 //
 // Epilogues on the float32 sums: bias; SwiGLU (the tile holds 16 gate rows and the 16 matching up
 // rows, so silu(gate) * up is local to a lane; pico_vllm/kernels/swiglu.py:36-41); float32 or
@@ -33,10 +35,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
 
-// The stream of one output tile: sums over k_begin .. k_end of W[wrow0][k] X[m][k] for the 32 tile rows
-// (wrow0: this lane's row of W) and 32 MT tokens, reduced over the 4 waves' k slices into
-// red[wave][token block][register][lane]; the caller sums the 4 waves after the barrier at the end.
-template <int MT, bool TAIL>
+// The sums of one output tile when K is no multiple of 64 (any multiple of 8): operands go through
+// registers, lane (i, h) reads W[row i][k0 + 32 h ..] and the activations alike; k beyond the range
+// reads as zero.  Sums over k_begin .. k_end of W[wrow0][k] X[m][k] for the 32 tile rows (wrow0: this
+// lane's row of W) and 32 MT tokens, each of the 4 waves over its slices, left in
+// red[wave][token block][register][lane]; the caller sums the waves after the barrier at the end.
+template <int MT>
 __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ wrow0,
                                               int m0, int M, int k_begin, int k_end, float (*red)[MT][16][64]) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
@@ -48,75 +52,27 @@ __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int 
   for (int t = 0; t < MT; t++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
-  struct Stage {
-    uint4 w[4], x[MT][4];
-  };
-  auto multiply = [&](const Stage& st) {
+  // this wave's slices start at k_begin + 64 (wave + 4 i)
+  for (int k0 = k_begin + 64 * wave; k0 < k_end; k0 += 256) {
+    u32x4 w[4], x[MT][4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int k = k0 + 32 * h + 8 * s;          // 8 consecutive k; K % 8 == 0, so all or nothing
+      const bool ok = k < k_end;
+      const u32x4 wv = *reinterpret_cast<const u32x4*>(wrow0 + (ok ? k : 0));
+      w[s] = ok ? wv : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        const u32x4 xv = *reinterpret_cast<const u32x4*>(xrow0[t] + (ok ? k : 0));
+        x[t][s] = ok ? xv : u32x4{0, 0, 0, 0};
+      }
+    }
 #pragma unroll
     for (int s = 0; s < 4; s++)
 #pragma unroll
       for (int t = 0; t < MT; t++)
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, st.w[s]),
-                                                         __builtin_bit_cast(bf16x8, st.x[t][s]), acc[t], 0, 0, 0);
-  };
-  // this wave's slices start at k_begin + 64 (wave + 4 i)
-  const int first = k_begin + 64 * wave;
-  if (!TAIL) {
-    // K % 64 == 0: every slice is whole.  DEPTH slices are in flight per wave.  The slices are
-    // taken in rounds of DEPTH: inside a round there is no branch (a branch between a load and the
-    // wait for an older one makes the compiler wait for everything); every step of a round
-    // multiplies one stage and refills it with the slice DEPTH ahead (beyond the wave's last
-    // slice the last one is read again and not used); the last round, the only one that can be
-    // partial, does not refill and multiplies only the slices that exist.
-    constexpr int DEPTH = MT == 1 ? 3 : 2;
-    if (first < k_end) {
-      const int n_slices = (k_end - first + 255) / 256;
-      const int rounds = (n_slices + DEPTH - 1) / DEPTH;
-      const int last = first + (n_slices - 1) * 256;
-      auto load_stage = [&](Stage& st, int slice) {
-        const int k0 = min(first + 256 * slice, last);
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-          st.w[s] = *reinterpret_cast<const uint4*>(wrow0 + k0 + 32 * h + 8 * s);
-#pragma unroll
-          for (int t = 0; t < MT; t++) st.x[t][s] = *reinterpret_cast<const uint4*>(xrow0[t] + k0 + 32 * h + 8 * s);
-        }
-      };
-      Stage st[DEPTH];
-#pragma unroll
-      for (int d = 0; d < DEPTH; d++) load_stage(st[d], d);
-      __builtin_amdgcn_sched_barrier(0);
-      for (int r = 0; r + 1 < rounds; r++) {      // every slice of these rounds exists
-#pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
-          multiply(st[d]);
-          __builtin_amdgcn_sched_barrier(0);     // keeps the refill from sinking next to its use
-          load_stage(st[d], (r + 1) * DEPTH + d);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      const int left = n_slices - (rounds - 1) * DEPTH;           // 1..DEPTH slices in the last round
-#pragma unroll
-      for (int d = 0; d < DEPTH; d++)
-        if (d < left) multiply(st[d]);
-    }
-  } else {
-    for (int k0 = first; k0 < k_end; k0 += 256) {
-      Stage st;
-#pragma unroll
-      for (int s = 0; s < 4; s++) {
-        const int k = k0 + 32 * h + 8 * s;          // 8 consecutive k; K % 8 == 0, so all or nothing
-        const bool ok = k < k_end;
-        const uint4 wv = *reinterpret_cast<const uint4*>(wrow0 + (ok ? k : 0));
-        st.w[s] = ok ? wv : make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int t = 0; t < MT; t++) {
-          const uint4 xv = *reinterpret_cast<const uint4*>(xrow0[t] + (ok ? k : 0));
-          st.x[t][s] = ok ? xv : make_uint4(0, 0, 0, 0);
-        }
-      }
-      multiply(st);
-    }
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[s]), __builtin_bit_cast(bf16x8, x[t][s]),
+                                                         acc[t], 0, 0, 0);
   }
 #pragma unroll
   for (int t = 0; t < MT; t++)
@@ -136,7 +92,9 @@ __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int 
 #define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 constexpr int SK_GROUP = 1024 + 16;
 template <int NX> constexpr int sk_stage_bytes() { return (4 + NX) * SK_GROUP; }
-template <int NX> constexpr int sk_depth() { return NX == 4 ? 2 : 3; }
+template <int NX> constexpr int sk_depth() { return NX >= 4 ? 2 : 3; }
+// waves per workgroup: two when a wave holds two blocks of tokens in LDS, so that three workgroups fit a compute unit
+template <int MT, int NX> constexpr int sk_waves() { return (MT == 2 && NX > 0) ? 2 : 4; }
 // s_waitcnt for "at most n vector memory operations outstanding", nothing else waited for
 constexpr int sk_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
@@ -144,14 +102,17 @@ template <int MT, int NX>
 constexpr int sk_smem_bytes() {
   constexpr int red = 4 * MT * 16 * 64 * 4;
   if (NX == 0) return red;
-  constexpr int stages = sk_depth<NX>() * 4 * sk_stage_bytes<NX>();
+  constexpr int stages = sk_depth<NX>() * sk_waves<MT, NX>() * sk_stage_bytes<NX>();
   return stages > red ? stages : red;
 }
 
 // Tile rows 0..15 are rows row_a .. of W, tile rows 16..31 rows row_b .. (clamped to n_rows - 1);
-// tokens m0 .. m0 + 8 NX - 1 (clamped to M - 1).  The sums of the 4 waves end up in
-// red[wave][0][register][lane] at the start of smem, as skinny_stream leaves them.
-template <int NX>
+// tokens m0 .. m0 + 8 NX - 1 (clamped to M - 1) in MT blocks of 32.  The sums end up in
+// red[v][token block][register][lane] at the start of smem, as skinny_stream leaves them: v = 0..3
+// holds the slices k_begin + 64 (v + 4 i) whatever the number of waves (a wave of a two-wave
+// workgroup keeps two sets of sums), so that a row's result does not depend on how many rows came
+// with it.
+template <int MT, int NX, int NWV>
 __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W,
                                                   int ldw, int row_a, int row_b, int n_rows, int m0, int M, int k_begin,
                                                   int k_end, char* smem) {
@@ -172,19 +133,26 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
   int rd[4];
 #pragma unroll
   for (int s = 0; s < 4; s++) rd[s] = (col >> 3) * SK_GROUP + (col & 7) * 128 + (((4 * h + s) ^ (col & 7)) << 4);
-  char* mine = smem + wave * STAGE;            // stage d of this wave: mine + d * 4 * STAGE
-  f32x16 acc;
+  char* mine = smem + wave * STAGE;            // stage d of this wave: mine + d * NWV * STAGE
+  constexpr int VW = 4 / NWV;                  // sets of sums per wave: slice i of the wave goes to set i % VW
+  static_assert(DEPTH % VW == 0, "a stage must always feed the same set of sums");
+  f32x16 acc[MT][VW];
 #pragma unroll
-  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int v = 0; v < VW; v++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[t][v][r] = 0.f;
 
-  const int first = k_begin + 64 * wave;       // this wave's slices start at k_begin + 64 (wave + 4 i)
+  constexpr int STRIDE = 64 * NWV;             // this wave's slices start at k_begin + 64 (wave + NWV i)
+  const int first = k_begin + 64 * wave;
   if (first < k_end) {
-    const int n_slices = (k_end - first + 255) / 256;
+    const int n_slices = (k_end - first + STRIDE - 1) / STRIDE;
     const int rounds = (n_slices + DEPTH - 1) / DEPTH;
-    const int last = first + (n_slices - 1) * 256;
+    const int last = first + (n_slices - 1) * STRIDE;
     auto issue = [&](int d, int slice) {       // beyond the wave's last slice the last one is copied again
-      const int k0 = min(first + 256 * slice, last);
-      char* dst = mine + d * 4 * STAGE;
+      const int k0 = min(first + STRIDE * slice, last);
+      char* dst = mine + d * NWV * STAGE;
 #pragma unroll
       for (int g = 0; g < 4; g++) __builtin_amdgcn_global_load_lds(GPTR(wsrc[g] + k0), LPTR(dst + g * SK_GROUP), 16, 0, 0);
 #pragma unroll
@@ -192,17 +160,20 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
         __builtin_amdgcn_global_load_lds(GPTR(xsrc[g] + k0), LPTR(dst + (4 + g) * SK_GROUP), 16, 0, 0);
     };
     auto multiply = [&](int d) {
-      const char* src = mine + d * 4 * STAGE;
-      u32x4 a[4], b[4];
+      const char* src = mine + d * NWV * STAGE;
+      u32x4 a[4], b[MT][4];
 #pragma unroll
       for (int s = 0; s < 4; s++) {
         a[s] = *reinterpret_cast<const u32x4*>(src + rd[s]);
-        b[s] = *reinterpret_cast<const u32x4*>(src + 4 * SK_GROUP + rd[s]);
+#pragma unroll
+        for (int t = 0; t < MT; t++) b[t][s] = *reinterpret_cast<const u32x4*>(src + (4 + 4 * t) * SK_GROUP + rd[s]);
       }
 #pragma unroll
       for (int s = 0; s < 4; s++)
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[s]), __builtin_bit_cast(bf16x8, b[s]),
-                                                      acc, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+          acc[t][d % VW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[s]),
+                                                                   __builtin_bit_cast(bf16x8, b[t][s]), acc[t][d % VW], 0, 0, 0);
     };
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) issue(d, d);
@@ -229,9 +200,13 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
       if (d < left) multiply(d);
   }
   __syncthreads();                             // every wave is done with its stages: the sums take their place
-  float(*red)[1][16][64] = reinterpret_cast<float(*)[1][16][64]>(smem);
+  float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
 #pragma unroll
-  for (int r = 0; r < 16; r++) red[wave][0][r][lane] = acc[r];
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int v = 0; v < VW; v++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) red[wave + NWV * v][t][r][lane] = acc[t][v][r];
   __syncthreads();
 }
 
@@ -242,14 +217,14 @@ __device__ __forceinline__ float (*skinny_tile(const bf16_t* __restrict__ X, int
                                                char* smem))[MT][16][64] {
   float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
   if constexpr (NX > 0) {
-    static_assert(MT == 1 && !TAIL, "the stream through LDS takes one block of tokens and whole slices");
-    skinny_stream_lds<NX>(X, ldx, W, ldw, row_a, row_b, n_rows, m0, M, k_begin, k_end, smem);
+    static_assert(!TAIL && NX <= 4 * MT, "the stream through LDS takes whole slices");
+    skinny_stream_lds<MT, NX, sk_waves<MT, NX>()>(X, ldx, W, ldw, row_a, row_b, n_rows, m0, M, k_begin, k_end, smem);
   } else {
     const int col = threadIdx.x & 31;
     const int wrow = col < 16 ? row_a + col : row_b + col - 16;
     // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
     // Only a k tail must read as zero, because it is summed into outputs that are stored.
-    skinny_stream<MT, TAIL>(X, ldx, W + (size_t)min(wrow, n_rows - 1) * ldw, m0, M, k_begin, k_end, red);
+    skinny_stream<MT>(X, ldx, W + (size_t)min(wrow, n_rows - 1) * ldw, m0, M, k_begin, k_end, red);
   }
   return red;
 }
@@ -270,8 +245,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
   float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
 
-  // thread (a = wave, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col`: sum of the 4 waves
-  const int a = wave;
+  // thread (a, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col`: sum of the 4 sets of slices
+  constexpr int NWV = sk_waves<MT, NX>();
+  for (int a = wave; a < 4; a += NWV)
 #pragma unroll
   for (int t = 0; t < MT; t++) {
     const int m = m0 + 32 * t + col;
@@ -343,17 +319,17 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   const float* b0 = bias;
   const bool tail = K % 64 != 0;
   // few rows and whole slices: the stream through LDS, with as many 8-token groups as hold tokens
-  const int nx = (mt == 1 && !tail) ? (M <= 8 ? 1 : M <= 16 ? 2 : 4) : 0;
+  const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH3(MT, EPI, TAIL, NX) \
-  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
 #define LAUNCH(EPI)                                               \
   do {                                                            \
     if (nx == 1) LAUNCH3(1, EPI, false, 1);                       \
     else if (nx == 2) LAUNCH3(1, EPI, false, 2);                  \
     else if (nx == 4) LAUNCH3(1, EPI, false, 4);                  \
+    else if (nx == 8) LAUNCH3(2, EPI, false, 8);                  \
     else if (mt == 1) LAUNCH3(1, EPI, true, 0);                   \
-    else if (tail) LAUNCH3(2, EPI, true, 0);                      \
-    else LAUNCH3(2, EPI, false, 0);                               \
+    else LAUNCH3(2, EPI, true, 0);                                \
   } while (0)
   if (epilogue == EPI_BF16) LAUNCH(EPI_BF16);
   else if (epilogue == EPI_F32) LAUNCH(EPI_F32);
@@ -392,7 +368,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
   const int row_b = rotated ? row_a + half : row_a + 16;
   float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX>(X, ldx, W, ldw, row_a, row_b, (nq + 2 * nkv) * d, m0, M, 0, K, smem);
 
-  const int a = wave;
+  constexpr int NWV = sk_waves<MT, NX>();
+  for (int a = wave; a < 4; a += NWV)
 #pragma unroll
   for (int t = 0; t < MT; t++) {
     const int m = m0 + 32 * t + col;
@@ -470,16 +447,16 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   dim3 grid((nq + 2 * nkv) * (d / 32), 1, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535, "pico_gemm_skinny_rope: too many rows");
   const bool tail = K % 64 != 0;
-  const int nx = (mt == 1 && !tail) ? (M <= 8 ? 1 : M <= 16 ? 2 : 4) : 0;
+  const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH(MT, TAIL, NX) \
-  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
+  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
       (bf16_t*)q_out, ldq, positions, slots, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
   if (nx == 1) LAUNCH(1, false, 1);
   else if (nx == 2) LAUNCH(1, false, 2);
   else if (nx == 4) LAUNCH(1, false, 4);
+  else if (nx == 8) LAUNCH(2, false, 8);
   else if (mt == 1) LAUNCH(1, true, 0);
-  else if (tail) LAUNCH(2, true, 0);
-  else LAUNCH(2, false, 0);
+  else LAUNCH(2, true, 0);
 #undef LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;
