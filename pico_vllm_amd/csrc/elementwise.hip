@@ -61,7 +61,6 @@ template <> __device__ __forceinline__ void store4_f32<bf16_t>(bf16_t* p, float4
 }
 
 // VEC: rows are handled four elements at a time (H % 4 == 0, so every row starts on 16 bytes).
-// All loads of an element group (the stream and up to MAX_SLABS slabs) are issued together.
 template <typename TD, typename TO, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    const float* __restrict__ w, TO* __restrict__ out,
@@ -73,48 +72,62 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   TO* o = out + (size_t)blockIdx.x * H;
   float ss = 0.f;
   if (VEC) {
-    // up to VPT groups of four elements per thread stay in registers from the sum of squares to
-    // the scaling; a longer row is read again for the second pass
+    // The launch gives a row H / 4 threads (up to 1024), so that a thread holds one group of four
+    // elements (up to VPT for a longer row) from the sum of squares to the scaling, and everything
+    // it needs (stream, slabs, weight) is requested before it waits for anything.
     constexpr int VPT = 4;
     const int stride = blockDim.x * 4;
-    const bool in_regs = H <= VPT * stride;
-    float4 keep[VPT];
+    if (H <= VPT * stride) {
+      float4 v[VPT], g[VPT];
 #pragma unroll
-    for (int j = 0; j < VPT; j++) keep[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = threadIdx.x * 4, j = 0; i < H; i += stride, j++) {
+      for (int j = 0; j < VPT; j++) {
+        const int i = threadIdx.x * 4 + j * stride;
+        v[j] = g[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (j * stride < H && i < H) {
+          v[j] = *reinterpret_cast<const float4*>(x + i);
+          g[j] = *reinterpret_cast<const float4*>(w + i);
+          if (dl) {
+            float4 d[MAX_SLABS];
+#pragma unroll
+            for (int s = 0; s < MAX_SLABS; s++)
+              d[s] = s < slabs ? load4_f32(dl + s * slab_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int s = 0; s < MAX_SLABS; s++) { v[j].x += d[s].x; v[j].y += d[s].y; v[j].z += d[s].z; v[j].w += d[s].w; }
+            if (!rows) *reinterpret_cast<float4*>(x + i) = v[j];
+          }
+          ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+        }
+      }
+      ss = block_sum(ss, scratch);
+      const float r = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+      for (int j = 0; j < VPT; j++) {
+        const int i = threadIdx.x * 4 + j * stride;
+        if (j * stride < H && i < H)
+          store4_f32(o + i, make_float4(v[j].x * r * g[j].x, v[j].y * r * g[j].y, v[j].z * r * g[j].z, v[j].w * r * g[j].w));
+      }
+      return;
+    }
+    // a row longer than 16384 elements is read twice
+    for (int i = threadIdx.x * 4; i < H; i += stride) {
       float4 v = *reinterpret_cast<const float4*>(x + i);
       if (dl) {
-        float4 d[MAX_SLABS];
-#pragma unroll
-        for (int s = 0; s < MAX_SLABS; s++)
-          d[s] = s < slabs ? load4_f32(dl + s * slab_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int s = 0; s < MAX_SLABS; s++) { v.x += d[s].x; v.y += d[s].y; v.z += d[s].z; v.w += d[s].w; }
+        for (int s = 0; s < slabs; s++) {
+          const float4 d = load4_f32(dl + s * slab_stride + i);
+          v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
         if (!rows) *reinterpret_cast<float4*>(x + i) = v;
       }
       ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-      if (in_regs) {
-#pragma unroll
-        for (int jj = 0; jj < VPT; jj++)
-          if (jj == j) keep[jj] = v;
-      }
     }
     ss = block_sum(ss, scratch);
     const float r = 1.0f / sqrtf(ss / (float)H + eps);
-    for (int i = threadIdx.x * 4, j = 0; i < H; i += stride, j++) {
-      float4 v;
-      if (in_regs) {
-        v = keep[0];
-#pragma unroll
-        for (int jj = 1; jj < VPT; jj++)
-          if (jj == j) v = keep[jj];
-      } else {
-        v = *reinterpret_cast<const float4*>(x + i);
-        if (dl && rows) {
-          for (int s = 0; s < slabs; s++) {
-            const float4 d = load4_f32(dl + s * slab_stride + i);
-            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
-          }
+    for (int i = threadIdx.x * 4; i < H; i += stride) {
+      float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (dl && rows) {
+        for (int s = 0; s < slabs; s++) {
+          const float4 d = load4_f32(dl + s * slab_stride + i);
+          v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
         }
       }
       const float4 g = *reinterpret_cast<const float4*>(w + i);
@@ -149,7 +162,8 @@ extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype
                    (uintptr_t)delta % 16 == 0 && slab_stride % 4 == 0;
   PICO_REQUIRE(eps > 0.f, "pico_add_rmsnorm: eps must be positive");
   if (T == 0) return 0;
-  const int threads = H >= 4096 ? 512 : (H >= 1024 ? 256 : 128);
+  // vector path: one thread per four elements, in whole waves, up to 1024
+  const int threads = vec ? min(1024, max(64, (H / 4 + 63) / 64 * 64)) : (H >= 4096 ? 512 : (H >= 1024 ? 256 : 128));
 #define LAUNCH(TD, TO)                                                                                                \
   do {                                                                                                                \
     if (vec)                                                                                                          \
@@ -205,10 +219,34 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   store_f32(out + idx, s * u);
 }
 
+// bfloat16 rows whose halves start on 16 bytes (I % 8 == 0): eight elements per thread, 16-byte loads and stores
+__global__ void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I8, size_t total8) {
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total8) return;
+  const size_t row = idx / I8, col = idx % I8;
+  const u32x4 g = *reinterpret_cast<const u32x4*>(gu + (row * 2 * I8 + col) * 8);
+  const u32x4 u = *reinterpret_cast<const u32x4*>(gu + (row * 2 * I8 + I8 + col) * 8);
+  u32x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float g0 = __uint_as_float(g[i] << 16), g1 = __uint_as_float(g[i] & 0xffff0000u);
+    const float u0 = __uint_as_float(u[i] << 16), u1 = __uint_as_float(u[i] & 0xffff0000u);
+    o[i] = pack2_bf16(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+  }
+  *reinterpret_cast<u32x4*>(out + idx * 8) = o;
+}
+
 extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && I > 0, "pico_swiglu: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   const size_t total = (size_t)T * I;
+  if (dtype == PICO_DTYPE_BF16 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t total8 = total / 8;
+    swiglu_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I / 8, total8);
+    PICO_LAUNCH_CHECK();
+    return 0;
+  }
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == PICO_DTYPE_F32)
     swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
@@ -249,7 +287,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
     T* x = row + (size_t)head * d;
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
       const float ang = (float)pos * inv_freq[j];
-      const float c = cosf(ang), s = sinf(ang);
+      float c, s;
+      sincosf(ang, &s, &c);
       const float a = load_f32(x + j), b = load_f32(x + j + half);
       store_f32(x + j, a * c - b * s);
       store_f32(x + j + half, b * c + a * s);
@@ -266,7 +305,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
   T* vc = v_cache + ((size_t)page * nkv + g) * d * P + off;
   for (int j = threadIdx.x; j < half; j += blockDim.x) {
     const float ang = (float)pos * inv_freq[j];
-    const float c = cosf(ang), s = sinf(ang);
+    float c, s;
+    sincosf(ang, &s, &c);
     const float a = load_f32(k + j), b = load_f32(k + j + half);
     store_f32(kc + j, a * c - b * s);
     store_f32(kc + j + half, b * c + a * s);

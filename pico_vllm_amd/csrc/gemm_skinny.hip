@@ -396,7 +396,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
         x1 = bf16_to_f32(f32_to_bf16(x1));
         x2 = bf16_to_f32(f32_to_bf16(x2));
         const float ang = pos * inv_freq[j0 + b];
-        const float c = cosf(ang), s = sinf(ang);
+        float c, s;
+        sincosf(ang, &s, &c);
         y1[b] = x1 * c - x2 * s;
         y2[b] = x2 * c + x1 * s;
       }

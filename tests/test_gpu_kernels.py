@@ -74,6 +74,10 @@ def test_swiglu(K, dtype):
     close(K.swiglu(gu.to(DEV)), P.swiglu(gu), dtype)
     g = gu[:, :172].float()
     close(K.swiglu(torch.cat([gu[:, :172], torch.ones(5, 172).to(dtype)], -1).to(DEV)), F.silu(g), dtype)
+    # halves that are multiples of 8 take the kernel with 16-byte loads in bfloat16
+    for T, I in ((3, 8), (70, 320), (33, 8960)):
+        gu = (torch.randn(T, 2 * I) * 2).to(dtype)
+        close(K.swiglu(gu.to(DEV)), P.swiglu(gu), dtype)
 
 
 @pytest.mark.parametrize("M,N,K_", [(1, 301, 136), (5, 64, 172), (70, 130, 64), (130, 17, 33)])
