@@ -2,6 +2,7 @@
 """Decode and prefill throughput at the Qwen2.5-1.5B shape with random weights on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
+  python bench.py --shape 7b --layers 8 --context 8192      (other sizes and context lengths)
 
 A step is one decode step of the engine (scheduler, model step from a HIP graph, sampling) at
 batch 8 with every request's context ending at 4096 tokens.  One JSON line goes to stdout:
@@ -33,6 +34,15 @@ CONFIG_1P5B = {
     "num_key_value_heads": 2, "intermediate_size": 8960, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
     "tie_word_embeddings": True, "max_position_embeddings": 131072, "hidden_act": "silu",
 }
+# BASELINE.json configs[3]: Qwen2.5-7B (measured with fewer layers when asked: --layers)
+CONFIG_7B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 152064, "hidden_size": 3584, "num_hidden_layers": 28, "num_attention_heads": 28,
+    "num_key_value_heads": 4, "intermediate_size": 18944, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
+    "tie_word_embeddings": False, "max_position_embeddings": 131072, "hidden_act": "silu",
+}
+SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", CONFIG_1P5B), "7b": ("Qwen2.5-7B shape", CONFIG_7B)}
+CONFIG = CONFIG_1P5B         # the shape being measured (set in main)
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 
@@ -66,7 +76,7 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
     """Fill `batch` requests so that the timed steps end at CONTEXT tokens, then time `steps` decode steps."""
     import torch
     eng = make_engine(model_dir, dtype, batch, model)
-    V = CONFIG_1P5B["vocab_size"]
+    V = CONFIG["vocab_size"]
     g = torch.Generator().manual_seed(batch)
     # while later prompts are still being prefilled the earlier requests already decode: leave room for that
     slack = batch * (-(-CONTEXT // PREFILL_TOKENS)) + 2
@@ -106,7 +116,7 @@ def prefill_point(model_dir, model, dtype, reps=3):
     import torch
     from pico_vllm_amd.engine.batch import SeqStep
     eng = make_engine(model_dir, dtype, 1, model)
-    V = CONFIG_1P5B["vocab_size"]
+    V = CONFIG["vocab_size"]
     ids = torch.randint(0, V, (PREFILL_TOKENS,), generator=torch.Generator().manual_seed(7)).tolist()
     m = eng.runner.manager
     times = []
@@ -123,7 +133,7 @@ def prefill_point(model_dir, model, dtype, reps=3):
         m.free_request(rid)
     dt = min(times[1:])
     return {"value": PREFILL_TOKENS / dt, "tokens": PREFILL_TOKENS, "ms": dt * 1e3,
-            "frac": prefill_flops(CONFIG_1P5B, PREFILL_TOKENS) / dt / MFMA_PEAK[dtype]}
+            "frac": prefill_flops(CONFIG, PREFILL_TOKENS) / dt / MFMA_PEAK[dtype]}
 
 
 def main() -> int:
@@ -138,17 +148,29 @@ def main() -> int:
     ap.add_argument("--write-model", metavar="DIR", default=None,
                     help="only write the random-weights model folder to DIR (to reuse with --model) and exit")
     ap.add_argument("--model", default=None, help="reuse a model folder instead of writing random weights")
+    ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
+    ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
+    ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
     a = ap.parse_args()
+    global CONFIG, CONTEXT
+    shape_name, full = SHAPES[a.shape]
+    CONFIG = dict(full)
+    if a.layers:
+        if not 0 < a.layers <= full["num_hidden_layers"]:
+            print(f"bench.py: --layers must be 1..{full['num_hidden_layers']}")
+            return 2
+        CONFIG["num_hidden_layers"] = a.layers
+    CONTEXT = a.context
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
         return 2
-    if a.steps + a.warmup >= CONTEXT // 2 - 200:
-        print("bench.py: steps + warmup must stay below 1848")
+    if CONTEXT < 2 * PREFILL_TOKENS or a.steps + a.warmup >= CONTEXT // 2 - 200:
+        print(f"bench.py: the context must be at least {2 * PREFILL_TOKENS} and steps + warmup below {CONTEXT // 2 - 200}")
         return 2
     import torch
     from pico_vllm_amd.weights.random_init import write_random_model
     if a.write_model:
-        write_random_model(a.write_model, CONFIG_1P5B, seed=0)
+        write_random_model(a.write_model, CONFIG, seed=0)
         print(f"wrote {a.write_model}")
         return 0
     tmp = None
@@ -157,8 +179,8 @@ def main() -> int:
         tmp = tempfile.mkdtemp(prefix="pico_bench_")
         model_dir = tmp
         t0 = time.time()
-        log("writing random Qwen2.5-1.5B-shaped weights ...")
-        write_random_model(model_dir, CONFIG_1P5B, seed=0)
+        log(f"writing random weights of the {shape_name}, {CONFIG['num_hidden_layers']} layers ...")
+        write_random_model(model_dir, CONFIG, seed=0)
         log(f"... {time.time() - t0:.0f}s")
     try:
         if a.prefill_only:
@@ -167,14 +189,18 @@ def main() -> int:
         main_res, model = decode_point(model_dir, None, a.dtype, a.batch, a.steps, a.warmup)
         log(f"decode batch {a.batch}: {main_res['tok_s']:.0f} tok/s, {main_res['ms_per_step']:.3f} ms/step")
         out = {
-            "metric": "decode tok/s @ batch 8, Qwen2.5-1.5B bf16 (plus batch 1/64 and prefill @ 2048 tok)",
+            "metric": f"decode tok/s @ batch {a.batch}, {shape_name.split()[0]} bf16 (plus batch 1/64 and prefill @ 2048 tok)",
             "value": round(main_res["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
             "warmup": a.warmup, "ms_per_step": round(main_res["ms_per_step"], 4), "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
-            "config": {"model": "Qwen2.5-1.5B shape", "global_batch": a.batch, "seq_len": CONTEXT,
-                       "parallelism": "single GPU", "layers": 28, "layers_run": 28, "hidden": 1536, "q_heads": 12,
-                       "kv_heads": 2, "head_dim": 128, "intermediate": 8960, "vocab": 151936, "tied": True,
+            "config": {"model": shape_name, "global_batch": a.batch, "seq_len": CONTEXT,
+                       "parallelism": "single GPU", "layers": full["num_hidden_layers"],
+                       "layers_run": CONFIG["num_hidden_layers"], "hidden": CONFIG["hidden_size"],
+                       "q_heads": CONFIG["num_attention_heads"], "kv_heads": CONFIG["num_key_value_heads"],
+                       "head_dim": CONFIG["hidden_size"] // CONFIG["num_attention_heads"],
+                       "intermediate": CONFIG["intermediate_size"], "vocab": CONFIG["vocab_size"],
+                       "tied": CONFIG["tie_word_embeddings"],
                        "page_size": 16, "prompt_len": int(main_res["prompt_len"]),
                        "context_in_timed_steps": round(main_res["context"], 1)},
             "roofline": {"bound": "hbm", "achieved": round(main_res["gbps"], 1), "peak": HBM_PEAK / 1e9,
