@@ -266,6 +266,8 @@ extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, h
 //     out[j]         = x[j] * cos - x[j + rot/2] * sin
 //     out[j + rot/2] = x[j + rot/2] * cos + x[j] * sin
 //   entries at index >= rot pass through unrotated.
+// Cosine and sine come from a table cos_sin [T][rot/2][2] that pico_rope_table fills once per
+// step: every layer of a step rotates by the same angles.
 // qkv: [T, (nq + 2 nkv) * d], rows [q heads | k heads | v heads]; q is rotated in place.
 // Cache of one layer: K pages [page][kv head][slot in page][d],
 //                     V pages [page][kv head][d][slot in page]  (slot contiguous).
@@ -274,21 +276,40 @@ extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, h
 // "store nothing" (padding rows of a captured batch).
 // Grid (T, nq + nkv); block 64.
 // ---------------------------------------------------------------------------
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float2* __restrict__ cos_sin, int half) {
+  const int t = blockIdx.x;
+  const float pos = (float)positions[t];
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    float c, s;
+    sincosf(pos * inv_freq[j], &s, &c);
+    cos_sin[(size_t)t * half + j] = make_float2(c, s);
+  }
+}
+
+extern "C" int pico_rope_table(const int* positions, const float* inv_freq, float* cos_sin, int T, int half,
+                               hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && half >= 0, "pico_rope_table: bad sizes");
+  PICO_REQUIRE((uintptr_t)cos_sin % 8 == 0, "pico_rope_table: the table must be 8-byte aligned");
+  if (T == 0 || half == 0) return 0;
+  rope_table_kernel<<<T, 64, 0, stream>>>(positions, inv_freq, (float2*)cos_sin, half);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
 template <typename T>
-__global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
-                                  const int* __restrict__ slots, const float* __restrict__ inv_freq,
+__global__ void rope_store_kernel(T* __restrict__ qkv, const float2* __restrict__ cos_sin,
+                                  const int* __restrict__ slots,
                                   T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv, int d, int rot,
                                   int P, int num_pages) {
   const int t = blockIdx.x, head = blockIdx.y;
-  const int pos = positions[t];
   T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
   const int half = rot >> 1;
+  const float2* cs = cos_sin + (size_t)t * half;
   if (head < nq) {
     T* x = row + (size_t)head * d;
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
-      const float ang = (float)pos * inv_freq[j];
-      float c, s;
-      sincosf(ang, &s, &c);
+      const float c = cs[j].x, s = cs[j].y;
       const float a = load_f32(x + j), b = load_f32(x + j + half);
       store_f32(x + j, a * c - b * s);
       store_f32(x + j + half, b * c + a * s);
@@ -304,9 +325,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
   T* kc = k_cache + (((size_t)page * nkv + g) * P + off) * d;
   T* vc = v_cache + ((size_t)page * nkv + g) * d * P + off;
   for (int j = threadIdx.x; j < half; j += blockDim.x) {
-    const float ang = (float)pos * inv_freq[j];
-    float c, s;
-    sincosf(ang, &s, &c);
+    const float c = cs[j].x, s = cs[j].y;
     const float a = load_f32(k + j), b = load_f32(k + j + half);
     store_f32(kc + j, a * c - b * s);
     store_f32(kc + j + half, b * c + a * s);
@@ -315,18 +334,19 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
   for (int j = threadIdx.x; j < d; j += blockDim.x) vc[(size_t)j * P] = v[j];
 }
 
-extern "C" int pico_rope_kv_store(void* qkv, int dtype, const int* positions, const int* slots,
-                                  const float* inv_freq, void* k_cache, void* v_cache, int T, int nq, int nkv, int d,
+extern "C" int pico_rope_kv_store(void* qkv, int dtype, const float* cos_sin, const int* slots,
+                                  void* k_cache, void* v_cache, int T, int nq, int nkv, int d,
                                   int rot, int P, int num_pages, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && d > 0 && P > 0 && num_pages > 0, "pico_rope_kv_store: bad sizes");
   PICO_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "pico_rope_kv_store: rotary size %d does not fit head size %d", rot, d);
+  PICO_REQUIRE(rot == 0 || (cos_sin != nullptr && (uintptr_t)cos_sin % 8 == 0), "pico_rope_kv_store: no table of cosines and sines");
   if (T == 0) return 0;
   dim3 grid(T, nq + nkv);
   if (dtype == PICO_DTYPE_F32)
-    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, positions, slots, inv_freq, (float*)k_cache,
+    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, (const float2*)cos_sin, slots, (float*)k_cache,
                                                       (float*)v_cache, nq, nkv, d, rot, P, num_pages);
   else if (dtype == PICO_DTYPE_BF16)
-    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, positions, slots, inv_freq, (bf16_t*)k_cache,
+    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, (const float2*)cos_sin, slots, (bf16_t*)k_cache,
                                                        (bf16_t*)v_cache, nq, nkv, d, rot, P, num_pages);
   else
     PICO_REQUIRE(false, "pico_rope_kv_store: unknown dtype %d", dtype);

@@ -348,6 +348,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
 // holds 16 rows j .. j + 15 of the head and the 16 rows j + d/2 .. they are rotated with, so a pair
 // is local to a lane as gate and up are in the SwiGLU epilogue; a tile of a v head holds 32
 // consecutive rows.  Needs rot == d and d % 32 == 0.
+//   cos_sin [M][d / 2][2] float32: cosine and sine of every token's angles (pico_rope_table);
 //   q_out [M, ldq] bfloat16 gets the rotated q heads at columns head * d + dim;
 //   K pages [page][kv head][slot][d], V pages [page][kv head][d][slot], P = 1 << pshift slots;
 //   slots[m] = page * P + slot of token m, negative: store nothing.
@@ -355,8 +356,8 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
 template <int MT, bool TAIL, int NX>
 __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
     const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
-    bf16_t* __restrict__ q_out, int ldq, const int* __restrict__ positions, const int* __restrict__ slots,
-    const float* __restrict__ inv_freq, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
+    bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
+    bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
     int nq, int nkv, int d, int pshift, int num_pages) {
   __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX>()];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
@@ -377,7 +378,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
     if (rotated) {
       if (a >= 2) continue;
       const int j0 = 16 * tp + 8 * a + 4 * h;        // this thread's four pairs (j, j + d/2)
-      const float pos = (float)positions[m];
+      const float2* cs = cos_sin + (size_t)m * half + j0;
       float y1[4], y2[4];
 #pragma unroll
       for (int b = 0; b < 4; b++) {
@@ -395,9 +396,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
         // the same key whether it came in a small step (here) or in a large one
         x1 = bf16_to_f32(f32_to_bf16(x1));
         x2 = bf16_to_f32(f32_to_bf16(x2));
-        const float ang = pos * inv_freq[j0 + b];
-        float c, s;
-        sincosf(ang, &s, &c);
+        const float c = cs[b].x, s = cs[b].y;
         y1[b] = x1 * c - x2 * s;
         y2[b] = x2 * c + x1 * s;
       }
@@ -431,9 +430,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
 }
 
 extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int ldw, const float* bias, void* q_out,
-                                     int ldq, const int* positions, const int* slots, const float* inv_freq,
+                                     int ldq, const float* cos_sin, const int* slots,
                                      void* k_cache, void* v_cache, int M, int K, int nq, int nkv, int d, int P,
                                      int num_pages, hipStream_t stream) {
+  PICO_REQUIRE(cos_sin != nullptr && (uintptr_t)cos_sin % 8 == 0, "pico_gemm_skinny_rope: no table of cosines and sines");
   PICO_REQUIRE(M > 0 && K > 0 && nq > 0 && nkv > 0 && num_pages > 0, "pico_gemm_skinny_rope: bad sizes");
   PICO_REQUIRE(d >= 32 && d % 32 == 0, "pico_gemm_skinny_rope: head size %d is not a multiple of 32", d);
   PICO_REQUIRE(P >= 1 && (P & (P - 1)) == 0, "pico_gemm_skinny_rope: page size %d is not a power of two", P);
@@ -451,7 +451,7 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH(MT, TAIL, NX) \
   gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
-      (bf16_t*)q_out, ldq, positions, slots, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
+      (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
   if (nx == 1) LAUNCH(1, false, 1);
   else if (nx == 2) LAUNCH(1, false, 2);
   else if (nx == 4) LAUNCH(1, false, 4);

@@ -270,33 +270,53 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int)
     return pages, P
 
 
-def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, inv_freq: torch.Tensor,
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """cos and sin of position * inv_freq in float32: [T, len(inv_freq), 2].  Every layer of a step
+    rotates by the same angles, so a step computes them once."""
+    _gpu(positions, inv_freq)
+    T = positions.numel()
+    _i32(positions, "positions", T)
+    if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous():
+        raise KernelError("inv_freq must be contiguous float32")
+    out = torch.empty(T, inv_freq.numel(), 2, dtype=torch.float32, device=positions.device)
+    lib = library.core()
+    _check(lib, lib.pico_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(out), T, inv_freq.numel(), _stream()))
+    return out
+
+
+def _check_table(cos_sin: Optional[torch.Tensor], T: int, half: int) -> None:
+    if half == 0:
+        return
+    if cos_sin is None or cos_sin.dtype != torch.float32 or cos_sin.shape != (T, half, 2) or not cos_sin.is_contiguous():
+        raise KernelError(f"the table of cosines and sines must be contiguous float32 [{T}, {half}, 2]")
+
+
+def rope_kv_store(qkv: torch.Tensor, cos_sin: Optional[torch.Tensor], slots: torch.Tensor,
                   k_cache: torch.Tensor, v_cache: torch.Tensor, nq: int, nkv: int, d: int, rotary_dim: int) -> None:
-    """Rotate q (in place) and k, write k and v of token t to slot ``slots[t]`` (page * page size +
-    offset in the page; negative: nothing is stored)."""
-    _gpu(qkv, positions, slots, inv_freq, k_cache, v_cache)
+    """Rotate q (in place) and k by the angles of ``cos_sin`` (``rope_table``; None when rotary_dim
+    is 0), write k and v of token t to slot ``slots[t]`` (page * page size + offset in the page;
+    negative: nothing is stored)."""
+    _gpu(qkv, cos_sin, slots, k_cache, v_cache)
     T = qkv.shape[0]
     if qkv.shape != (T, (nq + 2 * nkv) * d) or not qkv.is_contiguous():
         raise KernelError(f"qkv must be contiguous [T, {(nq + 2 * nkv) * d}], got {tuple(qkv.shape)}")
     pages, P = _check_cache(k_cache, v_cache, nkv, d)
     if k_cache.dtype != qkv.dtype:
         raise KernelError("cache and activations differ in dtype")
-    _i32(positions, "positions", T)
     _i32(slots, "slots", T)
-    if inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2 or not inv_freq.is_contiguous():
-        raise KernelError("inv_freq must be float32 of rotary_dim / 2 entries")
+    _check_table(cos_sin, T, rotary_dim // 2)
     lib = library.core()
-    _check(lib, lib.pico_rope_kv_store(_ptr(qkv), _dt(qkv), _ptr(positions), _ptr(slots), _ptr(inv_freq),
+    _check(lib, lib.pico_rope_kv_store(_ptr(qkv), _dt(qkv), _ptr(cos_sin) if rotary_dim else None, _ptr(slots),
                                        _ptr(k_cache), _ptr(v_cache), T, nq, nkv, d, rotary_dim, P, pages, _stream()))
 
 
-def gemm_skinny_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
-                     slots: torch.Tensor, inv_freq: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+def gemm_skinny_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: torch.Tensor,
+                     slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      nq: int, nkv: int, d: int) -> torch.Tensor:
     """The q/k/v projection of up to 64 tokens with bias, rotate-half encoding of q and k (over the
     whole head size) and the store of k and v at ``slots`` in one kernel; returns the encoded queries
     [M, nq * d].  w: [(nq + 2 nkv) * d, K] bfloat16, rows [q heads | k heads | v heads]."""
-    _gpu(a, w, bias, positions, slots, inv_freq, k_cache, v_cache)
+    _gpu(a, w, bias, cos_sin, slots, k_cache, v_cache)
     M, K = a.shape
     if w.shape != ((nq + 2 * nkv) * d, K):
         raise KernelError(f"gemm_skinny_rope: weight {tuple(w.shape)} is not [{(nq + 2 * nkv) * d}, {K}]")
@@ -309,14 +329,12 @@ def gemm_skinny_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
         raise KernelError("gemm_skinny_rope: the cache must be bfloat16")
     if d % 32 or P & (P - 1):
         raise KernelError("gemm_skinny_rope: head size must be a multiple of 32 and the page size a power of two")
-    _i32(positions, "positions", M)
     _i32(slots, "slots", M)
-    if inv_freq.dtype != torch.float32 or inv_freq.numel() != d // 2 or not inv_freq.is_contiguous():
-        raise KernelError("gemm_skinny_rope: inv_freq must be float32 of head size / 2 entries")
+    _check_table(cos_sin, M, d // 2)
     q = torch.empty(M, nq * d, dtype=torch.bfloat16, device=a.device)
     lib = library.core()
     _check(lib, lib.pico_gemm_skinny_rope(_ptr(a), a.stride(0) if M > 1 else K, _ptr(w), w.stride(0), _ptr(bias), _ptr(q),
-                                          nq * d, _ptr(positions), _ptr(slots), _ptr(inv_freq), _ptr(k_cache),
+                                          nq * d, _ptr(cos_sin), _ptr(slots), _ptr(k_cache),
                                           _ptr(v_cache), M, K, nq, nkv, d, P, pages, _stream()))
     return q
 

@@ -47,6 +47,7 @@ class StepContext:
     max_context: int = 1             # longest context in the batch
     all_decode: bool = False         # every sequence brings exactly one token
     host: Dict[str, Any] = field(default_factory=dict)   # numpy copies of the arrays above
+    shared: Dict[Any, Any] = field(default_factory=dict)  # what parts compute once per step and share between layers
 
 
 class Part:

@@ -116,6 +116,7 @@ class DecoderModel:
             return self._forward(ctx, storage)
 
     def _forward(self, ctx: StepContext, storage) -> torch.Tensor:
+        ctx.shared.clear()      # what layers share belongs to this pass (a context may be run again, as at graph capture)
         resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens])
         pending = None
         for i, e in enumerate(self.spec.run_order):

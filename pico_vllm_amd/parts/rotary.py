@@ -27,16 +27,23 @@ class RotaryHalf(PositionEncoding):
         inv = 1.0 / (self.theta ** (torch.arange(0, d, 2).float() / d))
         self.inv_freq = inv.to(device).contiguous()
 
+    def table(self, ctx) -> torch.Tensor:
+        """cos and sin of every token's angles, [T, rotary_dim / 2, 2]; the first layer of a step
+        that asks computes them, the others find them in ``ctx.shared``."""
+        key = ("rotary_half", self.rotary_dim, self.theta)
+        if key not in ctx.shared:
+            ctx.shared[key] = kernels.rope_table(ctx.positions[:ctx.num_tokens], self.inv_freq)
+        return ctx.shared[key]
+
     def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
-        kernels.rope_kv_store(qkv, ctx.positions, ctx.slot_mapping[kv.group], self.inv_freq,
-                              kv.k, kv.v, nq, nkv, d, self.rotary_dim)
+        kernels.rope_kv_store(qkv, self.table(ctx), ctx.slot_mapping[kv.group], kv.k, kv.v, nq, nkv, d, self.rotary_dim)
 
     def project_rotate_store(self, x, linear, ctx, kv, block_table, nq, nkv, d) -> torch.Tensor:
         # few tokens in bfloat16: projection, bias, rotation and cache store are one weight-streaming kernel
         if (self.rotary_dim == d and d % 32 == 0 and kv.k.dtype == torch.bfloat16
                 and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0 and kernels.skinny_ok(x, linear.weight)):
-            return kernels.gemm_skinny_rope(x, linear.weight, linear.bias_f32, ctx.positions, ctx.slot_mapping[kv.group],
-                                            self.inv_freq, kv.k, kv.v, nq, nkv, d)
+            return kernels.gemm_skinny_rope(x, linear.weight, linear.bias_f32, self.table(ctx), ctx.slot_mapping[kv.group],
+                                            kv.k, kv.v, nq, nkv, d)
         return super().project_rotate_store(x, linear, ctx, kv, block_table, nq, nkv, d)
 
 
@@ -45,11 +52,7 @@ class NoPosition(PositionEncoding):
     """No position encoding: keys and values are stored as they are."""
 
     def __init__(self, act_dtype: torch.dtype = torch.bfloat16):
-        self._empty = None
-
-    def load(self, tensors, device, dtype) -> None:
-        self._empty = torch.zeros(0, dtype=torch.float32, device=device)
+        pass
 
     def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
-        kernels.rope_kv_store(qkv, ctx.positions, ctx.slot_mapping[kv.group], self._empty,
-                              kv.k, kv.v, nq, nkv, d, 0)
+        kernels.rope_kv_store(qkv, None, ctx.slot_mapping[kv.group], kv.k, kv.v, nq, nkv, d, 0)

@@ -137,7 +137,11 @@ def test_rope_and_cache_store(K, dtype, nq, nkv, d, rot, Pg):
     x = qkv.clone().to(DEV)
     slots = torch.tensor([int(bt[int(b), int(p) // Pg]) * Pg + int(p) % Pg for b, p in zip(seq, pos)],
                          dtype=torch.int32, device=DEV)
-    K.rope_kv_store(x, pos, slots, inv, kc, vc, nq, nkv, d, rot)
+    table = K.rope_table(pos.to(DEV), inv)
+    want_cos, want_sin = P.rope_tables(pos.cpu(), rot, theta)
+    assert torch.allclose(table[..., 0].cpu(), want_cos[:, :rot // 2], atol=2e-6)
+    assert torch.allclose(table[..., 1].cpu(), want_sin[:, :rot // 2], atol=2e-6)
+    K.rope_kv_store(x, table, slots, kc, vc, nq, nkv, d, rot)
     # reference
     q, k, v = P.split_qkv(qkv.float(), nq, nkv, d)
     cos, sin = P.rope_tables(pos.cpu(), rot, theta)
@@ -416,8 +420,8 @@ def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias
     kc = torch.full((num_pages, nkv, Pg, d), 7.0, dtype=torch.bfloat16, device=DEV)
     vc = torch.full((num_pages, nkv, d, Pg), 7.0, dtype=torch.bfloat16, device=DEV)
     inv = (1.0 / (theta ** (torch.arange(0, d, 2).float() / d))).to(DEV)
-    q_out = K.gemm_skinny_rope(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), pos.to(DEV), slots.to(DEV), inv,
-                               kc, vc, nq, nkv, d)
+    q_out = K.gemm_skinny_rope(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), K.rope_table(pos.to(DEV), inv),
+                               slots.to(DEV), kc, vc, nq, nkv, d)
     qkv = (x.double() @ w.double().T + (0 if b is None else b.double())).float()
     q, k, v = P.split_qkv(qkv, nq, nkv, d)
     cos, sin = P.rope_tables(pos, d, theta)
