@@ -1,22 +1,24 @@
 // Paged attention on the matrix cores for bfloat16, specialised at compile time for one head
-// size D = PICO_HEAD_DIM (a multiple of 16 up to 256).  Two kernels share the tile code:
+// size D = PICO_HEAD_DIM (a multiple of 16 up to 256).
 //
-//   prefill / mixed  one workgroup (4 waves) per 128 query tokens of one sequence and one query
-//                    head; each wave owns 32 queries; keys and values of the sequence stream
-//                    through LDS in tiles of BN keys, from position 0 to the causal frontier.
-//                    A decode token is a sequence that brings one query.
+//   prefill / mixed  a workgroup owns a tile of query tokens of one sequence and one query head; keys
+//                    and values of the sequence stream through LDS in tiles, from position 0 to the
+//                    causal frontier.  A decode token is a sequence that brings one query.
+//                    D % 32 == 0: prefill16_kernel, 64 queries per workgroup, 16 per wave
+//                    (v_mfma_f32_16x16x32_bf16), one or two teams of four waves that share the key loop;
+//                    other D: prefill_kernel, 128 queries per workgroup, 32 per wave (32x32x16).
 //   decode           one workgroup per (sequence, kv head, split of the context); the
 //                    "queries" are the G query heads that share the kv head, so keys and values
 //                    are read once for the whole group (the reference's kernel re-reads them per
-//                    query head, pico_vllm/kernels/attention.py:96-105); two waves split the keys of a tile
-//                    (the other two only help to move tiles);
-//                    partial (max, sum, output) per split are merged by a second kernel.
+//                    query head, pico_vllm/kernels/attention.py:96-105).  decode16_kernel (G <= 16,
+//                    D % 32 == 0, D <= 128) loads its operands straight from the pages, decode_kernel
+//                    stages tiles in LDS; partial (max, sum, output) per split are merged by a second kernel.
 //
 // Formulas as in pico_vllm/kernels/attention.py:136-213: scores (q.k) * scale, key visible iff its
 // position <= the query's, online softmax in float32, probabilities rounded to bfloat16 for the
 // P.V product, float32 accumulators.
 //
-// Matrix-core layout (v_mfma_f32_32x32x16_bf16, D = A B, A 32x16, B 16x32): lane l supplies
+// Matrix-core layout of the 32-query kernels (v_mfma_f32_32x32x16_bf16, D = A B, A 32x16, B 16x32): lane l supplies
 // A[l % 32][8 (l / 32) + 0..7] and B[8 (l / 32) + 0..7][l % 32]; it receives, in register r,
 // D[8 (r / 4) + 4 (l / 32) + r % 4][l % 32].  Scores are computed TRANSPOSED, S^T = K Q^T, so a
 // query is a column: its 32 scores of a key tile sit in the 16 registers of two lanes (l, l ^ 32)
@@ -1009,7 +1011,7 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
   PICO_REQUIRE(num_seqs > 0 && num_tokens >= num_seqs, "pico_attn_prefill: bad batch (%d sequences, %d tokens)", num_seqs, num_tokens);
   PICO_REQUIRE(nq <= 65535, "pico_attn_prefill: too many heads");
   PICO_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "pico_attn_prefill: misaligned tensors");
-#if PICO_HEAD_DIM % 32 == 0 && !defined(PICO_PF_WIDE)
+#if PICO_HEAD_DIM % 32 == 0
   // the 16-query kernel addresses the cache with 32-bit byte offsets
   if ((uint64_t)num_pages * nkv * P * D * sizeof(bf16_t) < (1ull << 32)) {
     const int max_tiles = num_tokens / PF_BM + num_seqs;  // >= sum over sequences of ceil(len / PF_BM)
