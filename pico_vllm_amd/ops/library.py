@@ -46,7 +46,7 @@ def _hipcc() -> str:
                            "the HIP kernels cannot be built and there is no other code path")
 
 
-def _build_root() -> str:
+def build_root() -> str:
     """In-tree ``_build`` if it can be written, else a per-user folder under the temp dir."""
     tree = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "_build"))
     try:
@@ -78,7 +78,7 @@ def _say(msg: str) -> None:
 
 def build_library(name: str, sources: Sequence[str], defines: Sequence[str] = (), force: bool = False) -> str:
     """Compile ``sources`` (names under csrc/) into lib<name>.so and return its path."""
-    root = _build_root()
+    root = build_root()
     so = os.path.join(root, f"lib{name}.so")
     stamp = so + ".hash"
     digest = _digest(sources, defines)

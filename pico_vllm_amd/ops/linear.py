@@ -11,11 +11,44 @@ engine) they are widened on load and the result is rounded once.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
 
-from . import kernels
+from . import kernels, library
+
+# The library GEMM is picked by the library's own tuner (PyTorch's TunableOp: it times the rocBLAS and
+# hipBLASLt solutions for a shape once and keeps the fastest; on the 1.5B shapes with 2,048 rows that
+# is 91 us against 122 us for the gate/up product).  A step's row count is arbitrary, and tuning every
+# count would stall serving, so only row counts that are multiples of TUNE_ROWS (whole prompt portions)
+# are tuned; every other count takes the library's default choice.  Results are kept beside the built
+# kernels and read back by the next process.
+TUNE_ROWS = 512
+_tuner_state = {"ready": False, "tuning": None}
+
+
+def _library_tuning(rows: int) -> None:
+    tunable = torch.cuda.tunable
+    st = _tuner_state
+    if not st["ready"]:
+        st["ready"] = True
+        try:
+            path = os.path.join(library.build_root(), "tunableop_gemm.csv")
+            tunable.enable(True)
+            tunable.set_filename(path)
+            tunable.set_max_tuning_duration(30)
+            tunable.set_max_tuning_iterations(20)
+            if os.path.exists(path):
+                tunable.read_file(path)
+        except Exception:                      # a build of torch without the tuner: the default choice serves
+            st["ready"] = "off"
+    if st["ready"] == "off":
+        return
+    want = rows % TUNE_ROWS == 0
+    if st["tuning"] != want:
+        tunable.tuning_enable(want)
+        st["tuning"] = want
 
 
 class Linear:
@@ -41,6 +74,7 @@ class Linear:
             return kernels.gemm_skinny(x, self.weight, self.bias_f32, epi)
         if out_dtype == torch.float32:
             return kernels.gemm_bf16(x, self.weight, self.bias_f32, torch.float32)
+        _library_tuning(x.shape[0])
         if self.bias is not None:
             return torch.addmm(self.bias, x, self.weight.t())
         return torch.mm(x, self.weight.t())
