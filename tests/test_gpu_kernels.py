@@ -283,7 +283,7 @@ def test_sampling_top_p(K):
 
 
 # ---- matrix-core attention (bfloat16) ----------------------------------------------------------
-def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1):
+def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0):
     from pico_vllm_amd.ops.attention_fast import FastAttention
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(seed)
@@ -307,7 +307,7 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
     if decode:
         out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
     else:
-        out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale)
+        out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale, teams=teams)
     want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n))
                       for qb, kb, vb, n, p in zip(qs, ks, vs, new_lens, prefix_lens)], 0)
     return out.reshape(-1, nq, d), want
@@ -326,6 +326,56 @@ def test_fast_prefill_other_sizes_and_long_portions(K, nq, nkv, d, Pg):
     # portions longer than one 128-query tile, a decode token, a 2-token portion, long prefixes
     out, want = _fast_case([7, 1, 300, 2, 129], [0, 70, 45, 129, 500], nq, nkv, d, Pg, seed=3)
     close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("teams", [1, 2])
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64)])
+def test_fast_prefill_with_one_and_two_key_teams(K, nq, nkv, d, Pg, teams):
+    # the number of waves that share a query tile's key loop is a hint: every value gives the same attention;
+    # lengths around the 64-query tile and the 64- and 128-key tiles of one and two teams
+    out, want = _fast_case([63, 1, 65, 130, 2, 200], [0, 127, 1, 62, 191, 129], nq, nkv, d, Pg, seed=5, teams=teams)
+    close(out, want, torch.bfloat16)
+
+
+def test_fast_prefill_chooses_teams_by_the_shape_of_the_batch():
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    fa = FastAttention.__new__(FastAttention)
+    fa.nq = 12
+    assert fa.prefill_teams([2048], [2048]) == 2            # a causal triangle: the longest tile decides
+    assert fa.prefill_teams([512], [4096]) == 2             # few tiles
+    assert fa.prefill_teams([1] * 8, [4000] * 8) == 2       # decode tokens inside a mixed step
+    assert fa.prefill_teams([2048], [16384]) == 1           # many long, equal tiles
+
+
+def test_fast_prefill_with_a_cache_of_4_gib(K):
+    # offsets into such a cache do not fit 32 bits: the kernel with 64-bit addresses serves it;
+    # the pages used lie at both ends of the cache
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    nq, nkv, d, Pg = 2, 1, 64, 16
+    pages = (1 << 32) // (nkv * Pg * d * 2) + 7
+    g = torch.Generator().manual_seed(11)
+    n, prefix = 70, 90
+    N = n + prefix
+    k = torch.randn(N, nkv, d, generator=g).bfloat16().float()
+    v = torch.randn(N, nkv, d, generator=g).bfloat16().float()
+    q = torch.randn(n, nq, d, generator=g).bfloat16().float()
+    kc = torch.zeros(pages, nkv, Pg, d, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(pages, nkv, d, Pg, dtype=torch.bfloat16, device=DEV)
+    need = -(-N // Pg)
+    ids = [pages - 1 - 3 * j if j % 2 else 5 * j for j in range(need)]
+    for j, page in enumerate(ids):
+        m = min(Pg, N - j * Pg)
+        kc[page, :, :m, :] = k[j * Pg:j * Pg + m].transpose(0, 1).to(DEV, torch.bfloat16)
+        vc[page, :, :, :m] = v[j * Pg:j * Pg + m].permute(1, 2, 0).to(DEV, torch.bfloat16)
+    bt = torch.tensor([ids], dtype=torch.int32, device=DEV)
+    cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+    ctxl = torch.tensor([N], dtype=torch.int32, device=DEV)
+    fa = FastAttention(nq, nkv, d)
+    out = fa.prefill(q.reshape(n, nq * d).to(DEV, torch.bfloat16), kc, vc, bt, cu, ctxl, 1, 1.0 / math.sqrt(d))
+    want = P.causal_attention(q, k, v, q_positions=torch.arange(prefix, N))
+    close(out.reshape(n, nq, d), want, torch.bfloat16)
+    del kc, vc
+    torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(4, 1, 16, 16), (6, 3, 32, 8), (5, 5, 48, 16), (3, 1, 80, 32), (8, 2, 256, 64),
