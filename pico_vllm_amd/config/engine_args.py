@@ -6,7 +6,8 @@ uses 500 blocks of 16), ``max_seq_len`` (engine.py:41), ``max_num_seqs``
 (scheduler.py:84), ``use_cuda_graph`` and ``max_batch_size`` (engine.py:21-22;
 the graph here is a HIP graph), ``manual_seed`` (engine.py:30).
 ``max_num_batched_tokens`` (the token budget of a step; the reference prefills
-whole prompts, engine.py:305-306) and ``dtype`` have no counterpart there.
+whole prompts, engine.py:305-306), ``dtype`` and ``pipeline_decode`` (start the next decode
+step from the tokens on the device before the host has read them) have no counterpart there.
 """
 from __future__ import annotations
 
@@ -26,6 +27,7 @@ class EngineArgs:
     use_cuda_graph: bool = True          # replay pure-decode steps from a captured HIP graph
     max_batch_size: int = 8              # largest decode batch that has a graph
     manual_seed: int = 42
+    pipeline_decode: bool = True         # keep one decode step in flight while the host prepares the next
     device: str = "cuda:0"
 
     def validate(self) -> None:

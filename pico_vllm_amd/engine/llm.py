@@ -33,6 +33,12 @@ class RequestOutput:
     num_preemptions: int = 0
 
 
+@dataclass
+class _Inflight:
+    sampling: list          # the ScheduledSeq that get a token from this step, in the order of the sampled rows
+    ticket: tuple           # what Sampler.read wants
+
+
 class LLMEngine:
     def __init__(self, args: EngineArgs, model: Optional[DecoderModel] = None, tokenizer=None):
         args.validate()
@@ -54,6 +60,7 @@ class LLMEngine:
         self._next_id = 0
         self.requests: Dict[int, Request] = {}
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+        self._inflight: Optional[_Inflight] = None      # a launched step whose tokens have not been read
 
     # ---- the reference's trio -------------------------------------------
     def submit(self, prompt: Union[str, Sequence[int]], max_new_tokens: int = 16, temperature: float = 0.0,
@@ -73,45 +80,101 @@ class LLMEngine:
         return rid
 
     def step(self) -> List[RequestOutput]:
-        """One scheduling decision and one model step; returns the requests that finished in it."""
-        plan = self.scheduler.schedule()
+        """One scheduling decision and one model step; returns the requests found finished.
+
+        With ``pipeline_decode`` a step whose successor can be foreseen (every running request
+        decodes on, nobody waits, nobody reaches its length) stays in flight: the next call starts
+        that successor from the tokens on the device and only then reads this step's tokens, so
+        the GPU does not wait for the host between decode steps.  The tokens of a step in flight
+        are reported by the call that reads them; what is generated does not change."""
+        prev, self._inflight = self._inflight, None
+        done: List[RequestOutput] = []
+        plan = None
+        if prev is not None:
+            if self._foreseeable(prev):
+                plan = self.scheduler.schedule()
+                if not plan.preempted and [s.request for s in plan.seqs] == [s.request for s in prev.sampling] \
+                        and all(s.num_tokens == 1 for s in plan.seqs):
+                    nxt = self._launch(plan, from_device=True)
+                    done = self._resolve(prev)
+                    self._inflight = nxt
+                    return done
+            # not foreseeable after all (pages ran out): the tokens first, then what is left of the plan
+            done = self._resolve(prev)
+            if plan is not None:
+                plan.seqs = [s for s in plan.seqs if s.request.status is RequestStatus.RUNNING]
+        if plan is None:
+            plan = self.scheduler.schedule()
         self.stats["preemptions"] += len(plan.preempted)
         if not plan.seqs:
             if self.scheduler.has_unfinished():
                 raise RuntimeError("the scheduler found nothing to run although requests are unfinished")
-            return []
+            return done
+        launched = self._launch(plan)
+        if self.args.pipeline_decode and self._foreseeable(launched):
+            self._inflight = launched
+        else:
+            done += self._resolve(launched)
+        return done
+
+    def is_done(self) -> bool:
+        return self._inflight is None and not self.scheduler.has_unfinished()
+
+    # ---- a step in two halves -------------------------------------------
+    def _foreseeable(self, step: "_Inflight") -> bool:
+        """Whether the step after ``step`` is known before its tokens are: every running request
+        got a token in it and goes on decoding, nobody waits for admission, and nobody reaches
+        its length with that token (an end-of-sequence token cannot be foreseen: the request
+        then simply drops the one token computed too many)."""
+        if not self.args.pipeline_decode or self.scheduler.waiting:
+            return False
+        if [s.request for s in step.sampling] != self.scheduler.running:
+            return False
+        return all(r.num_generated < r.params.max_new_tokens and r.total_len < self.args.max_seq_len
+                   for r in self.scheduler.running)
+
+    def _launch(self, plan, from_device: bool = False) -> "_Inflight":
+        """Start the model step and the sampling of ``plan`` and advance what does not depend on the
+        values of the new tokens."""
         seqs = []
         for s in plan.seqs:
             r = s.request
-            toks = r.all_ids[r.num_computed:r.num_computed + s.num_tokens]
+            toks = [0] if from_device else r.all_ids[r.num_computed:r.num_computed + s.num_tokens]
             seqs.append(SeqStep(r.request_id, toks, [s.num_tokens - 1] if s.samples else []))
-        logits = self.runner.step(seqs)
+        logits = self.runner.step(seqs, self.sampler.device_tokens if from_device else None)
         sampling = [s for s in plan.seqs if s.samples]
-        new_tokens = self.sampler.sample(
+        ticket = self.sampler.launch(
             logits,
             [s.request.params.temperature for s in sampling], [s.request.params.top_p for s in sampling],
-            [s.request.seed for s in sampling], [len(s.request.generated_ids) for s in sampling])
-        done: List[RequestOutput] = []
+            [s.request.seed for s in sampling], [s.request.num_generated for s in sampling])
         for s in plan.seqs:
+            self.stats["decode_tokens" if s.num_tokens == 1 and s.request.num_generated else "prefill_tokens"] += s.num_tokens
             self.scheduler.on_step_done(s)
-            self.stats["decode_tokens" if s.num_tokens == 1 and s.request.generated_ids else "prefill_tokens"] += s.num_tokens
-        for s, tok in zip(sampling, new_tokens):
+        for s in sampling:
+            s.request.num_pending += 1
+        self.stats["steps"] += 1
+        return _Inflight(sampling, ticket)
+
+    def _resolve(self, step: "_Inflight") -> List[RequestOutput]:
+        """Read the tokens of a launched step and finish what they finish."""
+        done: List[RequestOutput] = []
+        for s, tok in zip(step.sampling, self.sampler.read(step.ticket)):
             r = s.request
+            if r.status is RequestStatus.FINISHED:      # ended by the token before this one: computed too many
+                continue
+            r.num_pending -= 1
             r.generated_ids.append(int(tok))
             reason = None
             # the end-of-sequence token is kept in the output (pico_vllm/engine.py:380-385)
             if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
                 reason = "eos"
-            elif r.is_max_len_finished():
+            elif len(r.generated_ids) >= r.params.max_new_tokens:    # the first sampled token counts (pico_vllm/scheduler.py:55-56)
                 reason = "length"
             if reason:
+                r.num_pending = 0
                 self.scheduler.finish(r, reason)
                 done.append(self._output(r))
-        self.stats["steps"] += 1
         return done
-
-    def is_done(self) -> bool:
-        return not self.scheduler.has_unfinished()
 
     # ---- helpers --------------------------------------------------------
     def _encode(self, prompt) -> List[int]:

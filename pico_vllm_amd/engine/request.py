@@ -32,6 +32,7 @@ class Request:
     finish_reason: Optional[str] = None       # "eos" or "length"
     num_computed: int = 0                     # tokens whose keys are in the cache
     num_preemptions: int = 0
+    num_pending: int = 0                      # tokens sampled on the device whose values the host has not read yet (up to 2)
 
     @property
     def all_ids(self) -> List[int]:
@@ -39,7 +40,11 @@ class Request:
 
     @property
     def total_len(self) -> int:
-        return len(self.input_ids) + len(self.generated_ids)
+        return len(self.input_ids) + len(self.generated_ids) + self.num_pending
+
+    @property
+    def num_generated(self) -> int:
+        return len(self.generated_ids) + self.num_pending
 
     @property
     def num_uncomputed(self) -> int:
@@ -48,4 +53,4 @@ class Request:
 
     def is_max_len_finished(self) -> bool:
         # the first sampled token counts (pico_vllm/scheduler.py:55-56)
-        return len(self.generated_ids) >= self.params.max_new_tokens
+        return self.num_generated >= self.params.max_new_tokens

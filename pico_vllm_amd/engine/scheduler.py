@@ -133,7 +133,10 @@ class Scheduler:
     def finish(self, req: Request, reason: str) -> None:
         """The request is done: its pages and state slot go back in this same step
         (the reference releases one step later, pico_vllm/engine.py:426-428)."""
-        self.manager.free_request(req.request_id)
-        self.running.remove(req)
+        if req in self.running:
+            self.manager.free_request(req.request_id)
+            self.running.remove(req)
+        else:                      # preempted while its last token was still on the device: it holds nothing
+            self.waiting.remove(req)
         req.status = RequestStatus.FINISHED
         req.finish_reason = reason

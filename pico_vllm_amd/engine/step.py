@@ -39,7 +39,9 @@ class ModelRunner:
         self.storage = CacheStorage(self.manager, specs, model.dtype, self.device)
         self.max_pages = -(-max_seq_len // page_size)
         self.max_seq_len = max_seq_len
-        self.buffers = BatchBuffers(self.device, max_tokens_per_step, max_seqs, self.max_pages,
+        # a decode batch is padded to the power of two its graph was captured at: rows for that too
+        rows = max(max_seqs, _bucket(min(max_seqs, max_graph_batch))) if use_graph else max_seqs
+        self.buffers = BatchBuffers(self.device, max(max_tokens_per_step, rows), rows, self.max_pages,
                                     max(1, len(self.manager.groups)))
         self.use_graph = use_graph
         self.max_graph_batch = max_graph_batch
@@ -48,19 +50,26 @@ class ModelRunner:
         self.tokens = 0
 
     # ---- one step -------------------------------------------------------
-    def step(self, seqs: List[SeqStep]) -> torch.Tensor:
+    def step(self, seqs: List[SeqStep], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Logits float32 [wanted, vocab] in the order of ``seqs`` and their ``want``.
 
         Pages for the new tokens must have been allocated (``manager.grow``);
-        afterwards the caller records the new lengths (``manager.advance``)."""
+        afterwards the caller records the new lengths (``manager.advance``).
+        ``device_tokens``: for a step of single tokens, int32 on the device whose entry b is the
+        token of sequence b; it replaces the (then meaningless) token ids of ``seqs``, so that
+        a decode step can start before the host knows the tokens the step before it sampled."""
+        if device_tokens is not None and any(len(s.tokens) != 1 for s in seqs):
+            raise BatchError("tokens from the device stand for single-token sequences only")
         for s in seqs:
             if self.manager.num_computed(s.req) + len(s.tokens) > self.max_seq_len:
                 raise BatchError(f"request {s.req!r} would grow beyond max_seq_len={self.max_seq_len}")
         decode_only = all(len(s.tokens) == 1 and list(s.want) == [0] for s in seqs)
         if self.use_graph and decode_only and len(seqs) <= self.max_graph_batch:
-            logits = self._step_graph(seqs)
+            logits = self._step_graph(seqs, device_tokens)
         else:
             ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size)
+            if device_tokens is not None:
+                ctx.token_ids[:len(seqs)].copy_(device_tokens[:len(seqs)])
             logits = self.model.forward(ctx, self.storage)
         self.steps += 1
         self.tokens += sum(len(s.tokens) for s in seqs)
@@ -71,13 +80,15 @@ class ModelRunner:
             self.manager.advance(s.req, self.manager.num_computed(s.req) + len(s.tokens))
 
     # ---- graph replay of decode steps -----------------------------------
-    def _step_graph(self, seqs: List[SeqStep]) -> torch.Tensor:
+    def _step_graph(self, seqs: List[SeqStep], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         B = len(seqs)
         size = _bucket(B)
         if size not in self._graphs:
             self._capture(size, seqs)
         graph, out = self._graphs[size]
-        build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size, pad_to=size)
+        ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size, pad_to=size)
+        if device_tokens is not None:
+            ctx.token_ids[:B].copy_(device_tokens[:B])
         graph.replay()
         return out[:B]
 

@@ -132,7 +132,7 @@ def test_submit_step_is_done_in_the_reference_manner():
     from pico_vllm_amd import EngineArgs
     from pico_vllm_amd.engine.llm import LLMEngine
     eng = LLMEngine(EngineArgs(model=model_dir("A"), dtype="float32", num_gpu_blocks=32, max_seq_len=128,
-                               use_cuda_graph=False))
+                               use_cuda_graph=False, pipeline_decode=False))
     a = eng.submit([1, 2, 3], max_new_tokens=1, temperature=0, top_p=1.0)
     b = eng.submit([4, 5, 6, 7], max_new_tokens=3, temperature=0, top_p=1.0, ignore_eos=True)
     done = []
@@ -147,3 +147,45 @@ def test_submit_step_is_done_in_the_reference_manner():
         eng.submit([1] * 200, max_new_tokens=10)
     with pytest.raises(ValueError):
         eng.submit([999], max_new_tokens=1)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graph", [False, True])
+def test_a_decode_step_in_flight_changes_nothing(dtype, graph):
+    # with pipeline_decode the next decode step starts from the tokens on the device before the host has
+    # read them; requests end by length and by the end-of-sequence token at different steps, one is
+    # sampled with a temperature, and pages are so few that requests are preempted
+    from pico_vllm_amd import SamplingParams
+    name = "B"
+    eos = CONFIGS[name]["eos_token_id"]
+    g = torch.Generator().manual_seed(8)
+    V = CONFIGS[name]["vocab_size"]
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (9, 30, 17, 5, 41)]
+    sps = [SamplingParams(max_new_tokens=n, temperature=t, top_p=p, seed=3, ignore_eos=ig)
+           for n, t, p, ig in ((25, 0.0, 1.0, False), (7, 0.0, 1.0, True), (40, 0.9, 0.8, False), (1, 0.0, 1.0, True),
+                               (33, 0.0, 1.0, False))]
+    outs = {}
+    for pipe in (False, True):
+        for blocks in (64, 14):
+            eng = llm(name, dtype, num_gpu_blocks=blocks, max_num_seqs=3, use_cuda_graph=graph, max_batch_size=4,
+                      pipeline_decode=pipe)
+            outs[pipe, blocks] = eng.generate(prompts, sps)
+            eng.engine.runner.manager.check()
+            assert eng.engine._inflight is None
+            assert eng.engine.runner.manager.groups[0].pool.num_free == blocks
+    base = outs[False, 64]
+    for o, sp in zip(base, sps):
+        assert 1 <= len(o.token_ids) <= sp.max_new_tokens
+        assert (o.finish_reason == "eos") == (not sp.ignore_eos and o.token_ids[-1] == eos)
+    if dtype == "float32":       # float32 logits do not depend on the batch, so neither do the tokens
+        for key, got in outs.items():
+            assert [(o.token_ids, o.finish_reason) for o in got] == [(o.token_ids, o.finish_reason) for o in base], key
+    else:                        # bfloat16: rounding depends on the batch; every greedy token is the plain argmax within rounding
+        greedy = [i for i, sp in enumerate(sps) if sp.temperature == 0.0]
+        for got in outs.values():
+            check_greedy(name, dtype, [prompts[i] for i in greedy], [got[i] for i in greedy])
+            for o, sp in zip(got, sps):
+                assert 1 <= len(o.token_ids) <= sp.max_new_tokens
+                assert (o.finish_reason == "eos") == (not sp.ignore_eos and o.token_ids[-1] == eos)
+    assert any(o.num_preemptions for o in outs[True, 14])
+
