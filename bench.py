@@ -27,20 +27,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12            # bytes/s, MI355X HBM3E
 MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# BASELINE.json configs[2]: Qwen2.5-1.5B
-CONFIG_1P5B = {
-    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
-    "vocab_size": 151936, "hidden_size": 1536, "num_hidden_layers": 28, "num_attention_heads": 12,
-    "num_key_value_heads": 2, "intermediate_size": 8960, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
-    "tie_word_embeddings": True, "max_position_embeddings": 131072, "hidden_act": "silu",
-}
-# BASELINE.json configs[3]: Qwen2.5-7B (measured with fewer layers when asked: --layers)
-CONFIG_7B = {
-    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
-    "vocab_size": 152064, "hidden_size": 3584, "num_hidden_layers": 28, "num_attention_heads": 28,
-    "num_key_value_heads": 4, "intermediate_size": 18944, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
-    "tie_word_embeddings": False, "max_position_embeddings": 131072, "hidden_act": "silu",
-}
+from pico_vllm_amd.config.presets import preset   # noqa: E402  (needs ROOT on the path)
+
+CONFIG_1P5B = preset("1.5b")       # BASELINE.json configs[2]: Qwen2.5-1.5B
+CONFIG_7B = preset("7b")           # BASELINE.json configs[3]: Qwen2.5-7B (measured with fewer layers when asked: --layers)
 SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", CONFIG_1P5B), "7b": ("Qwen2.5-7B shape", CONFIG_7B)}
 CONFIG = CONFIG_1P5B         # the shape being measured (set in main)
 CONTEXT = 4096

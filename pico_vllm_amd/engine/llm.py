@@ -64,9 +64,10 @@ class LLMEngine:
 
     # ---- the reference's trio -------------------------------------------
     def submit(self, prompt: Union[str, Sequence[int]], max_new_tokens: int = 16, temperature: float = 0.0,
-               top_p: float = 1.0, seed: Optional[int] = None, ignore_eos: bool = False) -> int:
+               top_p: float = 1.0, seed: Optional[int] = None, ignore_eos: bool = False,
+               stop_token_ids: Sequence[int] = ()) -> int:
         """Queue a request; returns its id (pico_vllm/engine.py:243-276)."""
-        params = SamplingParams(max_new_tokens, temperature, top_p, seed, ignore_eos)
+        params = SamplingParams(max_new_tokens, temperature, top_p, seed, ignore_eos, [int(t) for t in stop_token_ids])
         params.validate()
         ids = self._encode(prompt)
         V = self.model.spec.vocab_size
@@ -168,6 +169,8 @@ class LLMEngine:
             # the end-of-sequence token is kept in the output (pico_vllm/engine.py:380-385)
             if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
                 reason = "eos"
+            elif tok in r.params.stop_token_ids:
+                reason = "stop"
             elif len(r.generated_ids) >= r.params.max_new_tokens:    # the first sampled token counts (pico_vllm/scheduler.py:55-56)
                 reason = "length"
             if reason:
@@ -209,7 +212,7 @@ class LLM:
             sampling_params = [sampling_params] * len(prompts)
         if len(sampling_params) != len(prompts):
             raise ValueError("one SamplingParams per prompt, or one for all")
-        ids = [self.engine.submit(p, sp.max_new_tokens, sp.temperature, sp.top_p, sp.seed, sp.ignore_eos)
+        ids = [self.engine.submit(p, sp.max_new_tokens, sp.temperature, sp.top_p, sp.seed, sp.ignore_eos, sp.stop_token_ids)
                for p, sp in zip(prompts, sampling_params)]
         outs: Dict[int, RequestOutput] = {}
         while not self.engine.is_done():

@@ -6,12 +6,15 @@ names: --num-gpu-blocks 500 --block-size 16 (run_single.py:17-22),
   python -m pico_vllm_amd.run --model DIR --prompt-ids 1,2,3 --max-new-tokens 20
   python -m pico_vllm_amd.run --model DIR --prompt "The capital of France is"
   python -m pico_vllm_amd.run --write-random DIR --config config.json --seed 0
+  python -m pico_vllm_amd.run --random-config tiny-b --prompt-ids 5,17,3     (random weights of a named size)
 """
 from __future__ import annotations
 
 import argparse
 import json
+import shutil
 import sys
+import tempfile
 
 
 def main(argv=None) -> int:
@@ -37,19 +40,42 @@ def main(argv=None) -> int:
     ap.add_argument("--manual-seed", type=int, default=42)
     ap.add_argument("--write-random", metavar="DIR", help="write a random-weights model folder and exit")
     ap.add_argument("--config", help="config.json to use with --write-random")
+    ap.add_argument("--random-config", metavar="NAME", help="run on random weights of a named size "
+                    "(tiny-a, tiny-b, 1.5b, 7b, 32b) instead of --model; with --write-random: that size")
+    ap.add_argument("--no-pipeline-decode", dest="pipeline_decode", action="store_false", default=True,
+                    help="read every step's tokens before the next step starts")
     args = ap.parse_args(argv)
 
     if args.write_random:
-        if not args.config:
-            ap.error("--write-random needs --config")
+        if not (args.config or args.random_config):
+            ap.error("--write-random needs --config or --random-config")
+        from .config.presets import preset
         from .weights.random_init import write_random_model
-        with open(args.config) as f:
-            cfg = json.load(f)
+        if args.config:
+            with open(args.config) as f:
+                cfg = json.load(f)
+        else:
+            cfg = preset(args.random_config)
         write_random_model(args.write_random, cfg, args.seed or 0)
         print(f"wrote {args.write_random}")
         return 0
+    tmp = None
+    if args.random_config and not args.model:
+        from .config.presets import preset
+        from .weights.random_init import write_random_model
+        tmp = tempfile.mkdtemp(prefix="pico_random_")
+        write_random_model(tmp, preset(args.random_config), args.seed or 0)
+        args.model = tmp
     if not args.model:
-        ap.error("--model is required")
+        ap.error("--model or --random-config is required")
+    try:
+        return _generate(ap, args)
+    finally:
+        if tmp:
+            shutil.rmtree(tmp, ignore_errors=True)
+
+
+def _generate(ap, args) -> int:
     prompts = list(args.prompt) + [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     if not prompts:
         ap.error("give at least one --prompt or --prompt-ids")
@@ -69,7 +95,7 @@ def main(argv=None) -> int:
                     num_gpu_blocks=args.num_gpu_blocks, max_seq_len=args.max_seq_len,
                     max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
                     use_cuda_graph=args.use_cuda_graph, max_batch_size=args.max_batch_size,
-                    manual_seed=args.manual_seed)
+                    manual_seed=args.manual_seed, pipeline_decode=args.pipeline_decode)
     llm = LLM(tokenizer=tokenizer, engine_args=ea)
     sp = SamplingParams(args.max_new_tokens, args.temperature, args.top_p, args.seed, args.ignore_eos)
     for o in llm.generate(prompts, sp):

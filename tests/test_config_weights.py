@@ -182,3 +182,19 @@ def test_truncated_and_empty_folders(tmp_path):
     (tmp_path / "model.safetensors").write_bytes(data[:len(data) // 2])
     with pytest.raises(WeightsError, match="truncated"):
         load_checkpoint(str(tmp_path), _specs("A"), torch.bfloat16)
+
+
+def test_named_configurations_parse_and_the_tiny_ones_differ_in_every_size():
+    from pico_vllm_amd.config.model_config import Qwen2Config
+    from pico_vllm_amd.config.presets import PRESETS, preset
+    cfgs = {n: Qwen2Config.from_dict(preset(n)) for n in PRESETS}
+    a, b = cfgs["tiny-a"], cfgs["tiny-b"]
+    for f in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads", "num_key_value_heads", "head_dim",
+              "intermediate_size", "rms_norm_eps", "rope_theta", "tie_word_embeddings"):
+        assert getattr(a, f) != getattr(b, f), f
+    big = cfgs["1.5b"]
+    assert (big.hidden_size, big.num_attention_heads, big.num_key_value_heads, big.head_dim, big.vocab_size) == \
+        (1536, 12, 2, 128, 151936)
+    with pytest.raises(ValueError):
+        preset("3b")
+

@@ -189,3 +189,22 @@ def test_a_decode_step_in_flight_changes_nothing(dtype, graph):
                 assert (o.finish_reason == "eos") == (not sp.ignore_eos and o.token_ids[-1] == eos)
     assert any(o.num_preemptions for o in outs[True, 14])
 
+
+def test_stop_tokens_end_a_request_like_the_end_of_sequence_token():
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("A", [12], seed=6)
+    base = llm("A", "float32").generate(prompts, SamplingParams(max_new_tokens=12, temperature=0.0, ignore_eos=True))[0]
+    stop = base.token_ids[4]
+    first = base.token_ids.index(stop)
+    out = llm("A", "float32").generate(prompts, SamplingParams(max_new_tokens=12, temperature=0.0, ignore_eos=True,
+                                                               stop_token_ids=[stop]))[0]
+    assert out.finish_reason == "stop" and out.token_ids == base.token_ids[:first + 1]     # the stop token is kept
+
+
+def test_command_line_on_random_weights_of_a_named_size(capsys):
+    from pico_vllm_amd import run
+    assert run.main(["--random-config", "tiny-a", "--prompt-ids", "5,17,3", "--prompt-ids", "9", "--max-new-tokens", "6",
+                     "--ignore-eos", "--dtype", "float32", "--num-gpu-blocks", "16", "--max-seq-len", "64"]) == 0
+    lines = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")]
+    assert len(lines) == 2 and all("(length)" in l and len(l.split(")")[1].split()) == 6 for l in lines)
+
