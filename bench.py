@@ -3,6 +3,9 @@
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
   python bench.py --shape 7b --layers 8 --context 8192      (other sizes and context lengths)
+  python bench.py --workload serve --shape 7b --layers 8 --context 8192
+                                                            (64 requests, prompts of 128..4096 tokens, 256 new tokens each,
+                                                             continuous batching with prompts cut into portions)
 
 A step is one decode step of the engine (scheduler, model step from a HIP graph, sampling) at
 batch 8 with every request's context ending at 4096 tokens.  One JSON line goes to stdout:
@@ -126,6 +129,44 @@ def prefill_point(model_dir, model, dtype, reps=3):
             "frac": prefill_flops(CONFIG, PREFILL_TOKENS) / dt / MFMA_PEAK[dtype]}
 
 
+def serve_point(model_dir, dtype, requests, max_new):
+    """BASELINE.json's mixed workload: `requests` requests with prompt lengths uniform in 128..4096 (seeded) and
+    `max_new` new tokens each, all submitted at once; the scheduler admits, cuts prompts into portions of at most
+    2,048 tokens beside the decoding requests, decodes, finishes and frees."""
+    import torch
+    from pico_vllm_amd import EngineArgs
+    from pico_vllm_amd.engine.llm import LLMEngine
+    g = torch.Generator().manual_seed(requests)
+    lens = torch.randint(128, 4097, (requests,), generator=g).tolist()
+    block = 16
+    longest = max(lens) + max_new
+    if longest > CONTEXT:
+        raise SystemExit(f"bench.py: --context must be at least {longest} for this workload")
+    pages = sum(-(-(n + max_new) // block) for n in lens) + 8
+    eng = LLMEngine(EngineArgs(model=model_dir, dtype=dtype, block_size=block, num_gpu_blocks=pages, max_seq_len=CONTEXT,
+                               max_num_seqs=requests, max_num_batched_tokens=PREFILL_TOKENS, use_cuda_graph=True,
+                               max_batch_size=64))
+    V = CONFIG["vocab_size"]
+    # a short run first: kernels built and tuned, graphs captured for the batch sizes of the run's tail
+    for n in (PREFILL_TOKENS, 300):
+        eng.submit(torch.randint(0, V, (n,), generator=g).tolist(), max_new_tokens=4, ignore_eos=True)
+    while not eng.is_done():
+        eng.step()
+    torch.cuda.synchronize()
+    for n in lens:
+        eng.submit(torch.randint(0, V, (n,), generator=g).tolist(), max_new_tokens=max_new, temperature=0.0, ignore_eos=True)
+    steps0 = eng.stats["steps"]
+    t0 = time.perf_counter()
+    finished = 0
+    while not eng.is_done():
+        finished += len(eng.step())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert finished == requests
+    return {"seconds": dt, "steps": eng.stats["steps"] - steps0, "prompt_tokens": sum(lens), "new_tokens": requests * max_new,
+            "preemptions": eng.stats["preemptions"]}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,6 +182,10 @@ def main() -> int:
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
     ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve"],
+                    help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once")
+    ap.add_argument("--requests", type=int, default=64, help="requests of the serve workload")
+    ap.add_argument("--max-new", type=int, default=256, help="new tokens per request of the serve workload")
     a = ap.parse_args()
     global CONFIG, CONTEXT
     shape_name, full = SHAPES[a.shape]
@@ -173,6 +218,22 @@ def main() -> int:
         write_random_model(model_dir, CONFIG, seed=0)
         log(f"... {time.time() - t0:.0f}s")
     try:
+        if a.workload == "serve":
+            r = serve_point(model_dir, a.dtype, a.requests, a.max_new)
+            total = r["prompt_tokens"] + r["new_tokens"]
+            print(json.dumps({
+                "metric": f"tokens/s (prompt + new) serving {a.requests} requests at once, {shape_name.split()[0]} bf16",
+                "value": round(total / r["seconds"], 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+                "new_tokens_per_s": round(r["new_tokens"] / r["seconds"], 1), "seconds": round(r["seconds"], 3),
+                "steps": r["steps"], "ms_per_step": round(r["seconds"] / r["steps"] * 1e3, 4),
+                "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+                "data": "synthetic: random weights N(0, 0.02), uniform random token ids, prompt lengths uniform in 128..4096",
+                "config": {"model": shape_name, "requests": a.requests, "new_tokens_each": a.max_new,
+                           "prompt_tokens": r["prompt_tokens"], "layers": full["num_hidden_layers"],
+                           "layers_run": CONFIG["num_hidden_layers"], "hidden": CONFIG["hidden_size"],
+                           "max_num_batched_tokens": PREFILL_TOKENS, "max_seq_len": CONTEXT, "page_size": 16,
+                           "preemptions": r["preemptions"]}}), flush=True)
+            return 0
         if a.prefill_only:
             print(json.dumps({"prefill": prefill_point(model_dir, None, a.dtype)}), flush=True)
             return 0
