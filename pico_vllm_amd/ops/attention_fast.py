@@ -97,15 +97,30 @@ class FastAttention:
                 raise KernelError("sequence metadata must be contiguous int32")
 
     def __call__(self, qkv, cache, block_table, ctx, scale):
-        if ctx.all_decode and self.nq // self.nkv <= 32:
-            return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, ctx.num_seqs, scale,
-                               self.num_splits(ctx.num_seqs, ctx.max_context))
-        teams = 0
+        B = ctx.num_seqs
+        grouped = self.nq // self.nkv <= 32
+        if ctx.all_decode and grouped:
+            return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, B, scale,
+                               self.num_splits(B, ctx.max_context))
+        teams, lead = 0, 0
         if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
             cu = ctx.host["cu_seqlens"]
-            teams = self.prefill_teams(cu[1:ctx.num_seqs + 1] - cu[:ctx.num_seqs], ctx.host["context_lens"][:ctx.num_seqs])
-        return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, ctx.num_seqs, scale,
-                            teams=teams)
+            lens = cu[1:B + 1] - cu[:B]
+            while lead < B and lens[lead] == 1:
+                lead += 1
+            teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
+        if lead == 0 or not grouped:
+            return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, scale, teams=teams)
+        # A mixed step: the scheduler puts the decoding requests first.  Their tokens (one row each, rows
+        # 0 .. lead - 1) go through the decode kernel, which reads keys and values once for all query heads of
+        # a group; the prompt portions behind them through the prefill kernel, whose offsets are absolute.
+        out = torch.empty(qkv.shape[0], self.nq * self.d, dtype=torch.bfloat16, device=qkv.device)
+        self.decode(qkv[:lead], cache.k, cache.v, block_table[:lead], ctx.context_lens[:lead], lead, scale,
+                    self.num_splits(lead, ctx.max_context), out=out[:lead])
+        if lead < B:
+            self.prefill(qkv, cache.k, cache.v, block_table[lead:], ctx.cu_seqlens[lead:], ctx.context_lens[lead:],
+                         B - lead, scale, out=out, teams=teams)
+        return out
 
 
 def choose(nq: int, nkv: int, head_dim: int, window: int) -> Optional[FastAttention]:

@@ -283,7 +283,7 @@ def test_sampling_top_p(K):
 
 
 # ---- matrix-core attention (bfloat16) ----------------------------------------------------------
-def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0):
+def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0, as_step=False):
     from pico_vllm_amd.ops.attention_fast import FastAttention
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(seed)
@@ -304,7 +304,12 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
     wide[:, :nq * d] = torch.cat(qs, 0).reshape(T, nq * d).to(DEV, dtype)
     fa = FastAttention(nq, nkv, d)
     scale = 1.0 / math.sqrt(d)
-    if decode:
+    if as_step:          # the way the attention part calls it: the kernels are chosen from the shape of the batch
+        from types import SimpleNamespace
+        step = SimpleNamespace(num_seqs=B, all_decode=max(new_lens) == 1, max_context=max(totals), cu_seqlens=cu,
+                               context_lens=ctxl, host={"cu_seqlens": cu.cpu().numpy(), "context_lens": ctxl.cpu().numpy()})
+        out = fa(wide, SimpleNamespace(k=kc, v=vc), bt, step, scale)
+    elif decode:
         out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
     else:
         out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale, teams=teams)
@@ -334,6 +339,16 @@ def test_fast_prefill_with_one_and_two_key_teams(K, nq, nkv, d, Pg, teams):
     # the number of waves that share a query tile's key loop is a hint: every value gives the same attention;
     # lengths around the 64-query tile and the 64- and 128-key tiles of one and two teams
     out, want = _fast_case([63, 1, 65, 130, 2, 200], [0, 127, 1, 62, 191, 129], nq, nkv, d, Pg, seed=5, teams=teams)
+    close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(12, 2, 128, 16), (6, 3, 32, 8), (5, 5, 48, 16), (4, 1, 16, 16)])
+@pytest.mark.parametrize("new_lens,prefix_lens", [([1, 1, 1, 70, 2, 1], [300, 17, 64, 33, 129, 5]),     # decode rows first, as the scheduler orders them
+                                                  ([1, 1, 1, 1], [300, 17, 64, 0]),                      # decode only
+                                                  ([1, 40], [1000, 0]), ([9, 1, 1], [0, 20, 30])])      # no decode row in front
+def test_fast_attention_of_a_mixed_step(K, nq, nkv, d, Pg, new_lens, prefix_lens):
+    # leading single-token sequences go through the decode kernel, the rest through the prefill kernel
+    out, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=9, as_step=True)
     close(out, want, torch.bfloat16)
 
 
