@@ -1,0 +1,82 @@
+"""The kernels at the sizes of a real model: two layers of the Qwen2.5-1.5B shape with random weights.
+
+The tiny configurations of the other tests never reach the paths that only large sizes take (two key
+teams over a 2,048-token triangle, the 8960-wide contraction cut into seven ranges, a vocabulary of
+151,936, the library's matrix products for many rows).  The plain implementation on the CPU is too
+slow here, so the yardstick is the engine's own true 32-bit path, which the other tests pin to the
+plain implementation; the bfloat16 engine must follow it within bfloat16 rounding, whole, in
+portions, and token by token.
+"""
+import os
+import random
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": 151936, "hidden_size": 1536,
+    "num_hidden_layers": 2, "num_attention_heads": 12, "num_key_value_heads": 2, "intermediate_size": 8960,
+    "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "tie_word_embeddings": True, "max_position_embeddings": 32768,
+    "hidden_act": "silu",
+}
+N = 2300          # prompt: more than one 2,048-token portion
+
+
+@pytest.fixture(scope="module")
+def folder():
+    from pico_vllm_amd.weights.random_init import write_random_model
+    with tempfile.TemporaryDirectory(prefix="pico_large_") as d:
+        # queries and keys strong enough that attention is not uniform: a wrong key shows
+        write_random_model(d, SHAPE, 3, {"q_proj.weight": (3.0 / 1536) ** 0.5, "k_proj.weight": (3.0 / 1536) ** 0.5})
+        yield d
+
+
+def replay(folder, dtype, steps):
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    rep = TraceReplayer(folder, dtype, max_tokens=2 * 64 * (-(-N // 64)))
+    out = {}
+    for s in steps:
+        got = rep.run_step(s)
+        if got is not None:
+            out[s["step"]] = got
+    del rep
+    torch.cuda.empty_cache()
+    return out
+
+
+def test_bfloat16_follows_the_32_bit_path_at_the_1_5b_shape(folder):
+    rng = random.Random(1)
+    toks = [rng.randrange(SHAPE["vocab_size"]) for _ in range(N)]
+    want = [0, 1, 63, 64, 1000, 2047, 2048, N - 33, N - 1]
+    whole = [{"step": 0, "entries": [{"id": "a", "tokens": toks, "want": want}], "end": ["a"]}]
+    ref = replay(folder, "float32", whole)[0]
+    spread = float(ref.std())
+    assert np.isfinite(ref).all() and spread > 0.1
+
+    def check(got, rows, label):
+        err = got - ref[rows]
+        rms = float(np.sqrt((err ** 2).mean())) / spread
+        print(f"[large] {label}: rms error {rms:.2e} of the spread, argmax equal in {int((got.argmax(1) == ref[rows].argmax(1)).sum())}/{len(rows)} rows")
+        # bfloat16 rounding through two layers and the output matrix measures 1.7e-2 .. 2.7e-2 here; a wrong key,
+        # slice or page gives an error of the order of the spread itself
+        assert np.isfinite(got).all() and rms < 5e-2, (label, rms)
+
+    # whole: one step of 2,300 tokens (library GEMMs, two key teams)
+    check(replay(folder, "bfloat16", whole)[0], list(range(len(want))), "whole")
+    # portions of 2,048 + 220 (prefix attention), then the last 32 one by one (skinny GEMMs, decode attention)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:2048], "want": [0, 1, 63, 64, 1000, 2047]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[2048:N - 32], "want": [0]}], "end": []}]
+    for i in range(N - 32, N):
+        steps.append({"step": 2 + i - (N - 32), "entries": [{"id": "a", "tokens": [toks[i]], "want": [0] if i == N - 1 else []}], "end": []})
+    got = replay(folder, "bfloat16", steps)
+    check(got[0], [0, 1, 2, 3, 4, 5], "first portion")
+    check(got[1], [6], "second portion")
+    check(got[2 + 31], [8], "last token after 32 single steps")
+    # the 32-bit path itself: portions and single tokens give what the whole prompt gives
+    got32 = replay(folder, "float32", steps)
+    for key, rows in ((0, [0, 1, 2, 3, 4, 5]), (1, [6]), (2 + 31, [8])):
+        assert float(np.abs(got32[key] - ref[rows]).max()) <= 2e-4 * spread, key
