@@ -274,7 +274,7 @@ extern "C" int pico_swiglu(const void* gu, void* out, int dtype, int T, int I, h
 // slots[t] = page * P + position % P says where token t's key and value go (the host computes it
 // from the block table, as the reference does, pico_vllm/cache.py:143-156); a negative slot means
 // "store nothing" (padding rows of a captured batch).
-// Grid (T, nq + nkv); block 64.
+// Grid T; block 256 (one workgroup per token).
 // ---------------------------------------------------------------------------
 __global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                   float2* __restrict__ cos_sin, int half) {
@@ -302,36 +302,38 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float2* __restrict_
                                   const int* __restrict__ slots,
                                   T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv, int d, int rot,
                                   int P, int num_pages) {
-  const int t = blockIdx.x, head = blockIdx.y;
+  const int t = blockIdx.x;
   T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
   const int half = rot >> 1;
   const float2* cs = cos_sin + (size_t)t * half;
-  if (head < nq) {
-    T* x = row + (size_t)head * d;
-    for (int j = threadIdx.x; j < half; j += blockDim.x) {
-      const float c = cs[j].x, s = cs[j].y;
-      const float a = load_f32(x + j), b = load_f32(x + j + half);
-      store_f32(x + j, a * c - b * s);
-      store_f32(x + j + half, b * c + a * s);
-    }
-    return;
-  }
-  const int g = head - nq;
   const int slot = slots[t];
   const int page = slot / P, off = slot % P;
-  if (slot < 0 || page >= num_pages) return;  // padding row; the host has checked the rest
-  const T* k = row + (size_t)(nq + g) * d;
-  const T* v = row + (size_t)(nq + nkv + g) * d;
-  T* kc = k_cache + (((size_t)page * nkv + g) * P + off) * d;
-  T* vc = v_cache + ((size_t)page * nkv + g) * d * P + off;
-  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+  const bool store = slot >= 0 && page < num_pages;       // not a padding row; the host has checked the rest
+  // one pair (j, j + rot/2) of one q or k head per thread and turn; q is rotated in place, k goes to its page
+  for (int u = threadIdx.x; u < (nq + nkv) * half; u += blockDim.x) {
+    const int head = u / half, j = u - head * half;
+    const T* x = row + (size_t)head * d;
+    T* o;
+    if (head < nq) {
+      o = row + (size_t)head * d;
+    } else {
+      if (!store) continue;
+      o = k_cache + (((size_t)page * nkv + (head - nq)) * P + off) * d;
+    }
     const float c = cs[j].x, s = cs[j].y;
-    const float a = load_f32(k + j), b = load_f32(k + j + half);
-    store_f32(kc + j, a * c - b * s);
-    store_f32(kc + j + half, b * c + a * s);
+    const float a = load_f32(x + j), b = load_f32(x + j + half);
+    store_f32(o + j, a * c - b * s);
+    store_f32(o + j + half, b * c + a * s);
   }
-  for (int j = rot + threadIdx.x; j < d; j += blockDim.x) kc[j] = k[j];
-  for (int j = threadIdx.x; j < d; j += blockDim.x) vc[(size_t)j * P] = v[j];
+  if (!store) return;
+  for (int u = threadIdx.x; u < nkv * (d - rot); u += blockDim.x) {      // what is not rotated of k
+    const int g = u / (d - rot), j = rot + u % (d - rot);
+    k_cache[(((size_t)page * nkv + g) * P + off) * d + j] = row[(size_t)(nq + g) * d + j];
+  }
+  for (int u = threadIdx.x; u < nkv * d; u += blockDim.x) {
+    const int g = u / d, j = u - g * d;
+    v_cache[(((size_t)page * nkv + g) * d + j) * P + off] = row[(size_t)(nq + nkv + g) * d + j];
+  }
 }
 
 extern "C" int pico_rope_kv_store(void* qkv, int dtype, const float* cos_sin, const int* slots,
@@ -341,12 +343,13 @@ extern "C" int pico_rope_kv_store(void* qkv, int dtype, const float* cos_sin, co
   PICO_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "pico_rope_kv_store: rotary size %d does not fit head size %d", rot, d);
   PICO_REQUIRE(rot == 0 || (cos_sin != nullptr && (uintptr_t)cos_sin % 8 == 0), "pico_rope_kv_store: no table of cosines and sines");
   if (T == 0) return 0;
-  dim3 grid(T, nq + nkv);
+  const dim3 grid(T);
+  const int threads = (nq + nkv) * (rot / 2) >= 256 || nkv * d >= 256 ? 256 : 64;
   if (dtype == PICO_DTYPE_F32)
-    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, (const float2*)cos_sin, slots, (float*)k_cache,
+    rope_store_kernel<float><<<grid, threads, 0, stream>>>((float*)qkv, (const float2*)cos_sin, slots, (float*)k_cache,
                                                       (float*)v_cache, nq, nkv, d, rot, P, num_pages);
   else if (dtype == PICO_DTYPE_BF16)
-    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, (const float2*)cos_sin, slots, (bf16_t*)k_cache,
+    rope_store_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)qkv, (const float2*)cos_sin, slots, (bf16_t*)k_cache,
                                                        (bf16_t*)v_cache, nq, nkv, d, rot, P, num_pages);
   else
     PICO_REQUIRE(false, "pico_rope_kv_store: unknown dtype %d", dtype);
