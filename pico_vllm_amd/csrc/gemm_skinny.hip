@@ -93,16 +93,17 @@ __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int 
 constexpr int SK_GROUP = 1024 + 16;
 template <int NX> constexpr int sk_stage_bytes() { return (4 + NX) * SK_GROUP; }
 template <int NX> constexpr int sk_depth() { return NX >= 4 ? 2 : 3; }
-// waves per workgroup: two when a wave holds two blocks of tokens in LDS, so that three workgroups fit a compute unit
-template <int MT, int NX> constexpr int sk_waves() { return (MT == 2 && NX > 0) ? 2 : 4; }
+// waves per workgroup: two when a wave holds two blocks of tokens in LDS and the grid is large, so that
+// three workgroups fit a compute unit; four otherwise (FEW: at most one workgroup per compute unit anyway)
+template <int MT, int NX, bool FEW> constexpr int sk_waves() { return (MT == 2 && NX > 0 && !FEW) ? 2 : 4; }
 // s_waitcnt for "at most n vector memory operations outstanding", nothing else waited for
 constexpr int sk_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
-template <int MT, int NX>
+template <int MT, int NX, bool FEW>
 constexpr int sk_smem_bytes() {
   constexpr int red = 4 * MT * 16 * 64 * 4;
   if (NX == 0) return red;
-  constexpr int stages = sk_depth<NX>() * sk_waves<MT, NX>() * sk_stage_bytes<NX>();
+  constexpr int stages = sk_depth<NX>() * sk_waves<MT, NX, FEW>() * sk_stage_bytes<NX>();
   return stages > red ? stages : red;
 }
 
@@ -211,14 +212,14 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
 }
 
 // The 32 tile rows' sums for this workgroup's tokens, through LDS (NX > 0) or registers (NX == 0).
-template <int MT, bool TAIL, int NX>
+template <int MT, bool TAIL, int NX, bool FEW>
 __device__ __forceinline__ float (*skinny_tile(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
                                                int row_a, int row_b, int n_rows, int m0, int M, int k_begin, int k_end,
                                                char* smem))[MT][16][64] {
   float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
   if constexpr (NX > 0) {
     static_assert(!TAIL && NX <= 4 * MT, "the stream through LDS takes whole slices");
-    skinny_stream_lds<MT, NX, sk_waves<MT, NX>()>(X, ldx, W, ldw, row_a, row_b, n_rows, m0, M, k_begin, k_end, smem);
+    skinny_stream_lds<MT, NX, sk_waves<MT, NX, FEW>()>(X, ldx, W, ldw, row_a, row_b, n_rows, m0, M, k_begin, k_end, smem);
   } else {
     const int col = threadIdx.x & 31;
     const int wrow = col < 16 ? row_a + col : row_b + col - 16;
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
                                                           const float* __restrict__ bias, void* __restrict__ out,
                                                           int ldo, long long slab_stride, int M, int N, int K,
                                                           int k_per_wg) {
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX>()];
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, false>()];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int tile = blockIdx.x;
   const int m0 = blockIdx.z * 32 * MT;
@@ -243,10 +244,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
   const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, false>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
 
   // thread (a, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col`: sum of the 4 sets of slices
-  constexpr int NWV = sk_waves<MT, NX>();
+  constexpr int NWV = sk_waves<MT, NX, false>();
   for (int a = wave; a < 4; a += NWV)
 #pragma unroll
   for (int t = 0; t < MT; t++) {
@@ -321,7 +322,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   // few rows and whole slices: the stream through LDS, with as many 8-token groups as hold tokens
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH3(MT, EPI, TAIL, NX) \
-  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, false>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
 #define LAUNCH(EPI)                                               \
   do {                                                            \
     if (nx == 1) LAUNCH3(1, EPI, false, 1);                       \
@@ -359,7 +360,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
     bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
     bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
     int nq, int nkv, int d, int pshift, int num_pages) {
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX>()];
+  // the grid of this projection is small (one workgroup per 32 of (nq + 2 nkv) d rows): four waves always
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, true>()];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int tiles_per_head = d >> 5, half = d >> 1;
   const int head = blockIdx.x / tiles_per_head, tp = blockIdx.x % tiles_per_head;
@@ -367,9 +369,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
   const bool rotated = head < nq + nkv;
   const int row_a = head * d + (rotated ? 16 * tp : 32 * tp);
   const int row_b = rotated ? row_a + half : row_a + 16;
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX>(X, ldx, W, ldw, row_a, row_b, (nq + 2 * nkv) * d, m0, M, 0, K, smem);
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, true>(X, ldx, W, ldw, row_a, row_b, (nq + 2 * nkv) * d, m0, M, 0, K, smem);
 
-  constexpr int NWV = sk_waves<MT, NX>();
+  constexpr int NWV = sk_waves<MT, NX, true>();
   for (int a = wave; a < 4; a += NWV)
 #pragma unroll
   for (int t = 0; t < MT; t++) {
@@ -450,7 +452,7 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   const bool tail = K % 64 != 0;
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH(MT, TAIL, NX) \
-  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
+  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, true>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
       (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
   if (nx == 1) LAUNCH(1, false, 1);
   else if (nx == 2) LAUNCH(1, false, 2);
