@@ -34,7 +34,8 @@ from pico_vllm_amd.config.presets import preset   # noqa: E402  (needs ROOT on t
 
 CONFIG_1P5B = preset("1.5b")       # BASELINE.json configs[2]: Qwen2.5-1.5B
 CONFIG_7B = preset("7b")           # BASELINE.json configs[3]: Qwen2.5-7B (measured with fewer layers when asked: --layers)
-SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", CONFIG_1P5B), "7b": ("Qwen2.5-7B shape", CONFIG_7B)}
+SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", CONFIG_1P5B), "7b": ("Qwen2.5-7B shape", CONFIG_7B),
+          "32b": ("Qwen2.5-32B shape", preset("32b"))}
 CONFIG = CONFIG_1P5B         # the shape being measured (set in main)
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
