@@ -129,3 +129,50 @@ def test_uniform_numbers_are_a_pure_function_of_seed_and_index():
     a = [uniform(5, i) for i in range(1000)]
     assert a == [uniform(5, i) for i in range(1000)] and a != [uniform(6, i) for i in range(1000)]
     assert all(0.0 <= x < 1.0 for x in a) and 0.45 < sum(a) / 1000 < 0.55
+
+
+def test_a_token_that_the_host_has_not_read_yet_counts_as_a_token():
+    # the decode pipeline starts a step before the tokens of the step before it are known: the request
+    # then carries them as pending; the scheduler plans with them, the values arrive later
+    m, s = make()
+    r = req(0, 5, 4)
+    s.add_request(r)
+    plan = s.schedule()
+    assert plan.seqs[0].num_tokens == 5 and plan.seqs[0].samples
+    s.on_step_done(plan.seqs[0])
+    r.num_pending += 1                                  # sampled on the device, not read
+    assert r.total_len == 6 and r.num_uncomputed == 1 and r.num_generated == 1 and r.all_ids == [1, 2, 3, 4, 5]
+    plan = s.schedule()                                 # the next decode step can be planned already
+    assert [(x.request.request_id, x.num_tokens, x.samples) for x in plan.seqs] == [(0, 1, True)]
+    s.on_step_done(plan.seqs[0])
+    r.num_pending += 1
+    assert r.num_computed == 6 and r.total_len == 7
+    r.num_pending -= 1
+    r.generated_ids.append(11)                          # the first value arrives
+    assert r.total_len == 7 and r.all_ids[-1] == 11 and not r.is_max_len_finished()
+    m.check()
+
+
+def test_a_preempted_request_can_finish_while_it_waits():
+    # its last token was still on the device when it was preempted and turns out to end it
+    m, s = make(num_pages=4, page=16, max_seqs=2, budget=64)
+    a, b = req(0, 30, 30), req(1, 30, 30)
+    s.add_request(a)
+    s.add_request(b)
+    for x in s.schedule().seqs:
+        s.on_step_done(x)
+        x.request.num_pending += 1
+    for _ in range(40):                                 # decode until the pool runs dry and b is preempted
+        plan = s.schedule()
+        if plan.preempted:
+            break
+        for x in plan.seqs:
+            s.on_step_done(x)
+            x.request.num_pending -= 1
+            x.request.generated_ids.append(3)
+            x.request.num_pending += 1
+    assert plan.preempted == [b] and b.status is RequestStatus.WAITING and b.num_pending == 1
+    s.finish(b, "eos")
+    assert b.status is RequestStatus.FINISHED and list(s.waiting) == [] and s.running == [a]
+    m.check()
+
