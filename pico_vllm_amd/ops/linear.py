@@ -45,7 +45,8 @@ def _library_tuning(rows: int) -> None:
             st["ready"] = "off"
     if st["ready"] == "off":
         return
-    want = rows % TUNE_ROWS == 0
+    # never while a graph is being recorded: timing candidates does not belong into a graph
+    want = rows % TUNE_ROWS == 0 and not torch.cuda.is_current_stream_capturing()
     if st["tuning"] != want:
         tunable.tuning_enable(want)
         st["tuning"] = want
