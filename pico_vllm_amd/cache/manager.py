@@ -107,12 +107,12 @@ class CacheManager:
         return [max(0, _cdiv(new_len, self.page_size) - len(t)) for t in rc.tables]
 
     def can_grow(self, req: Hashable, new_len: int) -> bool:
-        return all(n <= g.pool.num_free for n, g in zip(self.pages_needed(req, new_len), self.groups))
+        return all(g.pool.ensure_free(n) for n, g in zip(self.pages_needed(req, new_len), self.groups))
 
     def grow(self, req: Hashable, new_len: int) -> bool:
         """Cover positions [0, new_len) in every group, or change nothing and return False."""
         need = self.pages_needed(req, new_len)
-        if any(n > g.pool.num_free for n, g in zip(need, self.groups)):
+        if not all(g.pool.ensure_free(n) for n, g in zip(need, self.groups)):
             return False
         rc = self.requests[req]
         for gi, (n, g, table) in enumerate(zip(need, self.groups, rc.tables)):
@@ -193,11 +193,13 @@ class CacheManager:
         return page * self.page_size + position % self.page_size
 
     # ---- invariants -----------------------------------------------------
-    def check(self) -> None:
-        """No page lost, none held more often than counted, none both free and held."""
+    def check(self, other_holders: Optional[Sequence[Dict[int, int]]] = None) -> None:
+        """No page lost, none held more often than counted, none both free and held.
+        ``other_holders``: per group, page -> count for holders that are no requests
+        (whoever registered a reclaim callback)."""
         for gi, g in enumerate(self.groups):
             g.pool.check()
-            holders: Dict[int, int] = {}
+            holders: Dict[int, int] = dict(other_holders[gi]) if other_holders else {}
             for rc in self.requests.values():
                 seen = set()
                 for p in rc.tables[gi]:

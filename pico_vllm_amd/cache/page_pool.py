@@ -5,11 +5,14 @@ The counterpart in the reference is BlockManager's allocator half
 by allocate, inc_ref / dec_ref that frees at zero.  Differences: allocation
 reports failure instead of raising from inside a step (blockmanager.py:77-78),
 there is no CPU tier, and giving back a page that is not held is an error.
+Like there (set_evict_callback, blockmanager.py:66-75) a holder of pages that
+it can do without (an index of shared prefixes, say) may register a callable
+that is asked to give pages back before an allocation is refused.
 """
 from __future__ import annotations
 
 from collections import deque
-from typing import List, Optional
+from typing import Callable, List, Optional
 
 
 class PagePoolError(RuntimeError):
@@ -26,6 +29,20 @@ class PagePool:
         self.peak_used = 0
         self.reuse_count = 0           # pages handed out that had been used before
         self._ever_used = [False] * num_pages
+        self._reclaim: Optional[Callable[[int], int]] = None
+
+    def set_reclaim_callback(self, cb: Optional[Callable[[int], int]]) -> None:
+        """``cb(n)`` is called when ``n`` more pages are wanted than are free; it releases
+        pages that it holds (through ``release``) and returns how many holders it dropped,
+        0 when it has nothing left to give."""
+        self._reclaim = cb
+
+    def ensure_free(self, n: int) -> bool:
+        """Whether ``n`` pages are free, after asking the reclaim callback for the difference."""
+        while n > len(self._free) and self._reclaim is not None:
+            if self._reclaim(n - len(self._free)) <= 0:
+                break
+        return n <= len(self._free)
 
     @property
     def num_free(self) -> int:
@@ -42,7 +59,7 @@ class PagePool:
         """n fresh pages with count 1 each, or None (and nothing taken) if fewer are free."""
         if n < 0:
             raise ValueError("cannot allocate a negative number of pages")
-        if n > len(self._free):
+        if not self.ensure_free(n):
             return None
         out = [self._free.popleft() for _ in range(n)]
         for p in out:

@@ -96,6 +96,39 @@ def test_prefix_sharing_counts():
         m.add_request("c"); m.add_request("d"); m.grow("c", 20); m.advance("c", 20); m.fork_prefix("c", "d", 20)
 
 
+def test_a_holder_of_spare_pages_is_asked_before_an_allocation_is_refused():
+    """The seam for an index of shared prefixes: it keeps finished requests' pages and gives
+    them back, oldest first, when the pool runs short (the reference's evict callback,
+    pico_vllm/blockmanager.py:66-75, scenario of tests/test_evict_recompute.py:185-226)."""
+    m = CacheManager({0: FULL}, 16, 4, 3)
+    pool = m.groups[0].pool
+    kept, asked = [], []
+
+    def reclaim(n):
+        asked.append(n)
+        gone = kept[:n]
+        del kept[:n]
+        pool.release(gone)
+        return len(gone)
+
+    pool.set_reclaim_callback(reclaim)
+    m.add_request("a"); assert m.grow("a", 48); m.advance("a", 48)
+    pages = list(m.block_table("a"))
+    pool.share(pages[:2]); kept.extend(pages[:2])         # the keeper holds a's first two pages
+    m.free_request("a")
+    assert pool.num_free == 2 and not asked
+    m.check([{p: 1 for p in kept}])
+    m.add_request("b"); assert m.grow("b", 32) and not asked            # fits without asking
+    m.add_request("c"); assert m.grow("c", 16) and asked == [1]         # one page short: the keeper gives its oldest
+    assert kept == pages[1:2] and m.block_table("c") == [pages[0]]
+    m.check([{p: 1 for p in kept}])
+    assert not m.can_grow("c", 48) and kept == []                       # asked again, gave its last, still short
+    assert m.grow("c", 32)
+    m.check()
+    assert not m.grow("b", 48) and asked[-1] == 1                       # nothing left to give: refused, nothing taken
+    m.check()
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_random_orders_never_lose_or_double_hold_a_page(seed):
     rng = random.Random(seed)
