@@ -16,7 +16,8 @@
 //     about the order of k).  The copy is asynchronous: DEPTH slices per wave are in flight
 //     without holding registers;
 //   * up to 32 tokens: 4 waves per workgroup; 33 to 64 tokens: 2 waves, each with both blocks of
-//     32 tokens, so that three workgroups still share the LDS of a compute unit;
+//     32 tokens, so that three workgroups still share the LDS of a compute unit, or on large grids
+//     4 waves with two tiles of W that share the activations (gemm_skinny_pair_kernel);
 //   * when the matrix is too small to fill the chip (N small), the k range is also split over
 //     workgroups (grid y); each writes a float32 partial slab that the consumer sums;
 //   * K % 64 != 0 (any multiple of 8): a plain loop with operands in registers.
@@ -26,6 +27,7 @@
 // bfloat16 store.  Layout of the 32x32 result tile: lane l holds output column (token) l % 32 and
 // tile rows 8 (r / 4) + 4 (l / 32) + r % 4 in register r.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -230,25 +232,13 @@ __device__ __forceinline__ float (*skinny_tile(const bf16_t* __restrict__ X, int
   return red;
 }
 
-template <int MT, int EPI, bool TAIL, int NX>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
-                                                          const bf16_t* __restrict__ W, int ldw,
-                                                          const float* __restrict__ bias, void* __restrict__ out,
-                                                          int ldo, long long slab_stride, int M, int N, int K,
-                                                          int k_per_wg) {
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, false>()];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
-  const int tile = blockIdx.x;
-  const int m0 = blockIdx.z * 32 * MT;
-  // the rows of W that tile rows 0..15 and 16..31 stand for
-  const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
-  const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
-  const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, false>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
-
-  // thread (a, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col`: sum of the 4 sets of slices
-  constexpr int NWV = sk_waves<MT, NX, false>();
-  for (int a = wave; a < 4; a += NWV)
+// Thread (a, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col` of tile `tile`: the sum of the
+// 4 sets of slices, then the epilogue.
+template <int MT, int EPI>
+__device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile, int a, int m0, int M, int N,
+                                              const float* __restrict__ bias, void* __restrict__ out, int ldo,
+                                              long long slab_stride) {
+  const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
 #pragma unroll
   for (int t = 0; t < MT; t++) {
     const int m = m0 + 32 * t + col;
@@ -296,6 +286,154 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   }
 }
 
+template <int MT, int EPI, bool TAIL, int NX>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
+                                                          const bf16_t* __restrict__ W, int ldw,
+                                                          const float* __restrict__ bias, void* __restrict__ out,
+                                                          int ldo, long long slab_stride, int M, int N, int K,
+                                                          int k_per_wg) {
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, false>()];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int tile = blockIdx.x;
+  const int m0 = blockIdx.z * 32 * MT;
+  // the rows of W that tile rows 0..15 and 16..31 stand for
+  const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
+  const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
+  const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, false>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
+
+  constexpr int NWV = sk_waves<MT, NX, false>();
+  for (int a = wave; a < 4; a += NWV) skinny_finish<MT, EPI>(red, tile, a, m0, M, N, bias, out, ldo, slab_stride);
+}
+
+// ---- 33 to 64 tokens, large grids: two tiles of W share the activations ---------------------------
+// With 64 tokens a slice of activations is twice the bytes of a tile's slice of W, and every tile
+// fetches it again from the L2: that traffic, not HBM, bounds the stream (the 55 MB gate/up matrix
+// brings 110 MB of activations with it).  Here a workgroup owns 64 rows of W, two tiles, and four
+// waves (r, p) = (wave / 2, wave % 2): wave (r, p) multiplies tile r by the slices of parity p, and
+// the two waves of a parity share the activations of their slice, each copying half of them.  What
+// is shared needs a barrier per step; a step is one slice per parity, two stages alternate.  Slice
+// s of the k range still goes to set s % 4 of the sums, so a row's result is what the other
+// kernels give.
+constexpr int SK_PAIR_MIN_WGS = 160;      // below this many workgroups the one-tile kernel spreads the stream over more compute units
+constexpr int SK_PAIR_HALF = 16 * SK_GROUP;          // one parity of a stage: [W tile 0: 4 groups][W tile 1: 4][activations: 8]
+constexpr int SK_PAIR_STAGE = 2 * SK_PAIR_HALF;
+constexpr int SK_PAIR_SMEM = 2 * SK_PAIR_STAGE;      // 66,560 bytes: two workgroups share a compute unit; holds 2 x 32 KB of sums
+static_assert(SK_PAIR_SMEM >= 2 * 4 * 2 * 16 * 64 * 4, "the sums of both tiles take the place of the stages");
+
+// rows_a[r], rows_b[r]: the rows of W that tile rows 0..15 and 16..31 of tile r stand for.  Leaves the sums of
+// tile r in red[r][set][token block][register][lane] at the start of smem.
+__device__ __forceinline__ void skinny_stream_pair(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W,
+                                                   int ldw, int row_a, int row_b, int n_rows, int m0, int M, int k_begin,
+                                                   int k_end, char* smem) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = wave >> 1, p = wave & 1;
+  const int col = lane & 31, h = lane >> 5, rho = lane >> 3, pos = lane & 7;
+  const bf16_t* wsrc[4];
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    const int row = min((g < 2 ? row_a + 8 * g : row_b + 8 * (g - 2)) + rho, n_rows - 1);
+    wsrc[g] = W + (size_t)row * ldw + 8 * (pos ^ rho);
+  }
+  const bf16_t* xsrc[4];                       // this wave copies the token groups 4 r .. 4 r + 3 of its parity's slice
+#pragma unroll
+  for (int g = 0; g < 4; g++) xsrc[g] = X + (size_t)min(m0 + 8 * (4 * r + g) + rho, M - 1) * ldx + 8 * (pos ^ rho);
+  int rd[4];
+#pragma unroll
+  for (int s = 0; s < 4; s++) rd[s] = (col >> 3) * SK_GROUP + (col & 7) * 128 + (((4 * h + s) ^ (col & 7)) << 4);
+  f32x16 acc[2][2];                            // [token block][set of the wave: slice i of the wave goes to set i % 2]
+#pragma unroll
+  for (int t = 0; t < 2; t++)
+#pragma unroll
+    for (int v = 0; v < 2; v++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) acc[t][v][q] = 0.f;
+
+  const int n_total = (k_end - k_begin) >> 6;  // whole slices: the caller has checked
+  const int n_steps = (n_total + 1) >> 1;      // the same for every wave: the barriers below are met by all
+  const int n_mine = (n_total + 1 - p) >> 1;   // slices k_begin + 64 (p + 2 i), i < n_mine
+  auto issue = [&](int d, int i) {
+    if (i >= n_mine) return;
+    const int k0 = k_begin + 64 * (p + 2 * i);
+    char* half = smem + d * SK_PAIR_STAGE + p * SK_PAIR_HALF;
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+      __builtin_amdgcn_global_load_lds(GPTR(wsrc[g] + k0), LPTR(half + (4 * r + g) * SK_GROUP), 16, 0, 0);
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+      __builtin_amdgcn_global_load_lds(GPTR(xsrc[g] + k0), LPTR(half + (8 + 4 * r + g) * SK_GROUP), 16, 0, 0);
+  };
+  auto multiply = [&](auto dc, int i) {
+    constexpr int d = decltype(dc)::value;     // stage and set of the sums alike
+    if (i >= n_mine) return;
+    const char* half = smem + d * SK_PAIR_STAGE + p * SK_PAIR_HALF;
+    u32x4 a[4], b[2][4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      a[s] = *reinterpret_cast<const u32x4*>(half + 4 * r * SK_GROUP + rd[s]);
+#pragma unroll
+      for (int t = 0; t < 2; t++) b[t][s] = *reinterpret_cast<const u32x4*>(half + (8 + 4 * t) * SK_GROUP + rd[s]);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+        acc[t][d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[s]), __builtin_bit_cast(bf16x8, b[t][s]),
+                                                            acc[t][d], 0, 0, 0);
+  };
+  issue(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int i = 0; i < n_steps; i += 2) {
+    // The copies of step i have landed for this wave, after the barrier for all; every wave has also
+    // issued the products of step i - 1 by then, so its operand reads of the other stage are complete
+    // and the stage can be filled again.  The compiler does not order LDS reads after these copies by itself.
+    __builtin_amdgcn_s_waitcnt(sk_vmcnt(0));
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    issue(1, i + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(std::integral_constant<int, 0>{}, i);
+    __builtin_amdgcn_sched_barrier(0);
+    if (i + 1 < n_steps) {
+      __builtin_amdgcn_s_waitcnt(sk_vmcnt(0));
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      issue(0, i + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(std::integral_constant<int, 1>{}, i + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __syncthreads();                             // every wave is done with the stages: the sums take their place
+  float(*red)[2][16][64] = reinterpret_cast<float(*)[2][16][64]>(smem) + 4 * r;
+#pragma unroll
+  for (int t = 0; t < 2; t++)
+#pragma unroll
+    for (int v = 0; v < 2; v++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) red[p + 2 * v][t][q][lane] = acc[t][v][q];
+  __syncthreads();
+}
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __restrict__ X, int ldx,
+                                                               const bf16_t* __restrict__ W, int ldw,
+                                                               const float* __restrict__ bias, void* __restrict__ out,
+                                                               int ldo, long long slab_stride, int M, int N, int K,
+                                                               int k_per_wg) {
+  __shared__ __attribute__((aligned(16))) char smem[SK_PAIR_SMEM];
+  const int wave = threadIdx.x >> 6;
+  const int tile = 2 * blockIdx.x + (wave >> 1);     // of this wave while it streams
+  const int m0 = blockIdx.z * 64;
+  const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
+  const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
+  const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
+  skinny_stream_pair(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
+  float(*red)[2][16][64] = reinterpret_cast<float(*)[2][16][64]>(smem);
+  for (int item = wave; item < 8; item += 4)         // (tile of the pair, a)
+    skinny_finish<2, EPI>(red + 4 * (item >> 2), 2 * blockIdx.x + (item >> 2), item & 3, m0, M, N, bias, out, ldo, slab_stride);
+}
+
 // k_splits > 1 is allowed for EPI_F32 only: slab y (float32 [M, ldo]) lies at out + y * slab_stride and
 // holds the partial sum over its k range; the bias goes into slab 0.
 extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* out, int ldo,
@@ -321,6 +459,19 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   const bool tail = K % 64 != 0;
   // few rows and whole slices: the stream through LDS, with as many 8-token groups as hold tokens
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
+  // 33 to 64 tokens and enough tiles: two tiles of W per workgroup share the activations
+  const bool pair = nx == 8 && (long long)((tiles + 1) / 2) * ky >= SK_PAIR_MIN_WGS;
+  if (pair) {
+    dim3 pgrid((tiles + 1) / 2, ky, grid.z);
+#define LAUNCHP(EPI) \
+  gemm_skinny_pair_kernel<EPI><<<pgrid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+    if (epilogue == EPI_BF16) LAUNCHP(EPI_BF16);
+    else if (epilogue == EPI_F32) LAUNCHP(EPI_F32);
+    else LAUNCHP(EPI_SWIGLU);
+#undef LAUNCHP
+    PICO_LAUNCH_CHECK();
+    return 0;
+  }
 #define LAUNCH3(MT, EPI, TAIL, NX) \
   gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, false>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
 #define LAUNCH(EPI)                                               \

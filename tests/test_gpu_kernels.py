@@ -424,7 +424,10 @@ def test_fast_kernels_refuse_what_they_cannot_do(K):
 # ---- weight-streaming GEMM --------------------------------------------------------------------
 @pytest.mark.parametrize("M,N,K_", [(1, 2048, 1536), (8, 1536, 1536), (64, 1536, 8960), (33, 301, 136), (5, 384, 192),
                                    (2, 64, 320), (17, 1000, 264), (12, 1536, 1536), (16, 90, 64), (24, 512, 1024),
-                                   (32, 301, 256), (9, 1000, 8960)])
+                                   (32, 301, 256), (9, 1000, 8960),
+                                   # more than 32 tokens and many tiles: two tiles a workgroup (an odd number of tiles,
+                                   # an odd number of slices, a single slice)
+                                   (50, 10270, 192), (40, 10400, 64), (64, 10240, 320)])
 def test_gemm_skinny_epilogues(K, M, N, K_):
     g = torch.Generator().manual_seed(M * N)
     a = torch.randn(M, K_, generator=g).bfloat16()
