@@ -33,6 +33,20 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// The rows of W behind a 32-row tile: tile rows 0..15 are rows row_a .. row_a + va - 1 of W, tile rows
+// 16..31 rows row_b .. row_b + vb - 1 (va >= 1, vb >= 0, at most 16 each).  Tile rows without a row of
+// their own read the last row of their half again (the same cache lines: no traffic); what they sum
+// is never stored.  A tile with fewer rows is how the host makes the number of workgroups fit the
+// chip: a compute unit takes in about 25 GB/s whatever runs on it, so the time of a launch is what
+// the fullest compute unit has to read, and 560 tiles on 256 compute units cost as much as 768.
+struct TileRows {
+  int row_a, row_b, va, vb;
+  __device__ __forceinline__ int row(int tile_row) const {     // the row of W that tile row `tile_row` reads
+    const bool second = tile_row >= 16 && vb > 0;
+    return second ? row_b + min(tile_row - 16, vb - 1) : row_a + min(tile_row, va - 1);
+  }
+};
+
 #define EPI_BF16 0     // out bf16 [M, N]
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
@@ -94,7 +108,9 @@ __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int 
 #define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 constexpr int SK_GROUP = 1024 + 16;
 template <int NX> constexpr int sk_stage_bytes() { return (4 + NX) * SK_GROUP; }
-template <int NX> constexpr int sk_depth() { return NX >= 4 ? 2 : 3; }
+// slices in flight per wave.  FEW (at most one workgroup per compute unit, the whole LDS is its own): as many
+// as fit, because such a launch is a chain of memory latencies, not a stream
+template <int NX, bool FEW> constexpr int sk_depth() { return FEW ? (NX <= 2 ? 6 : NX == 4 ? 4 : 3) : (NX >= 4 ? 2 : 3); }
 // waves per workgroup: two when a wave holds two blocks of tokens in LDS and the grid is large, so that
 // three workgroups fit a compute unit; four otherwise (FEW: at most one workgroup per compute unit anyway)
 template <int MT, int NX, bool FEW> constexpr int sk_waves() { return (MT == 2 && NX > 0 && !FEW) ? 2 : 4; }
@@ -105,30 +121,27 @@ template <int MT, int NX, bool FEW>
 constexpr int sk_smem_bytes() {
   constexpr int red = 4 * MT * 16 * 64 * 4;
   if (NX == 0) return red;
-  constexpr int stages = sk_depth<NX>() * sk_waves<MT, NX, FEW>() * sk_stage_bytes<NX>();
+  constexpr int stages = sk_depth<NX, FEW>() * sk_waves<MT, NX, FEW>() * sk_stage_bytes<NX>();
   return stages > red ? stages : red;
 }
 
-// Tile rows 0..15 are rows row_a .. of W, tile rows 16..31 rows row_b .. (clamped to n_rows - 1);
+// The sums of tile `tr`;
 // tokens m0 .. m0 + 8 NX - 1 (clamped to M - 1) in MT blocks of 32.  The sums end up in
 // red[v][token block][register][lane] at the start of smem, as skinny_stream leaves them: v = 0..3
 // holds the slices k_begin + 64 (v + 4 i) whatever the number of waves (a wave of a two-wave
 // workgroup keeps two sets of sums), so that a row's result does not depend on how many rows came
 // with it.
-template <int MT, int NX, int NWV>
+template <int MT, int NX, int NWV, int DEPTH>
 __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W,
-                                                  int ldw, int row_a, int row_b, int n_rows, int m0, int M, int k_begin,
+                                                  int ldw, TileRows tr, int m0, int M, int k_begin,
                                                   int k_end, char* smem) {
-  constexpr int DEPTH = sk_depth<NX>(), STAGE = sk_stage_bytes<NX>(), LOADS = 4 + NX;
+  constexpr int STAGE = sk_stage_bytes<NX>(), LOADS = 4 + NX;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int col = lane & 31, h = lane >> 5, rho = lane >> 3, pos = lane & 7;
   // sources of this lane's 16 bytes in each group, at k = 0
   const bf16_t* wsrc[4];
 #pragma unroll
-  for (int g = 0; g < 4; g++) {
-    const int row = min((g < 2 ? row_a + 8 * g : row_b + 8 * (g - 2)) + rho, n_rows - 1);
-    wsrc[g] = W + (size_t)row * ldw + 8 * (pos ^ rho);
-  }
+  for (int g = 0; g < 4; g++) wsrc[g] = W + (size_t)tr.row(8 * g + rho) * ldw + 8 * (pos ^ rho);
   const bf16_t* xsrc[NX];
 #pragma unroll
   for (int g = 0; g < NX; g++) xsrc[g] = X + (size_t)min(m0 + 8 * g + rho, M - 1) * ldx + 8 * (pos ^ rho);
@@ -216,36 +229,54 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
 // The 32 tile rows' sums for this workgroup's tokens, through LDS (NX > 0) or registers (NX == 0).
 template <int MT, bool TAIL, int NX, bool FEW>
 __device__ __forceinline__ float (*skinny_tile(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
-                                               int row_a, int row_b, int n_rows, int m0, int M, int k_begin, int k_end,
+                                               TileRows tr, int m0, int M, int k_begin, int k_end,
                                                char* smem))[MT][16][64] {
   float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
   if constexpr (NX > 0) {
     static_assert(!TAIL && NX <= 4 * MT, "the stream through LDS takes whole slices");
-    skinny_stream_lds<MT, NX, sk_waves<MT, NX, FEW>()>(X, ldx, W, ldw, row_a, row_b, n_rows, m0, M, k_begin, k_end, smem);
+    skinny_stream_lds<MT, NX, sk_waves<MT, NX, FEW>(), sk_depth<NX, FEW>()>(X, ldx, W, ldw, tr, m0, M, k_begin, k_end, smem);
   } else {
-    const int col = threadIdx.x & 31;
-    const int wrow = col < 16 ? row_a + col : row_b + col - 16;
-    // Rows beyond the matrix are clamped to its last row: what they contribute is never stored.
     // Only a k tail must read as zero, because it is summed into outputs that are stored.
-    skinny_stream<MT>(X, ldx, W + (size_t)min(wrow, n_rows - 1) * ldw, m0, M, k_begin, k_end, red);
+    skinny_stream<MT>(X, ldx, W + (size_t)tr.row(threadIdx.x & 31) * ldw, m0, M, k_begin, k_end, red);
   }
   return red;
 }
 
-// Thread (a, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col` of tile `tile`: the sum of the
-// 4 sets of slices, then the epilogue.
+// Which rows of W stand behind tile `tile` when a tile has `rows` of them (`rows` pairs for SwiGLU: gate rows
+// in the first half of the tile, the matching up rows in the second).
+template <int EPI>
+__device__ __forceinline__ TileRows skinny_rows(int tile, int rows, int N) {
+  TileRows tr;
+  if (EPI == EPI_SWIGLU) {
+    const int I = N / 2;
+    tr.row_a = min(tile * rows, I - 1);
+    tr.row_b = I + tr.row_a;
+    tr.va = tr.vb = min(rows, I - tr.row_a);
+  } else {
+    tr.row_a = min(tile * rows, N - 1);
+    tr.row_b = tr.row_a + 16;
+    tr.va = min(min(rows, 16), N - tr.row_a);
+    tr.vb = max(0, min(rows - 16, N - tr.row_b));
+  }
+  return tr;
+}
+
+// Thread (a, lane) finishes tile rows 8 a + 4 h + 0..3 of column `col` of tile `tile` of `rows` rows
+// (pairs): the sum of the 4 sets of slices, then the epilogue.
 template <int MT, int EPI>
-__device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile, int a, int m0, int M, int N,
+__device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile, int rows, int a, int m0, int M, int N,
                                               const float* __restrict__ bias, void* __restrict__ out, int ldo,
                                               long long slab_stride) {
   const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int t0 = 8 * a + 4 * h;                      // this thread's first tile row
+  if (t0 >= rows) return;
 #pragma unroll
   for (int t = 0; t < MT; t++) {
     const int m = m0 + 32 * t + col;
     if (m >= M) continue;
     if (EPI == EPI_SWIGLU) {
       if (a >= 2) continue;
-      const int I = N / 2, gi = tile * 16 + 8 * a + 4 * h;
+      const int I = N / 2, gi = tile * rows + t0;
       float v[4];
 #pragma unroll
       for (int b = 0; b < 4; b++) {
@@ -260,9 +291,9 @@ __device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile
       bf16_t* o = (bf16_t*)out + (size_t)m * ldo + gi;
 #pragma unroll
       for (int b = 0; b < 4; b++)
-        if (gi + b < I) store_f32(o + b, v[b]);
+        if (t0 + b < rows && gi + b < I) store_f32(o + b, v[b]);
     } else {
-      const int n = tile * 32 + 8 * a + 4 * h;
+      const int n = tile * rows + t0;
       float v[4];
 #pragma unroll
       for (int b = 0; b < 4; b++) {
@@ -275,12 +306,12 @@ __device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile
         float* o = (float*)out + (size_t)blockIdx.y * slab_stride + (size_t)m * ldo + n;
 #pragma unroll
         for (int b = 0; b < 4; b++)
-          if (n + b < N) o[b] = v[b];
+          if (t0 + b < rows && n + b < N) o[b] = v[b];
       } else {
         bf16_t* o = (bf16_t*)out + (size_t)m * ldo + n;
 #pragma unroll
         for (int b = 0; b < 4; b++)
-          if (n + b < N) store_f32(o + b, v[b]);
+          if (t0 + b < rows && n + b < N) store_f32(o + b, v[b]);
       }
     }
   }
@@ -291,19 +322,15 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias, void* __restrict__ out,
                                                           int ldo, long long slab_stride, int M, int N, int K,
-                                                          int k_per_wg) {
+                                                          int k_per_wg, int rows) {
   __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, false>()];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
+  const int wave = threadIdx.x >> 6;
   const int tile = blockIdx.x;
   const int m0 = blockIdx.z * 32 * MT;
-  // the rows of W that tile rows 0..15 and 16..31 stand for
-  const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
-  const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, false>(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
-
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, false>(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
   constexpr int NWV = sk_waves<MT, NX, false>();
-  for (int a = wave; a < 4; a += NWV) skinny_finish<MT, EPI>(red, tile, a, m0, M, N, bias, out, ldo, slab_stride);
+  for (int a = wave; a < 4; a += NWV) skinny_finish<MT, EPI>(red, tile, rows, a, m0, M, N, bias, out, ldo, slab_stride);
 }
 
 // ---- 33 to 64 tokens, large grids: two tiles of W share the activations ---------------------------
@@ -321,20 +348,16 @@ constexpr int SK_PAIR_STAGE = 2 * SK_PAIR_HALF;
 constexpr int SK_PAIR_SMEM = 2 * SK_PAIR_STAGE;      // 66,560 bytes: two workgroups share a compute unit; holds 2 x 32 KB of sums
 static_assert(SK_PAIR_SMEM >= 2 * 4 * 2 * 16 * 64 * 4, "the sums of both tiles take the place of the stages");
 
-// rows_a[r], rows_b[r]: the rows of W that tile rows 0..15 and 16..31 of tile r stand for.  Leaves the sums of
-// tile r in red[r][set][token block][register][lane] at the start of smem.
+// tr: the tile of this wave.  Leaves the sums of tile r in red[r][set][token block][register][lane] at the start of smem.
 __device__ __forceinline__ void skinny_stream_pair(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W,
-                                                   int ldw, int row_a, int row_b, int n_rows, int m0, int M, int k_begin,
+                                                   int ldw, TileRows tr, int m0, int M, int k_begin,
                                                    int k_end, char* smem) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = wave >> 1, p = wave & 1;
   const int col = lane & 31, h = lane >> 5, rho = lane >> 3, pos = lane & 7;
   const bf16_t* wsrc[4];
 #pragma unroll
-  for (int g = 0; g < 4; g++) {
-    const int row = min((g < 2 ? row_a + 8 * g : row_b + 8 * (g - 2)) + rho, n_rows - 1);
-    wsrc[g] = W + (size_t)row * ldw + 8 * (pos ^ rho);
-  }
+  for (int g = 0; g < 4; g++) wsrc[g] = W + (size_t)tr.row(8 * g + rho) * ldw + 8 * (pos ^ rho);
   const bf16_t* xsrc[4];                       // this wave copies the token groups 4 r .. 4 r + 3 of its parity's slice
 #pragma unroll
   for (int g = 0; g < 4; g++) xsrc[g] = X + (size_t)min(m0 + 8 * (4 * r + g) + rho, M - 1) * ldx + 8 * (pos ^ rho);
@@ -425,13 +448,49 @@ __global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __r
   const int wave = threadIdx.x >> 6;
   const int tile = 2 * blockIdx.x + (wave >> 1);     // of this wave while it streams
   const int m0 = blockIdx.z * 64;
-  const int row_a = EPI == EPI_SWIGLU ? tile * 16 : tile * 32;
-  const int row_b = EPI == EPI_SWIGLU ? N / 2 + tile * 16 : tile * 32 + 16;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  skinny_stream_pair(X, ldx, W, ldw, row_a, row_b, N, m0, M, k_begin, k_end, smem);
+  constexpr int ROWS = EPI == EPI_SWIGLU ? 16 : 32;
+  skinny_stream_pair(X, ldx, W, ldw, skinny_rows<EPI>(tile, ROWS, N), m0, M, k_begin, k_end, smem);
   float(*red)[2][16][64] = reinterpret_cast<float(*)[2][16][64]>(smem);
   for (int item = wave; item < 8; item += 4)         // (tile of the pair, a)
-    skinny_finish<2, EPI>(red + 4 * (item >> 2), 2 * blockIdx.x + (item >> 2), item & 3, m0, M, N, bias, out, ldo, slab_stride);
+    skinny_finish<2, EPI>(red + 4 * (item >> 2), 2 * blockIdx.x + (item >> 2), ROWS, item & 3, m0, M, N, bias, out, ldo, slab_stride);
+}
+
+// How many rows of W (pairs of rows for the SwiGLU and rotation epilogues, `unit` = 2 rows) a tile gets:
+// the time of a launch goes with what the fullest compute unit reads, its workgroups' rows of W and the
+// activations that each workgroup reads again, so among 4, 3, 2 and 1 quarters of a tile take the height
+// with the least of it; ties go to the taller tile.  total: rows (pairs) of the matrix; k_splits: ranges
+// of k, each a workgroup of its own; x_rows: rows of activations a workgroup fetches per slice.
+static const int SK_COMPUTE_UNITS = 256;
+static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, long long* cost_out = nullptr) {
+  int best = 0;
+  long long best_cost = 0;
+  for (int q = 4; q >= 1; q--) {
+    const int h = q * (8 / unit);                    // rows or pairs per tile
+    const long long wgs = (total + h - 1) / h * k_splits;
+    const long long cost = (wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS * (h * unit + x_rows);
+    if (best == 0 || cost < best_cost) best = h, best_cost = cost;
+  }
+  if (cost_out) *cost_out = best_cost;
+  return best;
+}
+
+// Into how many ranges of whole 256-wide steps the k of a small matrix [N, K] is cut, each range a
+// workgroup of its own that leaves a float32 slab of partial sums: the cut for which the fullest
+// compute unit reads least (ties: fewer slabs).  It depends on the matrix alone, never on the number
+// of tokens, so that a token's sums are formed in the same order whatever comes with it.
+extern "C" int pico_gemm_skinny_k_splits(int N, int K, int max_splits) {
+  int best = 1;
+  long long best_cost = 0;
+  for (int want = 1; want <= max_splits; want++) {
+    const int per = ((K + want - 1) / want + 255) / 256 * 256;
+    if ((K + per - 1) / per != want) continue;       // ranges would be empty
+    long long cost;
+    skinny_tile_height(N, 1, want, 8, &cost);
+    cost *= per;
+    if (want == 1 || cost < best_cost) best = want, best_cost = cost;
+  }
+  return best;
 }
 
 // k_splits > 1 is allowed for EPI_F32 only: slab y (float32 [M, ldo]) lies at out + y * slab_stride and
@@ -449,16 +508,20 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   const int n_out = epilogue == EPI_SWIGLU ? N / 2 : N;
   PICO_REQUIRE(ldo >= n_out, "pico_gemm_skinny: output row stride too small");
   const int mt = M <= 32 ? 1 : 2;
-  const int tiles = epilogue == EPI_SWIGLU ? (N / 2 + 15) / 16 : (N + 31) / 32;
   const int k_per_wg = ((K + k_splits - 1) / k_splits + 255) / 256 * 256;
   const int ky = (K + k_per_wg - 1) / k_per_wg;
   PICO_REQUIRE(ky == k_splits, "pico_gemm_skinny: K=%d cannot be cut into %d ranges of whole 256-wide steps (got %d)", K, k_splits, ky);
-  dim3 grid(tiles, ky, (M + 32 * mt - 1) / (32 * mt));
-  PICO_REQUIRE(grid.z <= 65535 && grid.y <= 65535, "pico_gemm_skinny: too many blocks");
-  const float* b0 = bias;
   const bool tail = K % 64 != 0;
   // few rows and whole slices: the stream through LDS, with as many 8-token groups as hold tokens
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
+  const int unit = epilogue == EPI_SWIGLU ? 2 : 1;
+  const int total = epilogue == EPI_SWIGLU ? N / 2 : N;
+  // up to 32 tokens: the tile height that fills the chip best; more: whole tiles
+  const int rows = mt == 1 ? skinny_tile_height(total, unit, ky, M <= 8 ? 8 : M <= 16 ? 16 : 32) : 32 / unit;
+  const int tiles = (total + rows - 1) / rows;
+  dim3 grid(tiles, ky, (M + 32 * mt - 1) / (32 * mt));
+  PICO_REQUIRE(grid.z <= 65535 && grid.y <= 65535, "pico_gemm_skinny: too many blocks");
+  const float* b0 = bias;
   // 33 to 64 tokens and enough tiles: two tiles of W per workgroup share the activations
   const bool pair = nx == 8 && (long long)((tiles + 1) / 2) * ky >= SK_PAIR_MIN_WGS;
   if (pair) {
@@ -473,7 +536,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
     return 0;
   }
 #define LAUNCH3(MT, EPI, TAIL, NX) \
-  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, false>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, false>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
 #define LAUNCH(EPI)                                               \
   do {                                                            \
     if (nx == 1) LAUNCH3(1, EPI, false, 1);                       \
@@ -497,9 +560,9 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
 // bias, rotate-half position encoding of q and k (pico_vllm/kernels/fused_rope_kvcache_store.py:51-101
 // fuses the rotation with the store; here both ride on the projection) and the store of k and v
 // into the paged cache.  W = [q heads | k heads | v heads] x d rows.  A tile of a q or k head
-// holds 16 rows j .. j + 15 of the head and the 16 rows j + d/2 .. they are rotated with, so a pair
-// is local to a lane as gate and up are in the SwiGLU epilogue; a tile of a v head holds 32
-// consecutive rows.  Needs rot == d and d % 32 == 0.
+// holds `pairs` (16, 8 or 4: what fills the chip best) rows j .. of the head and the rows j + d/2 ..
+// they are rotated with, so a pair is local to a lane as gate and up are in the SwiGLU epilogue; a
+// tile of a v head holds 2 `pairs` consecutive rows.  Needs rot == d and d % 32 == 0.
 //   cos_sin [M][d / 2][2] float32: cosine and sine of every token's angles (pico_rope_table);
 //   q_out [M, ldq] bfloat16 gets the rotated q heads at columns head * d + dim;
 //   K pages [page][kv head][slot][d], V pages [page][kv head][d][slot], P = 1 << pshift slots;
@@ -510,28 +573,69 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
     const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
     bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
     bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
-    int nq, int nkv, int d, int pshift, int num_pages) {
+    int nq, int nkv, int d, int pshift, int num_pages, int pairs) {
   // the grid of this projection is small (one workgroup per 32 of (nq + 2 nkv) d rows): four waves always
   __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, true>()];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
-  const int tiles_per_head = d >> 5, half = d >> 1;
+  const int half = d >> 1, tiles_per_head = half / pairs;
   const int head = blockIdx.x / tiles_per_head, tp = blockIdx.x % tiles_per_head;
   const int m0 = blockIdx.z * 32 * MT;
   const bool rotated = head < nq + nkv;
-  const int row_a = head * d + (rotated ? 16 * tp : 32 * tp);
-  const int row_b = rotated ? row_a + half : row_a + 16;
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, true>(X, ldx, W, ldw, row_a, row_b, (nq + 2 * nkv) * d, m0, M, 0, K, smem);
+  TileRows tr;
+  if (rotated) {                      // `pairs` dimensions j and the ones they are rotated with
+    tr.row_a = head * d + pairs * tp;
+    tr.row_b = tr.row_a + half;
+    tr.va = tr.vb = pairs;
+  } else {                            // 2 `pairs` consecutive dimensions
+    tr.row_a = head * d + 2 * pairs * tp;
+    tr.row_b = tr.row_a + 16;
+    tr.va = min(2 * pairs, 16);
+    tr.vb = 2 * pairs - tr.va;
+  }
+  // What the epilogue needs besides the sums is read now, so that the stream hides the latency: thread
+  // (wave a, lane (col, h)) finishes tile rows 8 a + 4 h + 0..3 of token block t's column `col`.
+  static_assert(sk_waves<MT, NX, true>() == 4, "one wave per 8 tile rows");
+  const int a = wave, t0 = 8 * a + 4 * h;
+  const bool mine = rotated ? (a < 2 && t0 < pairs) : t0 < 2 * pairs;
+  const int e0 = rotated ? pairs * tp + t0 : 2 * pairs * tp + t0;      // first of this thread's four head dimensions
+  float b1[4] = {0.f, 0.f, 0.f, 0.f}, b2[4] = {0.f, 0.f, 0.f, 0.f};
+  float2 cs[MT][4];
+  int slot[MT];
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    slot[t] = -1;
+#pragma unroll
+    for (int b = 0; b < 4; b++) cs[t][b] = make_float2(1.f, 0.f);
+  }
+  if (mine) {
+    if (bias) {
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        b1[b] = bias[head * d + e0 + b];
+        if (rotated) b2[b] = bias[head * d + e0 + b + half];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+      const int m = m0 + 32 * t + col;
+      if (m >= M) continue;
+      if (head >= nq) slot[t] = slots[m];
+      if (rotated) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) cs[t][b] = cos_sin[(size_t)m * half + e0 + b];
+      }
+    }
+  }
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, true>(X, ldx, W, ldw, tr, m0, M, 0, K, smem);
+  if (!mine) return;
 
-  constexpr int NWV = sk_waves<MT, NX, true>();
-  for (int a = wave; a < 4; a += NWV)
 #pragma unroll
   for (int t = 0; t < MT; t++) {
     const int m = m0 + 32 * t + col;
     if (m >= M) continue;
+    const int page = slot[t] >> pshift;
+    if (head >= nq && (slot[t] < 0 || page >= num_pages)) continue;   // padding row; the host has checked the rest
     if (rotated) {
-      if (a >= 2) continue;
-      const int j0 = 16 * tp + 8 * a + 4 * h;        // this thread's four pairs (j, j + d/2)
-      const float2* cs = cos_sin + (size_t)m * half + j0;
       float y1[4], y2[4];
 #pragma unroll
       for (int b = 0; b < 4; b++) {
@@ -541,42 +645,26 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
           x1 += red[w][t][4 * a + b][lane];
           x2 += red[w][t][4 * (a + 2) + b][lane];
         }
-        if (bias) {
-          x1 += bias[head * d + j0 + b];
-          x2 += bias[head * d + j0 + b + half];
-        }
         // rounded as the projection's output is when it goes through memory, so that a token gets
         // the same key whether it came in a small step (here) or in a large one
-        x1 = bf16_to_f32(f32_to_bf16(x1));
-        x2 = bf16_to_f32(f32_to_bf16(x2));
-        const float c = cs[b].x, s = cs[b].y;
-        y1[b] = x1 * c - x2 * s;
-        y2[b] = x2 * c + x1 * s;
+        x1 = bf16_to_f32(f32_to_bf16(x1 + b1[b]));
+        x2 = bf16_to_f32(f32_to_bf16(x2 + b2[b]));
+        const float c = cs[t][b].x, sn = cs[t][b].y;
+        y1[b] = x1 * c - x2 * sn;
+        y2[b] = x2 * c + x1 * sn;
       }
-      bf16_t* o;
-      if (head < nq) {
-        o = q_out + (size_t)m * ldq + head * d + j0;
-      } else {
-        const int slot = slots[m];
-        const int page = slot >> pshift;
-        if (slot < 0 || page >= num_pages) continue;   // padding row; the host has checked the rest
-        o = k_cache + ((((size_t)page * nkv + (head - nq)) << pshift) + (slot & ((1 << pshift) - 1))) * d + j0;
-      }
+      bf16_t* o = head < nq ? q_out + (size_t)m * ldq + head * d + e0
+                            : k_cache + ((((size_t)page * nkv + (head - nq)) << pshift) + (slot[t] & ((1 << pshift) - 1))) * d + e0;
       *reinterpret_cast<uint2*>(o) = make_uint2(pack2_bf16(y1[0], y1[1]), pack2_bf16(y1[2], y1[3]));
       *reinterpret_cast<uint2*>(o + half) = make_uint2(pack2_bf16(y2[0], y2[1]), pack2_bf16(y2[2], y2[3]));
     } else {
-      const int slot = slots[m];
-      const int page = slot >> pshift;
-      if (slot < 0 || page >= num_pages) continue;
-      const int n0 = 32 * tp + 8 * a + 4 * h;          // this thread's four head dimensions
-      bf16_t* o = v_cache + ((((size_t)page * nkv + (head - nq - nkv)) * d + n0) << pshift) + (slot & ((1 << pshift) - 1));
+      bf16_t* o = v_cache + ((((size_t)page * nkv + (head - nq - nkv)) * d + e0) << pshift) + (slot[t] & ((1 << pshift) - 1));
 #pragma unroll
       for (int b = 0; b < 4; b++) {
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) v += red[w][t][4 * a + b][lane];
-        if (bias) v += bias[head * d + n0 + b];
-        o[(size_t)b << pshift] = f32_to_bf16(v);
+        o[(size_t)b << pshift] = f32_to_bf16(v + b1[b]);
       }
     }
   }
@@ -598,13 +686,18 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   const int mt = M <= 32 ? 1 : 2;
   int pshift = 0;
   while ((1 << pshift) < P) pshift++;
-  dim3 grid((nq + 2 * nkv) * (d / 32), 1, (M + 32 * mt - 1) / (32 * mt));
+  int pairs = 16;
+  if (mt == 1) {                      // 12 pairs would not divide d / 2
+    pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, M <= 8 ? 8 : M <= 16 ? 16 : 32);
+    if (pairs == 12) pairs = 16;
+  }
+  dim3 grid((nq + 2 * nkv) * (d / 2 / pairs), 1, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535, "pico_gemm_skinny_rope: too many rows");
   const bool tail = K % 64 != 0;
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH(MT, TAIL, NX) \
   gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, true>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
-      (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages)
+      (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages, pairs)
   if (nx == 1) LAUNCH(1, false, 1);
   else if (nx == 2) LAUNCH(1, false, 2);
   else if (nx == 4) LAUNCH(1, false, 4);

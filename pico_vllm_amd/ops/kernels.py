@@ -7,6 +7,7 @@ must live on the GPU; there is no CPU path.
 from __future__ import annotations
 
 import ctypes
+import functools
 from typing import Optional
 
 import torch
@@ -246,17 +247,12 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+@functools.lru_cache(maxsize=None)
 def skinny_k_splits(N: int, K: int, max_splits: int = 8) -> int:
-    """How many workgroups share the k range of a small matrix: enough workgroups to cover the chip,
-    ranges of whole 256-wide steps, every range non-empty."""
-    tiles = -(-N // 32)
-    want = max(1, min(max_splits, 512 // max(1, tiles), K // 256))
-    while want > 1:
-        per = -(-(-(-K // want)) // 256) * 256
-        if -(-K // per) == want:
-            return want
-        want -= 1
-    return 1
+    """Into how many ranges of whole 256-wide steps the k of a small matrix is cut, each range a
+    workgroup of its own that leaves a slab of partial sums: the cut with which the fullest compute
+    unit reads least.  It depends on the matrix alone, never on the number of tokens."""
+    return int(library.core().pico_gemm_skinny_k_splits(N, K, max_splits))
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int):
