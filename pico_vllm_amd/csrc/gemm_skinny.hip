@@ -342,7 +342,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 // is shared needs a barrier per step; a step is one slice per parity, two stages alternate.  Slice
 // s of the k range still goes to set s % 4 of the sums, so a row's result is what the other
 // kernels give.
-constexpr int SK_PAIR_MIN_WGS = 160;      // below this many workgroups the one-tile kernel spreads the stream over more compute units
 constexpr int SK_PAIR_HALF = 16 * SK_GROUP;          // one parity of a stage: [W tile 0: 4 groups][W tile 1: 4][activations: 8]
 constexpr int SK_PAIR_STAGE = 2 * SK_PAIR_HALF;
 constexpr int SK_PAIR_SMEM = 2 * SK_PAIR_STAGE;      // 66,560 bytes: two workgroups share a compute unit; holds 2 x 32 KB of sums
@@ -443,17 +442,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __r
                                                                const bf16_t* __restrict__ W, int ldw,
                                                                const float* __restrict__ bias, void* __restrict__ out,
                                                                int ldo, long long slab_stride, int M, int N, int K,
-                                                               int k_per_wg) {
+                                                               int k_per_wg, int rows) {
   __shared__ __attribute__((aligned(16))) char smem[SK_PAIR_SMEM];
   const int wave = threadIdx.x >> 6;
   const int tile = 2 * blockIdx.x + (wave >> 1);     // of this wave while it streams
   const int m0 = blockIdx.z * 64;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  constexpr int ROWS = EPI == EPI_SWIGLU ? 16 : 32;
-  skinny_stream_pair(X, ldx, W, ldw, skinny_rows<EPI>(tile, ROWS, N), m0, M, k_begin, k_end, smem);
+  skinny_stream_pair(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
   float(*red)[2][16][64] = reinterpret_cast<float(*)[2][16][64]>(smem);
   for (int item = wave; item < 8; item += 4)         // (tile of the pair, a)
-    skinny_finish<2, EPI>(red + 4 * (item >> 2), 2 * blockIdx.x + (item >> 2), ROWS, item & 3, m0, M, N, bias, out, ldo, slab_stride);
+    skinny_finish<2, EPI>(red + 4 * (item >> 2), 2 * blockIdx.x + (item >> 2), rows, item & 3, m0, M, N, bias, out, ldo, slab_stride);
 }
 
 // How many rows of W (pairs of rows for the SwiGLU and rotation epilogues, `unit` = 2 rows) a tile gets:
@@ -462,13 +460,14 @@ __global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __r
 // with the least of it; ties go to the taller tile.  total: rows (pairs) of the matrix; k_splits: ranges
 // of k, each a workgroup of its own; x_rows: rows of activations a workgroup fetches per slice.
 static const int SK_COMPUTE_UNITS = 256;
-static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, long long* cost_out = nullptr) {
+static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, long long* cost_out = nullptr,
+                              int tiles_per_wg = 1) {
   int best = 0;
   long long best_cost = 0;
   for (int q = 4; q >= 1; q--) {
     const int h = q * (8 / unit);                    // rows or pairs per tile
-    const long long wgs = (total + h - 1) / h * k_splits;
-    const long long cost = (wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS * (h * unit + x_rows);
+    const long long wgs = (total + h * tiles_per_wg - 1) / (h * tiles_per_wg) * k_splits;
+    const long long cost = (wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS * (h * unit * tiles_per_wg + x_rows);
     if (best == 0 || cost < best_cost) best = h, best_cost = cost;
   }
   if (cost_out) *cost_out = best_cost;
@@ -516,18 +515,21 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
   const int unit = epilogue == EPI_SWIGLU ? 2 : 1;
   const int total = epilogue == EPI_SWIGLU ? N / 2 : N;
-  // up to 32 tokens: the tile height that fills the chip best; more: whole tiles
-  const int rows = mt == 1 ? skinny_tile_height(total, unit, ky, M <= 8 ? 8 : M <= 16 ? 16 : 32) : 32 / unit;
+  // the tile height that fills the chip best; 33 to 64 tokens and whole slices: also whether two tiles of
+  // W per workgroup, which share the activations, do better than one
+  long long cost1, cost2 = 0;
+  int rows = skinny_tile_height(total, unit, ky, mt == 2 ? 64 : M <= 8 ? 8 : M <= 16 ? 16 : 32, &cost1);
+  const int rows2 = nx == 8 ? skinny_tile_height(total, unit, ky, 64, &cost2, 2) : 0;
+  const bool pair = nx == 8 && cost2 < cost1;
+  if (pair) rows = rows2;
   const int tiles = (total + rows - 1) / rows;
   dim3 grid(tiles, ky, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535 && grid.y <= 65535, "pico_gemm_skinny: too many blocks");
   const float* b0 = bias;
-  // 33 to 64 tokens and enough tiles: two tiles of W per workgroup share the activations
-  const bool pair = nx == 8 && (long long)((tiles + 1) / 2) * ky >= SK_PAIR_MIN_WGS;
   if (pair) {
     dim3 pgrid((tiles + 1) / 2, ky, grid.z);
 #define LAUNCHP(EPI) \
-  gemm_skinny_pair_kernel<EPI><<<pgrid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg)
+  gemm_skinny_pair_kernel<EPI><<<pgrid, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
     if (epilogue == EPI_BF16) LAUNCHP(EPI_BF16);
     else if (epilogue == EPI_F32) LAUNCHP(EPI_F32);
     else LAUNCHP(EPI_SWIGLU);
@@ -686,11 +688,8 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   const int mt = M <= 32 ? 1 : 2;
   int pshift = 0;
   while ((1 << pshift) < P) pshift++;
-  int pairs = 16;
-  if (mt == 1) {                      // 12 pairs would not divide d / 2
-    pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, M <= 8 ? 8 : M <= 16 ? 16 : 32);
-    if (pairs == 12) pairs = 16;
-  }
+  int pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, mt == 2 ? 64 : M <= 8 ? 8 : M <= 16 ? 16 : 32);
+  if (pairs == 12) pairs = 16;        // 12 pairs would not divide d / 2
   dim3 grid((nq + 2 * nkv) * (d / 2 / pairs), 1, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535, "pico_gemm_skinny_rope: too many rows");
   const bool tail = K % 64 != 0;
