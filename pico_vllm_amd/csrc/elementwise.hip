@@ -61,7 +61,7 @@ template <> __device__ __forceinline__ void store4_f32<bf16_t>(bf16_t* p, float4
 }
 
 // VEC: rows are handled four elements at a time (H % 4 == 0, so every row starts on 16 bytes).
-template <typename TD, typename TO, bool VEC>
+template <typename TD, typename TO, bool VEC, int VPT = 4>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    const float* __restrict__ w, TO* __restrict__ out,
                                    const int* __restrict__ rows, int H, float eps, int slabs, size_t slab_stride) {
@@ -75,7 +75,6 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
     // The launch gives a row H / 4 threads (up to 1024), so that a thread holds one group of four
     // elements (up to VPT for a longer row) from the sum of squares to the scaling, and everything
     // it needs (stream, slabs, weight) is requested before it waits for anything.
-    constexpr int VPT = 4;
     const int stride = blockDim.x * 4;
     if (H <= VPT * stride) {
       float4 v[VPT], g[VPT];
@@ -164,9 +163,14 @@ extern "C" int pico_add_rmsnorm(float* resid, const void* delta, int delta_dtype
   if (T == 0) return 0;
   // vector path: one thread per four elements, in whole waves, up to 1024
   const int threads = vec ? min(1024, max(64, (H / 4 + 63) / 64 * 64)) : (H >= 4096 ? 512 : (H >= 1024 ? 256 : 128));
+  // groups of four elements per thread: one where the row fits (fewer registers, more rows in flight)
+  const bool one = vec && H <= threads * 4;
 #define LAUNCH(TD, TO)                                                                                                \
   do {                                                                                                                \
-    if (vec)                                                                                                          \
+    if (one)                                                                                                          \
+      add_rmsnorm_kernel<TD, TO, true, 1><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H,   \
+                                                                     eps, slabs, (size_t)slab_stride);               \
+    else if (vec)                                                                                                     \
       add_rmsnorm_kernel<TD, TO, true><<<T, threads, 0, stream>>>(resid, (const TD*)delta, w, (TO*)out, rows, H, eps, \
                                                                   slabs, (size_t)slab_stride);                       \
     else                                                                                                              \
