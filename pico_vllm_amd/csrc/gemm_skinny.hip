@@ -456,16 +456,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __r
 
 // How many rows of W (pairs of rows for the SwiGLU and rotation epilogues, `unit` = 2 rows) a tile gets:
 // the time of a launch goes with what the fullest compute unit reads, its workgroups' rows of W and the
-// activations that each workgroup reads again, so among 4, 3, 2 and 1 quarters of a tile take the height
-// with the least of it; ties go to the taller tile.  total: rows (pairs) of the matrix; k_splits: ranges
+// activations that each workgroup reads again, so take the height with the least of it (a tile taller than
+// 32 rows, whose blocks share the activations, would read less still, but left with one workgroup of few
+// slices in flight per compute unit it measured slower); ties go to the taller tile.  total: rows (pairs) of the matrix; k_splits: ranges
 // of k, each a workgroup of its own; x_rows: rows of activations a workgroup fetches per slice.
 static const int SK_COMPUTE_UNITS = 256;
 static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, long long* cost_out = nullptr,
-                              int tiles_per_wg = 1) {
+                              int tiles_per_wg = 1, int step = 1) {
   int best = 0;
   long long best_cost = 0;
-  for (int q = 4; q >= 1; q--) {
-    const int h = q * (8 / unit);                    // rows or pairs per tile
+  for (int h = 32 / unit; h >= 1; h -= step) {       // rows or pairs per tile
     const long long wgs = (total + h * tiles_per_wg - 1) / (h * tiles_per_wg) * k_splits;
     const long long cost = (wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS * (h * unit * tiles_per_wg + x_rows);
     if (best == 0 || cost < best_cost) best = h, best_cost = cost;
@@ -688,8 +688,9 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   const int mt = M <= 32 ? 1 : 2;
   int pshift = 0;
   while ((1 << pshift) < P) pshift++;
-  int pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, mt == 2 ? 64 : M <= 8 ? 8 : M <= 16 ? 16 : 32);
-  if (pairs == 12) pairs = 16;        // 12 pairs would not divide d / 2
+  // 16, 12, 8 or 4 pairs a tile; 12 would not divide d / 2
+  int pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, mt == 2 ? 64 : M <= 8 ? 8 : M <= 16 ? 16 : 32, nullptr, 1, 4);
+  if (pairs == 12) pairs = 16;
   dim3 grid((nq + 2 * nkv) * (d / 2 / pairs), 1, (M + 32 * mt - 1) / (32 * mt));
   PICO_REQUIRE(grid.z <= 65535, "pico_gemm_skinny_rope: too many rows");
   const bool tail = K % 64 != 0;
