@@ -461,13 +461,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __r
 // slices in flight per compute unit it measured slower); ties go to the taller tile.  total: rows (pairs) of the matrix; k_splits: ranges
 // of k, each a workgroup of its own; x_rows: rows of activations a workgroup fetches per slice.
 static const int SK_COMPUTE_UNITS = 256;
-static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, long long* cost_out = nullptr,
+static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, double* cost_out = nullptr,
                               int tiles_per_wg = 1, int step = 1) {
   int best = 0;
-  long long best_cost = 0;
+  double best_cost = 0;
   for (int h = 32 / unit; h >= 1; h -= step) {       // rows or pairs per tile
     const long long wgs = (total + h * tiles_per_wg - 1) / (h * tiles_per_wg) * k_splits;
-    const long long cost = (wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS * (h * unit * tiles_per_wg + x_rows);
+    // whole rounds of workgroups while they are few; many rounds run into one another
+    const double rounds = wgs <= 4 * SK_COMPUTE_UNITS ? (double)((wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS)
+                                                      : (double)wgs / SK_COMPUTE_UNITS;
+    const double cost = rounds * (h * unit * tiles_per_wg + x_rows);
     if (best == 0 || cost < best_cost) best = h, best_cost = cost;
   }
   if (cost_out) *cost_out = best_cost;
@@ -480,11 +483,11 @@ static int skinny_tile_height(long long total, int unit, int k_splits, int x_row
 // of tokens, so that a token's sums are formed in the same order whatever comes with it.
 extern "C" int pico_gemm_skinny_k_splits(int N, int K, int max_splits) {
   int best = 1;
-  long long best_cost = 0;
+  double best_cost = 0;
   for (int want = 1; want <= max_splits; want++) {
     const int per = ((K + want - 1) / want + 255) / 256 * 256;
     if ((K + per - 1) / per != want) continue;       // ranges would be empty
-    long long cost;
+    double cost;
     skinny_tile_height(N, 1, want, 8, &cost);
     cost *= per;
     if (want == 1 || cost < best_cost) best = want, best_cost = cost;
@@ -517,7 +520,7 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   const int total = epilogue == EPI_SWIGLU ? N / 2 : N;
   // the tile height that fills the chip best; 33 to 64 tokens and whole slices: also whether two tiles of
   // W per workgroup, which share the activations, do better than one
-  long long cost1, cost2 = 0;
+  double cost1, cost2 = 0;
   int rows = skinny_tile_height(total, unit, ky, mt == 2 ? 64 : M <= 8 ? 8 : M <= 16 ? 16 : 32, &cost1);
   const int rows2 = nx == 8 ? skinny_tile_height(total, unit, ky, 64, &cost2, 2) : 0;
   const bool pair = nx == 8 && cost2 < cost1;
