@@ -5,7 +5,7 @@
 //                    and values of the sequence stream through LDS in tiles, from position 0 to the
 //                    causal frontier.  A decode token is a sequence that brings one query.
 //                    D % 32 == 0: prefill16_kernel, 64 queries per workgroup, 16 per wave
-//                    (v_mfma_f32_16x16x32_bf16), one or two teams of four waves that share the key loop;
+//                    (v_mfma_f32_16x16x32_bf16), one to three teams of four waves that share the key loop;
 //                    other D: prefill_kernel, 128 queries per workgroup, 32 per wave (32x32x16).
 //   decode           one workgroup per (sequence, kv head, split of the context); the
 //                    "queries" are the G query heads that share the kv head, so keys and values
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void prefill_kernel(
 // ---------------------------------------------------------------------------
 // v_mfma_f32_16x16x32_bf16 (A 16x32, B 32x16): lane l = (c, kq) = (l % 16, l / 16) supplies
 // A[c][8 kq + 0..7] and B[8 kq + 0..7][c] and receives D[4 kq + r][c] in register r.
-// A workgroup owns 64 queries of one sequence and one head.  Its waves form KT teams of four;
+// A workgroup owns 64 queries of one sequence and one head.  Its waves form KT (1 to 3) teams of four;
 // the four waves of a team own 16 queries each, and team t works on keys 64 t .. 64 t + 63 of every
 // LDS tile of 64 KT keys, so the long key loop of a late query tile is shared by KT waves per
 // SIMD whose softmax and matrix products overlap; the teams' results are merged through LDS at the
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void prefill_kernel(
 #if PICO_HEAD_DIM % 32 == 0
 typedef float f32x4p __attribute__((ext_vector_type(4)));
 constexpr int PF_BM = 64;                         // queries per workgroup
-constexpr int PF_KT_MAX = D <= 128 ? 2 : 1;       // teams of four waves: one or two
+constexpr int PF_KT_MAX = D <= 128 ? 2 : 1;       // 2: one, two or three teams of four waves; 1: one team
 constexpr int PF_KS = D / 32;                     // contraction steps of a 16-key block
 constexpr int PF_DT = D / 16;                     // 16-wide tiles of the output's head dimension
 
@@ -550,10 +550,10 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
 }
 
 // grid: x = query head, y = (sequence, 64-query tile), late (long) tiles first.  One team keeps three
-// workgroups on a compute unit, which serves many long, equal tiles best; two teams halve the key
+// workgroups on a compute unit, which serves many long, equal tiles best; two or three teams cut the key
 // loop of the longest tile, which decides when the tiles are few or unequal (a causal triangle).
 template <int KT>
-__global__ __launch_bounds__(256 * KT, KT == 1 ? 3 : 2) void prefill16_kernel(
+__global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
@@ -1021,6 +1021,10 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
       prefill16_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                                    (const bf16_t*)v_cache, block_table, max_pages, cu_seqlens,
                                                    context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+    else if (teams == 3 && PF_KT_MAX == 2)
+      prefill16_kernel<PF_KT_MAX == 2 ? 3 : 1><<<grid, 768, 0, stream>>>(
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
+          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
     else
       prefill16_kernel<PF_KT_MAX><<<grid, 256 * PF_KT_MAX, 0, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,

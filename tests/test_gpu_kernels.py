@@ -333,12 +333,12 @@ def test_fast_prefill_other_sizes_and_long_portions(K, nq, nkv, d, Pg):
     close(out, want, torch.bfloat16)
 
 
-@pytest.mark.parametrize("teams", [1, 2])
+@pytest.mark.parametrize("teams", [1, 2, 3])
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64)])
-def test_fast_prefill_with_one_and_two_key_teams(K, nq, nkv, d, Pg, teams):
+def test_fast_prefill_with_one_to_three_key_teams(K, nq, nkv, d, Pg, teams):
     # the number of waves that share a query tile's key loop is a hint: every value gives the same attention;
-    # lengths around the 64-query tile and the 64- and 128-key tiles of one and two teams
-    out, want = _fast_case([63, 1, 65, 130, 2, 200], [0, 127, 1, 62, 191, 129], nq, nkv, d, Pg, seed=5, teams=teams)
+    # lengths around the 64-query tile and the 64-, 128- and 192-key tiles of one to three teams
+    out, want = _fast_case([63, 1, 65, 130, 2, 200, 193], [0, 127, 1, 62, 191, 129, 383], nq, nkv, d, Pg, seed=5, teams=teams)
     close(out, want, torch.bfloat16)
 
 
@@ -356,9 +356,9 @@ def test_fast_prefill_chooses_teams_by_the_shape_of_the_batch():
     from pico_vllm_amd.ops.attention_fast import FastAttention
     fa = FastAttention.__new__(FastAttention)
     fa.nq = 12
-    assert fa.prefill_teams([2048], [2048]) == 2            # a causal triangle: the longest tile decides
-    assert fa.prefill_teams([512], [4096]) == 2             # few tiles
-    assert fa.prefill_teams([1] * 8, [4000] * 8) == 2       # decode tokens inside a mixed step
+    assert fa.prefill_teams([2048], [2048]) == 3            # a causal triangle: the longest tile decides
+    assert fa.prefill_teams([512], [4096]) == 3             # few tiles
+    assert fa.prefill_teams([1] * 8, [4000] * 8) == 3       # decode tokens inside a mixed step
     assert fa.prefill_teams([2048], [16384]) == 1           # many long, equal tiles
 
 
