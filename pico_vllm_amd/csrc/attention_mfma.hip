@@ -420,6 +420,52 @@ struct PfFetch {
   static constexpr int N = D / 32;          // chunks of K and of V^T per thread
   u32x4 k[N], v[N];                         // plain vectors: a struct copy would go through memory
   int page_k[N], page_v;
+  // What does not change from tile to tile, for whole tiles (every key exists) of pages of 8 or 16 keys:
+  // the thread's chunks of K are 16 KT keys apart, whole pages, so they sit at the same place k_in
+  // (in bytes) inside their pages and their page numbers stand 16 KT / P entries apart in the block table,
+  // the first at byte k_bt of the tile's entries; v_in and v_bt likewise for its chunks of V^T.
+  uint32_t k_in, v_in, k_bt, v_bt;
+
+  __device__ __forceinline__ void init(int g, int nkv, int pshift) {
+    const int P = 1 << pshift;
+    const int key = (int)threadIdx.x / KCH;
+    k_in = (((uint32_t)g << pshift) + (key & (P - 1))) * (2 * D) + ((int)threadIdx.x % KCH) * 16;
+    k_bt = (uint32_t)(key >> pshift) * 4;
+    const int vkey = 8 * ((int)threadIdx.x % VCH);
+    v_in = ((((uint32_t)g * D + threadIdx.x / VCH) << pshift) + (vkey & (P - 1))) * 2;
+    v_bt = (uint32_t)(vkey >> pshift) * 4;
+  }
+  // bt_tile: the block table at the tile's first page
+  __device__ __forceinline__ void load_pages_full(const int* __restrict__ bt_tile, int pshift, int num_pages) {
+    const char* b = reinterpret_cast<const char*>(bt_tile);
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      page_k[i] = min(max(*reinterpret_cast<const int*>(b + (size_t)((((PF_NT / KCH) * i) >> pshift) * 4) + k_bt), 0), num_pages - 1);
+    page_v = min(max(*reinterpret_cast<const int*>(b + v_bt), 0), num_pages - 1);
+  }
+  // page_bytes: bytes of one page of K (and of V): nkv * P * D * 2, below 2^24 (the caller has checked)
+  __device__ __forceinline__ void fetch_full(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                                             uint32_t page_bytes, int pshift) {
+    const char* kb = reinterpret_cast<const char*>(k_cache);
+    const char* vb = reinterpret_cast<const char*>(v_cache);
+#pragma unroll
+    for (int i = 0; i < N; i++) k[i] = *reinterpret_cast<const u32x4*>(kb + (__umul24(page_k[i], page_bytes) + k_in));
+    const uint32_t off0 = __umul24(page_v, page_bytes) + v_in;
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      v[i] = *reinterpret_cast<const u32x4*>(vb + (size_t)((uint32_t)((PF_NT / VCH) * i) << (pshift + 1)) + off0);
+  }
+  __device__ __forceinline__ void commit_full(PfTiles<KT>& t) const {
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int c = threadIdx.x + PF_NT * i;
+      *reinterpret_cast<u32x4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
+    }
+    const int kc = threadIdx.x % VCH;
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      *reinterpret_cast<u32x4*>(&t.vt[(threadIdx.x / VCH + (PF_NT / VCH) * i) * PF_VROW + kc * 8]) = v[i];
+  }
 
   // chunk i of this thread: K chunk c = tid + PF_NT i is key c / KCH, part c % KCH; V^T chunk c is
   // head dimension c / VCH, keys 8 (c % VCH) .. + 7, and c % VCH = tid % VCH for every i.
@@ -603,19 +649,18 @@ __global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
   const bf16_t* krow = &tiles.k[(64 * team + 8 * (col >> 2) + (col & 3)) * KROW + 8 * kq];
   const bf16_t* vrow = &tiles.vt[col * PF_VROW + 64 * team + 8 * kq];
   PfFetch<KT> regs;
+  // Whole tiles of pages of 8 or 16 keys take the short way: no clamping of positions, nothing to mask,
+  // addresses from what init() has prepared.  The last tiles and other pages go the long way.  Two loops
+  // and no branch inside them: a branch between the loads would force a wait for the ones before it.
+  const uint32_t page_bytes = ((uint32_t)nkv << pshift) * (2 * D);
+  const int n_full = (pshift <= 4 && page_bytes < (1u << 24) && num_pages < (1 << 24)) ? kv_end / PF_TK : 0;
+  regs.init(g, nkv, pshift);
   regs.load_pages(bt, pshift, num_pages, 0, kv_end);
   regs.fetch(k_cache, v_cache, g, nkv, pshift, 0, kv_end);
   regs.load_pages(bt, pshift, num_pages, PF_TK, kv_end);
-  for (int tile_start = 0; tile_start < kv_end; tile_start += PF_TK) {
-    __syncthreads();                                            // everyone is done with the previous tile
-    regs.commit(tiles, tile_start, kv_end);
-    __syncthreads();
-    // the next tile's keys and values (clamped to the last key if there is no next tile) and the
-    // page numbers of the tile after it; no branch, so no wait is forced here
-    regs.fetch(k_cache, v_cache, g, nkv, pshift, tile_start + PF_TK, kv_end);
-    regs.load_pages(bt, pshift, num_pages, tile_start + 2 * PF_TK, kv_end);
+  auto attend = [&](int tile_start) {
     const int key0 = tile_start + 64 * team;                    // this team's keys
-    if (!wave_active || key0 > wave_last_pos) continue;
+    if (!wave_active || key0 > wave_last_pos) return;
     if (key0 + 63 <= wave_first_pos) {
       pf_attend<2, false, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
     } else if (key0 + 32 <= wave_last_pos) {
@@ -623,6 +668,25 @@ __global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
     } else {   // the second pair of 16-key blocks lies wholly beyond the causal frontier of this wave
       pf_attend<1, true, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
     }
+  };
+  int ti = 0;
+  for (; ti + 2 < n_full; ti++) {            // this tile, the next and the one after it are whole
+    __syncthreads();                                            // everyone is done with the previous tile
+    regs.commit_full(tiles);
+    __syncthreads();
+    regs.fetch_full(k_cache, v_cache, page_bytes, pshift);
+    regs.load_pages_full(bt + (((ti + 2) * PF_TK) >> pshift), pshift, num_pages);
+    attend(ti * PF_TK);
+  }
+  for (int tile_start = ti * PF_TK; tile_start < kv_end; tile_start += PF_TK) {
+    __syncthreads();
+    regs.commit(tiles, tile_start, kv_end);
+    __syncthreads();
+    // the next tile's keys and values (clamped to the last key if there is no next tile) and the
+    // page numbers of the tile after it
+    regs.fetch(k_cache, v_cache, g, nkv, pshift, tile_start + PF_TK, kv_end);
+    regs.load_pages(bt, pshift, num_pages, tile_start + 2 * PF_TK, kv_end);
+    attend(tile_start);
   }
   if (KT > 1) {
     // merge the teams through LDS (reusing the tile memory): lane-wise, the layouts agree
