@@ -4,7 +4,7 @@
 //   prefill / mixed  a workgroup owns a tile of query tokens of one sequence and one query head; keys
 //                    and values of the sequence stream through LDS in tiles, from position 0 to the
 //                    causal frontier.  A decode token is a sequence that brings one query.
-//                    D % 32 == 0: prefill16_kernel, 64 queries per workgroup, 16 per wave
+//                    D % 32 == 0: prefill16_kernel, 64 (or 128) queries per workgroup, 16 (or 2 x 16) per wave
 //                    (v_mfma_f32_16x16x32_bf16), one to three teams of four waves that share the key loop;
 //                    other D: prefill_kernel, 128 queries per workgroup, 32 per wave (32x32x16).
 //   decode           one workgroup per (sequence, kv head, split of the context); the
@@ -530,67 +530,77 @@ struct PfState {
   f32x4p o[PF_DT];     // O^T tiles: rows = head dimension, column = query
 };
 
-// The 64 keys of one team (its first NPAIR pairs of 16-key blocks) against the wave's 16 query
-// columns, one softmax update: raw scores, p = 2^(s c - m c) with c = scale * log2(e); the reference
+// The 64 keys of one team (its first NPAIR pairs of 16-key blocks) against the wave's NQB blocks of 16 query
+// columns (every operand read from LDS serves the NQB blocks), one softmax update per block: raw scores,
+// p = 2^(s c - m c) with c = scale * log2(e); the reference
 // maximum may lag behind the running maximum by up to 8 in the exponent and the accumulators are
 // rescaled only when a column of the wave outgrows that (see attend_tile).
 // krow: row 8 (col / 4) + col % 4 of the team's keys in LDS, vrow: row col of V^T at the team's keys,
 // both at this lane quarter's 16 bytes; key_pos0: position of the team's first key.
-template <int NPAIR, bool MASK, int PF_VROW>
-__device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow, const bf16x8* q, PfState& st, float c,
-                                          int key_pos0, int q_pos) {
+template <int NPAIR, bool MASK, int PF_VROW, int NQB>
+__device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow, const bf16x8 (&q)[NQB][PF_KS],
+                                          PfState (&st)[NQB], float c, int key_pos0, const int (&q_pos)[NQB]) {
   const int kq = (threadIdx.x & 63) >> 4;
-  f32x4p s[2 * NPAIR];
+  f32x4p s[NQB][2 * NPAIR];
 #pragma unroll
   for (int j = 0; j < 2 * NPAIR; j++) {
-    s[j] = f32x4p{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < NQB; b++) s[b][j] = f32x4p{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int step = 0; step < PF_KS; step++) {
       const bf16x8 a = __builtin_bit_cast(
           bf16x8, *reinterpret_cast<const u32x4*>(krow + (32 * (j / 2) + 4 * (j % 2)) * KROW + 32 * step));
-      s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[step], s[j], 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < NQB; b++) s[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[b][step], s[b][j], 0, 0, 0);
     }
   }
-  float mx = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < 2 * NPAIR; j++)
+  for (int b = 0; b < NQB; b++) {
+    float mx = -INFINITY;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      if (MASK && key_pos0 + 32 * (j / 2) + 8 * kq + 4 * (j % 2) + r > q_pos) s[j][r] = -INFINITY;
-      mx = fmaxf(mx, s[j][r]);
+    for (int j = 0; j < 2 * NPAIR; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        if (MASK && key_pos0 + 32 * (j / 2) + 8 * kq + 4 * (j % 2) + r > q_pos[b]) s[b][j][r] = -INFINITY;
+        mx = fmaxf(mx, s[b][j][r]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(st[b].m, mx);
+    const bool outgrown = (m_new - st[b].m) * c > 8.0f;        // also true while the reference is -inf
+    if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {          // the same decision for the whole wave
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((st[b].m - m_use) * c);
+      st[b].l *= alpha;
+      st[b].m = m_new;
+#pragma unroll
+      for (int tt = 0; tt < PF_DT; tt++) st[b].o[tt] *= alpha;
     }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  const float m_new = fmaxf(st.m, mx);
-  const bool outgrown = (m_new - st.m) * c > 8.0f;           // also true while the reference is -inf
-  if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {          // the same decision for the whole wave
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f((st.m - m_use) * c);
-    st.l *= alpha;
-    st.m = m_new;
+    const float mc = ((st[b].m == -INFINITY) ? 0.f : st[b].m) * c;
+    float sum = 0.f;
 #pragma unroll
-    for (int tt = 0; tt < PF_DT; tt++) st.o[tt] *= alpha;
+    for (int j = 0; j < 2 * NPAIR; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[b][j][r], c, -mc));
+        s[b][j][r] = p;
+        sum += p;
+      }
+    st[b].l += sum;
   }
-  const float mc = ((st.m == -INFINITY) ? 0.f : st.m) * c;
-  float sum = 0.f;
-#pragma unroll
-  for (int j = 0; j < 2 * NPAIR; j++)
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const float p = __builtin_amdgcn_exp2f(fmaf(s[j][r], c, -mc));
-      s[j][r] = p;
-      sum += p;
-    }
-  st.l += sum;
 #pragma unroll
   for (int m = 0; m < NPAIR; m++) {
-    const bf16x8 b = __builtin_bit_cast(
-        bf16x8, u32x4{pack2_bf16(s[2 * m][0], s[2 * m][1]), pack2_bf16(s[2 * m][2], s[2 * m][3]),
-                      pack2_bf16(s[2 * m + 1][0], s[2 * m + 1][1]), pack2_bf16(s[2 * m + 1][2], s[2 * m + 1][3])});
+    bf16x8 pb[NQB];
+#pragma unroll
+    for (int b = 0; b < NQB; b++)
+      pb[b] = __builtin_bit_cast(
+          bf16x8, u32x4{pack2_bf16(s[b][2 * m][0], s[b][2 * m][1]), pack2_bf16(s[b][2 * m][2], s[b][2 * m][3]),
+                        pack2_bf16(s[b][2 * m + 1][0], s[b][2 * m + 1][1]), pack2_bf16(s[b][2 * m + 1][2], s[b][2 * m + 1][3])});
 #pragma unroll
     for (int tt = 0; tt < PF_DT; tt++) {
       const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(vrow + 16 * tt * PF_VROW + 32 * m));
-      st.o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, st.o[tt], 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < NQB; b++) st[b].o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[b], st[b].o[tt], 0, 0, 0);
     }
   }
 }
@@ -598,17 +608,22 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
 // grid: x = query head, y = (sequence, 64-query tile), late (long) tiles first.  One team keeps three
 // workgroups on a compute unit, which serves many long, equal tiles best; two or three teams cut the key
 // loop of the longest tile, which decides when the tiles are few or unequal (a causal triangle).
-template <int KT>
-__global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
+// NQB = 2 (one team only): a wave owns two blocks of 16 queries and a workgroup 128, so every K and V^T
+// operand read from LDS feeds two products; LDS traffic, which bounds the kernel when there is work for
+// every compute unit, halves per product, at the price of registers for two waves per SIMD.
+template <int KT, int NQB = 1>
+__global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefill16_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
     float scale) {
+  static_assert(NQB == 1 || KT == 1, "two query blocks a wave: one team");
   constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
+  constexpr int BMQ = PF_BM * NQB;            // queries per workgroup
   __shared__ PfTiles<KT> tiles;
   int b = 0, tile = (int)blockIdx.y, ntiles = 0;
   for (; b < num_seqs; b++) {
-    ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
+    ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + BMQ - 1) / BMQ;
     if (tile < ntiles) break;
     tile -= ntiles;
   }
@@ -621,31 +636,38 @@ __global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
   const int lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
   const int* bt = block_table + (size_t)b * max_pages;
 
-  const int q_idx = tile * PF_BM + wave * 16 + col;            // index among the sequence's new tokens
-  const bool q_ok = q_idx < new_len;
-  const int q_pos = prefix + q_idx;
-  bf16x8 qf[PF_KS];
-  {
-    const bf16_t* qrow = q + (size_t)(tok0 + (q_ok ? q_idx : 0)) * q_stride + (size_t)head * D + 8 * kq;
+  const int wave_q0 = tile * BMQ + wave * 16 * NQB;            // the wave's first query among the sequence's new tokens
+  int q_idx[NQB], q_pos[NQB];
+  bool q_ok[NQB];
+  bf16x8 qf[NQB][PF_KS];
+#pragma unroll
+  for (int qb = 0; qb < NQB; qb++) {
+    q_idx[qb] = wave_q0 + 16 * qb + col;
+    q_ok[qb] = q_idx[qb] < new_len;
+    q_pos[qb] = prefix + q_idx[qb];
+    const bf16_t* qrow = q + (size_t)(tok0 + (q_ok[qb] ? q_idx[qb] : 0)) * q_stride + (size_t)head * D + 8 * kq;
 #pragma unroll
     for (int step = 0; step < PF_KS; step++) {
       u32x4 v = u32x4{0, 0, 0, 0};
-      if (q_ok) v = *reinterpret_cast<const u32x4*>(qrow + 32 * step);
-      qf[step] = __builtin_bit_cast(bf16x8, v);
+      if (q_ok[qb]) v = *reinterpret_cast<const u32x4*>(qrow + 32 * step);
+      qf[qb][step] = __builtin_bit_cast(bf16x8, v);
     }
   }
-  const int wave_first_pos = prefix + tile * PF_BM + wave * 16;         // lowest query position of the wave
-  const int wave_last_pos = min(wave_first_pos + 15, ctx - 1);          // highest real one
-  const bool wave_active = tile * PF_BM + wave * 16 < new_len;
-  const int kv_end = min(ctx, prefix + min(new_len, (tile + 1) * PF_BM));  // keys beyond the tile's last query are never needed
+  const int wave_first_pos = prefix + wave_q0;                              // lowest query position of the wave
+  const int wave_last_pos = min(wave_first_pos + 16 * NQB - 1, ctx - 1);    // highest real one
+  const bool wave_active = wave_q0 < new_len;
+  const int kv_end = min(ctx, prefix + min(new_len, (tile + 1) * BMQ));   // keys beyond the tile's last query are never needed
 
   const float c = scale * 1.4426950408889634f;                 // scores go through 2^x
   const int pshift = 31 - __clz(P);                            // page sizes are powers of two
-  PfState st;
-  st.m = -INFINITY;
-  st.l = 0.f;
+  PfState st[NQB];
 #pragma unroll
-  for (int tt = 0; tt < PF_DT; tt++) st.o[tt] = f32x4p{0.f, 0.f, 0.f, 0.f};
+  for (int qb = 0; qb < NQB; qb++) {
+    st[qb].m = -INFINITY;
+    st[qb].l = 0.f;
+#pragma unroll
+    for (int tt = 0; tt < PF_DT; tt++) st[qb].o[tt] = f32x4p{0.f, 0.f, 0.f, 0.f};
+  }
   const bf16_t* krow = &tiles.k[(64 * team + 8 * (col >> 2) + (col & 3)) * KROW + 8 * kq];
   const bf16_t* vrow = &tiles.vt[col * PF_VROW + 64 * team + 8 * kq];
   PfFetch<KT> regs;
@@ -662,11 +684,11 @@ __global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
     const int key0 = tile_start + 64 * team;                    // this team's keys
     if (!wave_active || key0 > wave_last_pos) return;
     if (key0 + 63 <= wave_first_pos) {
-      pf_attend<2, false, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
+      pf_attend<2, false, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
     } else if (key0 + 32 <= wave_last_pos) {
-      pf_attend<2, true, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
+      pf_attend<2, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
     } else {   // the second pair of 16-key blocks lies wholly beyond the causal frontier of this wave
-      pf_attend<1, true, PF_VROW>(krow, vrow, qf, st, c, key0, q_pos);
+      pf_attend<1, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
     }
   };
   int ti = 0;
@@ -688,8 +710,9 @@ __global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
     regs.load_pages(bt, pshift, num_pages, tile_start + 2 * PF_TK, kv_end);
     attend(tile_start);
   }
-  if (KT > 1) {
+  if constexpr (KT > 1) {
     // merge the teams through LDS (reusing the tile memory): lane-wise, the layouts agree
+    PfState& s0 = st[0];
     __syncthreads();
     float* xo = reinterpret_cast<float*>(&tiles);              // [team - 1][wave][PF_DT * 4 + 2][64 lanes]
     constexpr int PER_WAVE = (PF_DT * 4 + 2) * 64;
@@ -700,43 +723,46 @@ __global__ __launch_bounds__(256 * KT, KT == 2 ? 2 : 3) void prefill16_kernel(
 #pragma unroll
       for (int tt = 0; tt < PF_DT; tt++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) mine[(4 * tt + r) * 64] = st.o[tt][r];
-      mine[(PF_DT * 4) * 64] = st.m;
-      mine[(PF_DT * 4 + 1) * 64] = st.l;
+        for (int r = 0; r < 4; r++) mine[(4 * tt + r) * 64] = s0.o[tt][r];
+      mine[(PF_DT * 4) * 64] = s0.m;
+      mine[(PF_DT * 4 + 1) * 64] = s0.l;
     }
     __syncthreads();
     if (team > 0) return;
-    float M = st.m;
+    float M = s0.m;
 #pragma unroll
     for (int t = 1; t < KT; t++) M = fmaxf(M, xo[((t - 1) * 4 + wave) * PER_WAVE + (PF_DT * 4) * 64 + lane]);
     const float m_use = (M == -INFINITY) ? 0.f : M;
-    const float a0 = __builtin_amdgcn_exp2f((st.m - m_use) * c);
-    st.l *= a0;
+    const float a0 = __builtin_amdgcn_exp2f((s0.m - m_use) * c);
+    s0.l *= a0;
 #pragma unroll
-    for (int tt = 0; tt < PF_DT; tt++) st.o[tt] *= a0;
+    for (int tt = 0; tt < PF_DT; tt++) s0.o[tt] *= a0;
 #pragma unroll
     for (int t = 1; t < KT; t++) {
       const float* theirs = xo + ((t - 1) * 4 + wave) * PER_WAVE + lane;
       const float at = __builtin_amdgcn_exp2f((theirs[(PF_DT * 4) * 64] - m_use) * c);
-      st.l += at * theirs[(PF_DT * 4 + 1) * 64];
+      s0.l += at * theirs[(PF_DT * 4 + 1) * 64];
 #pragma unroll
       for (int tt = 0; tt < PF_DT; tt++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) st.o[tt][r] += at * theirs[(4 * tt + r) * 64];
+        for (int r = 0; r < 4; r++) s0.o[tt][r] += at * theirs[(4 * tt + r) * 64];
     }
   }
-  if (!q_ok) return;
-  float l = st.l;
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  const float inv_l = 1.0f / l;
-  bf16_t* orow = out + ((size_t)(tok0 + q_idx) * nq + head) * D + 4 * kq;
 #pragma unroll
-  for (int tt = 0; tt < PF_DT; tt++) {
-    uint2 v;
-    v.x = pack2_bf16(st.o[tt][0] * inv_l, st.o[tt][1] * inv_l);
-    v.y = pack2_bf16(st.o[tt][2] * inv_l, st.o[tt][3] * inv_l);
-    *reinterpret_cast<uint2*>(orow + 16 * tt) = v;
+  for (int qb = 0; qb < NQB; qb++) {
+    if (!q_ok[qb]) continue;
+    float l = st[qb].l;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const float inv_l = 1.0f / l;
+    bf16_t* orow = out + ((size_t)(tok0 + q_idx[qb]) * nq + head) * D + 4 * kq;
+#pragma unroll
+    for (int tt = 0; tt < PF_DT; tt++) {
+      uint2 v;
+      v.x = pack2_bf16(st[qb].o[tt][0] * inv_l, st[qb].o[tt][1] * inv_l);
+      v.y = pack2_bf16(st[qb].o[tt][2] * inv_l, st[qb].o[tt][3] * inv_l);
+      *reinterpret_cast<uint2*>(orow + 16 * tt) = v;
+    }
   }
 }
 #endif
@@ -1081,7 +1107,12 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
     const int max_tiles = num_tokens / PF_BM + num_seqs;  // >= sum over sequences of ceil(len / PF_BM)
     PICO_REQUIRE(max_tiles <= 65535, "pico_attn_prefill: %d tokens are too many for one launch", num_tokens);
     dim3 grid(nq, max_tiles);
-    if (teams == 1 || PF_KT_MAX == 1)
+    if (teams == 4 && PF_KT_MAX == 2) {      // 128 queries a workgroup, two blocks of 16 a wave
+      grid.y = num_tokens / (2 * PF_BM) + num_seqs;
+      prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 256, 0, stream>>>(
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
+          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+    } else if (teams == 1 || PF_KT_MAX == 1)
       prefill16_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                                    (const bf16_t*)v_cache, block_table, max_pages, cu_seqlens,
                                                    context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);

@@ -32,18 +32,26 @@ class FastAttention:
         return max(1, min(by_fill, by_len, 64))
 
     def prefill_teams(self, new_lens, context_lens) -> int:
-        """How many teams of four waves share the key loop of a 64-query tile: three cut the longest
-        workgroup's loop to a third, which decides while the work (in 64 x 64 tiles) would not keep 256
-        compute units busy for the time the longest tile takes (41.9 us against 44.2 with two teams and
-        57.5 with one for 2,048 tokens of 12 heads); one leaves room for three workgroups per unit, which
-        serves many long tiles best (230 against 311 us for eight such prompts)."""
-        longest, total = 1, 0
+        """The shape of the prefill workgroups.  1 to 3: teams of four waves that share the key loop of a
+        64-query tile; three cut the longest workgroup's loop to a third, which decides while the work (in
+        64 x 64 tiles) would not keep 256 compute units busy for the time the longest tile takes (41 us
+        against 43 with two teams and 52 with one for 2,048 tokens of 12 heads); one leaves room for three
+        workgroups per unit, which serves many long tiles best (214 against 308 us for eight such prompts).
+        4: one team whose waves own two blocks of 16 queries, 128 queries a workgroup: half the LDS traffic
+        per product, which is the bound when every compute unit has plenty to do (184 us for the eight
+        prompts, 622 against 825 us for four portions of 2,048 tokens after 2,048 with 40 heads), but coarser
+        tiles, so only for much work in portions that fill them."""
+        longest, total, tokens, padded = 1, 0, 0, 0
         for n, c in zip(new_lens, context_lens):
             n, c = int(n), int(c)
             tiles = -(-n // 64)
             longest = max(longest, -(-c // 64))
             total += tiles * max(1, (2 * c - n) // 128)      # mean key tiles of the portion's query tiles
-        return 1 if total * self.nq >= 256 * longest else 3
+            tokens += n
+            padded += -(-n // 128) * 128
+        if total * self.nq < 256 * longest:
+            return 3
+        return 4 if total * self.nq >= 256 * 64 and 4 * tokens >= 3 * padded else 1
 
     def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
                 scale: float, out: Optional[torch.Tensor] = None, teams: int = 0) -> torch.Tensor:

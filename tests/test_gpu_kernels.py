@@ -333,12 +333,14 @@ def test_fast_prefill_other_sizes_and_long_portions(K, nq, nkv, d, Pg):
     close(out, want, torch.bfloat16)
 
 
-@pytest.mark.parametrize("teams", [1, 2, 3])
-@pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64)])
-def test_fast_prefill_with_one_to_three_key_teams(K, nq, nkv, d, Pg, teams):
-    # the number of waves that share a query tile's key loop is a hint: every value gives the same attention;
-    # lengths around the 64-query tile and the 64-, 128- and 192-key tiles of one to three teams
-    out, want = _fast_case([63, 1, 65, 130, 2, 200, 193], [0, 127, 1, 62, 191, 129, 383], nq, nkv, d, Pg, seed=5, teams=teams)
+@pytest.mark.parametrize("teams", [1, 2, 3, 4])
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64), (4, 1, 96, 32)])
+def test_fast_prefill_with_every_shape_of_workgroup(K, nq, nkv, d, Pg, teams):
+    # the shape of the workgroups (1 to 3 teams on a 64-query tile, 4: two query blocks a wave, 128-query tiles)
+    # is a hint: every value gives the same attention; lengths around the 64- and 128-query tiles and the
+    # 64-, 128- and 192-key tiles of one to three teams; pages of 8 and 16 keys take the short way in whole tiles
+    out, want = _fast_case([63, 1, 65, 130, 2, 200, 193, 127, 257], [0, 127, 1, 62, 191, 129, 383, 1, 64], nq, nkv, d, Pg, seed=5,
+                           teams=teams)
     close(out, want, torch.bfloat16)
 
 
@@ -359,7 +361,8 @@ def test_fast_prefill_chooses_teams_by_the_shape_of_the_batch():
     assert fa.prefill_teams([2048], [2048]) == 3            # a causal triangle: the longest tile decides
     assert fa.prefill_teams([512], [4096]) == 3             # few tiles
     assert fa.prefill_teams([1] * 8, [4000] * 8) == 3       # decode tokens inside a mixed step
-    assert fa.prefill_teams([2048], [16384]) == 1           # many long, equal tiles
+    assert fa.prefill_teams([2048], [16384]) == 4           # many long, equal tiles that fill 128 queries
+    assert fa.prefill_teams([32] * 64, [2032] * 64) == 1    # much work in short portions
 
 
 def test_fast_prefill_with_a_cache_of_4_gib(K):
