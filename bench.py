@@ -168,6 +168,42 @@ def serve_point(model_dir, dtype, requests, max_new):
             "preemptions": eng.stats["preemptions"]}
 
 
+def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20):
+    """The prefill attention kernel alone on ``nseq`` portions of ``new_len`` tokens after ``prefix`` cached ones,
+    with the shape's heads; ``shape``: what FastAttention.prefill_teams would return, 0 = ask it."""
+    import torch
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    nq, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d, P, dev = cfg["hidden_size"] // nq, 16, "cuda"
+    g = torch.Generator(device=dev).manual_seed(0)
+    ctx = new_len + prefix
+    per = -(-ctx // P)
+    pages = nseq * per + 8
+    kc = torch.randn(pages, nkv, P, d, device=dev, generator=g).bfloat16()
+    vc = torch.randn(pages, nkv, d, P, device=dev, generator=g).bfloat16()
+    bt = torch.randperm(pages, device=dev, generator=g)[: nseq * per].int().reshape(nseq, per).contiguous()
+    q = torch.randn(nseq * new_len, (nq + 2 * nkv) * d, device=dev, generator=g).bfloat16()
+    cu = torch.arange(0, (nseq + 1) * new_len, new_len, dtype=torch.int32, device=dev)
+    cl = torch.full((nseq,), ctx, dtype=torch.int32, device=dev)
+    fa = FastAttention(nq, nkv, d)
+    shape = shape or fa.prefill_teams([new_len] * nseq, [ctx] * nseq)
+    run = lambda: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, teams=shape)
+    out = torch.empty(nseq * new_len, nq * d, dtype=torch.bfloat16, device=dev)
+    run = lambda: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, out=out, teams=shape)
+    for _ in range(5):
+        run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / reps * 1e3
+    flops = 4.0 * nq * d * nseq * (new_len * prefix + new_len * (new_len + 1) / 2)
+    return {"us": round(us, 1), "shape": shape, "tflops": round(flops / us / 1e6, 1), "frac": round(flops / (us * 1e-6) / MFMA_PEAK["bfloat16"], 4)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -187,6 +223,8 @@ def main() -> int:
                     help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once")
     ap.add_argument("--requests", type=int, default=64, help="requests of the serve workload")
     ap.add_argument("--max-new", type=int, default=256, help="new tokens per request of the serve workload")
+    ap.add_argument("--attention", metavar="SEQS,NEW,PREFIX[,SHAPE]", default=None,
+                    help="time only the prefill attention kernel on SEQS portions of NEW tokens after PREFIX cached ones")
     a = ap.parse_args()
     global CONFIG, CONTEXT
     shape_name, full = SHAPES[a.shape]
@@ -205,6 +243,13 @@ def main() -> int:
         return 2
     import torch
     from pico_vllm_amd.weights.random_init import write_random_model
+    if a.attention:
+        nums = [int(x) for x in a.attention.split(",")]
+        r = attention_point(CONFIG, nums[0], nums[1], nums[2], nums[3] if len(nums) > 3 else 0)
+        print(json.dumps({"metric": "prefill attention kernel", "unit": "us", "value": r["us"], "workgroup_shape": r["shape"],
+                          "tflops": r["tflops"], "frac_of_bf16_peak": r["frac"], "sequences": nums[0], "new_tokens": nums[1],
+                          "prefix": nums[2], "heads": CONFIG["num_attention_heads"], "kv_heads": CONFIG["num_key_value_heads"]}))
+        return 0
     if a.write_model:
         write_random_model(a.write_model, CONFIG, seed=0)
         print(f"wrote {a.write_model}")
