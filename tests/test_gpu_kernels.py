@@ -354,6 +354,16 @@ def test_fast_attention_of_a_mixed_step(K, nq, nkv, d, Pg, new_lens, prefix_lens
     close(out, want, torch.bfloat16)
 
 
+def test_fast_attention_of_a_step_with_much_work(K):
+    # eight portions of 256 tokens after 2,048 with 16 heads: the step is served by the workgroups of 128 queries
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    fa = FastAttention.__new__(FastAttention)
+    fa.nq = 16
+    assert fa.prefill_teams([256] * 8, [2304] * 8) == 4
+    out, want = _fast_case([256] * 8, [2048] * 8, 16, 4, 32, 16, seed=13, as_step=True)
+    close(out, want, torch.bfloat16)
+
+
 def test_fast_prefill_chooses_teams_by_the_shape_of_the_batch():
     from pico_vllm_amd.ops.attention_fast import FastAttention
     fa = FastAttention.__new__(FastAttention)
