@@ -313,6 +313,10 @@ def main() -> int:
                 pts[f"decode_b{b}"] = round(r["tok_s"], 1)
                 pts[f"decode_b{b}_hbm_frac"] = round(r["gbps"] * 1e9 / HBM_PEAK, 4)
                 log(f"decode batch {b}: {r['tok_s']:.0f} tok/s, {r['ms_per_step']:.3f} ms/step")
+            if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16":
+                # the one figure the reference publishes for this model: 97 tok/s at batch 1 on its authors' card
+                # (README.md:9,43-45 of the reference); other hardware, so a context, not a baseline
+                pts["decode_b1_vs_reference_published"] = round(pts["decode_b1"] / 97.0, 2)
             out["points"] = pts
         print(json.dumps(out), flush=True)
     finally:
