@@ -2,9 +2,9 @@
 // out = X W^T with X [M <= 64 per launch block, K] and W [N, K] bfloat16, K contiguous in both.
 // The cost is reading W once from HBM, so the kernel is built around that stream:
 //
-//   * a workgroup owns 32 rows of W (one output tile) and one range of k; its waves take
-//     interleaved 64-wide k slices of that range and are summed through LDS in a fixed order,
-//     so the split over k needs no atomics and results are reproducible;
+//   * a workgroup owns up to 32 rows of W (one output tile; how many of the 32 the host decides, see
+//     TileRows) and one range of k; its waves take interleaved 64-wide k slices of that range and are
+//     summed through LDS in a fixed order, so the split over k needs no atomics and results are reproducible;
 //   * a slice of a wave (32 rows x 128 bytes of W, and of the activations as many 8-token groups
 //     as hold tokens) does not go through registers.  A lane that reads its own row of W makes
 //     every load instruction touch 32 cache lines, and the address unit of the compute unit, not
