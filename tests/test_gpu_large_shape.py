@@ -51,7 +51,12 @@ def replay(folder, dtype, steps):
 def test_bfloat16_follows_the_32_bit_path_at_the_1_5b_shape(folder):
     rng = random.Random(1)
     toks = [rng.randrange(SHAPE["vocab_size"]) for _ in range(N)]
-    want = [0, 1, 63, 64, 1000, 2047, 2048, N - 33, N - 1]
+    # after the two large portions come portions of 40, 17 and 9 tokens (the weight-streaming kernels for 33 to 64,
+    # 17 to 32 and 9 to 16 rows at these matrix sizes), then single tokens
+    small = [40, 17, 9]
+    cut = N - 32 - sum(small)                      # where the second large portion ends
+    ends = [cut + sum(small[:i + 1]) - 1 for i in range(len(small))]
+    want = [0, 1, 63, 64, 1000, 2047, 2048] + ends + [N - 1]
     whole = [{"step": 0, "entries": [{"id": "a", "tokens": toks, "want": want}], "end": ["a"]}]
     ref = replay(folder, "float32", whole)[0]
     spread = float(ref.std())
@@ -65,18 +70,28 @@ def test_bfloat16_follows_the_32_bit_path_at_the_1_5b_shape(folder):
         # slice or page gives an error of the order of the spread itself
         assert np.isfinite(got).all() and rms < 5e-2, (label, rms)
 
-    # whole: one step of 2,300 tokens (library GEMMs, two key teams)
+    # whole: one step of 2,300 tokens (library GEMMs, key teams)
     check(replay(folder, "bfloat16", whole)[0], list(range(len(want))), "whole")
-    # portions of 2,048 + 220 (prefix attention), then the last 32 one by one (skinny GEMMs, decode attention)
+    # portions of 2,048 + the rest of the large part (prefix attention), the small portions, then the last 32 one by
+    # one (skinny GEMMs, decode attention)
     steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:2048], "want": [0, 1, 63, 64, 1000, 2047]}], "end": []},
-             {"step": 1, "entries": [{"id": "a", "tokens": toks[2048:N - 32], "want": [0]}], "end": []}]
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[2048:cut], "want": [0]}], "end": []}]
+    at = cut
+    for n in small:
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": toks[at:at + n], "want": [n - 1]}], "end": []})
+        at += n
+    first_single = len(steps)
     for i in range(N - 32, N):
-        steps.append({"step": 2 + i - (N - 32), "entries": [{"id": "a", "tokens": [toks[i]], "want": [0] if i == N - 1 else []}], "end": []})
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": [toks[i]], "want": [0] if i == N - 1 else []}], "end": []})
+    last = len(steps) - 1
+    assert at == N - 32 and last == first_single + 31
     got = replay(folder, "bfloat16", steps)
     check(got[0], [0, 1, 2, 3, 4, 5], "first portion")
     check(got[1], [6], "second portion")
-    check(got[2 + 31], [8], "last token after 32 single steps")
+    for j, n in enumerate(small):
+        check(got[2 + j], [7 + j], f"portion of {n}")
+    check(got[last], [len(want) - 1], "last token after 32 single steps")
     # the 32-bit path itself: portions and single tokens give what the whole prompt gives
     got32 = replay(folder, "float32", steps)
-    for key, rows in ((0, [0, 1, 2, 3, 4, 5]), (1, [6]), (2 + 31, [8])):
+    for key, rows in ((0, [0, 1, 2, 3, 4, 5]), (1, [6]), (2, [7]), (3, [8]), (4, [9]), (last, [len(want) - 1])):
         assert float(np.abs(got32[key] - ref[rows]).max()) <= 2e-4 * spread, key
