@@ -95,3 +95,43 @@ def test_bfloat16_follows_the_32_bit_path_at_the_1_5b_shape(folder):
     got32 = replay(folder, "float32", steps)
     for key, rows in ((0, [0, 1, 2, 3, 4, 5]), (1, [6]), (2, [7]), (3, [8]), (4, [9]), (last, [len(want) - 1])):
         assert float(np.abs(got32[key] - ref[rows]).max()) <= 2e-4 * spread, key
+
+
+def test_decoding_40_requests_together_gives_what_each_gives_alone(folder):
+    """At these sizes a batch of 40 decoding requests takes the kernels for 33 to 64 rows and another
+    split of the context than a request alone; the logits of a request must not depend on it beyond
+    the rounding of bfloat16 (the sums of the weight-streaming kernels are the same bit for bit, the
+    attention merges its splits in another order)."""
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    rng = random.Random(2)
+    R = 40
+    prompts = [[rng.randrange(SHAPE["vocab_size"]) for _ in range((5 if i % 2 else 500) + i)] for i in range(R)]    # short and long contexts
+    nexts = [[rng.randrange(SHAPE["vocab_size"]) for _ in range(2)] for _ in range(R)]
+    rep = TraceReplayer(folder, "bfloat16", max_tokens=R * 576, max_live=R)
+
+    def prefill(i):
+        return rep.run_step({"step": 0, "entries": [{"id": str(i), "tokens": prompts[i], "want": [len(prompts[i]) - 1]}], "end": []})
+
+    # alone: prompt, then two single tokens
+    alone = []
+    for i in range(R):
+        rows = [prefill(i)[0]]
+        for t in nexts[i]:
+            rows.append(rep.run_step({"step": 1, "entries": [{"id": str(i), "tokens": [t], "want": [0]}], "end": []})[0])
+        rep.run_step({"step": 2, "entries": [], "end": [str(i)]})
+        alone.append(rows)
+    # together: the prompts one after the other (as above), then all 40 decode in one step, twice
+    for i in range(R):
+        got = prefill(i)[0]
+        assert np.array_equal(got, alone[i][0]), i          # the same kernels on the same inputs
+    for k in range(2):
+        got = rep.run_step({"step": 3 + k, "entries": [{"id": str(i), "tokens": [nexts[i][k]], "want": [0]} for i in range(R)],
+                            "end": []})
+        ref = np.stack([alone[i][1 + k] for i in range(R)])
+        spread = float(ref.std())
+        rms = float(np.sqrt(((got - ref) ** 2).mean())) / spread
+        same = int((got.argmax(1) == ref.argmax(1)).sum())
+        print(f"[large] 40 together, decode step {k}: rms difference {rms:.2e} of the spread, argmax equal in {same}/{R} rows")
+        assert rms < 5e-3 and same >= R - 2, (k, rms, same)
+    del rep
+    torch.cuda.empty_cache()
