@@ -56,6 +56,8 @@ class LLMEngine:
                                    args.max_seq_len)
         self.sampler = Sampler(self.model.device, args.max_num_seqs)
         self.eos_token_id = self.model.spec.eos_token_id
+        if self.eos_token_id is None and tokenizer is not None:     # the reference's source for it, pico_vllm/engine.py:48
+            self.eos_token_id = getattr(tokenizer, "eos_token_id", None)
         self.tokenizer = tokenizer
         self._next_id = 0
         self.requests: Dict[int, Request] = {}

@@ -1,11 +1,13 @@
 """Generation through the entry point against the plain implementation: the workloads of the two
 tiny configurations, greedy and with temperature, chunked prompts mixed with decoding, HIP graph
 replay of decode steps, and what happens when pages run out."""
+import os
+
 import pytest
 import torch
 
 import plain_qwen2 as P
-from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
+from tiny_configs import CONFIGS, PAGE_SIZE, TINY_A, model_dir
 
 pytestmark = pytest.mark.gpu
 
@@ -208,3 +210,38 @@ def test_command_line_on_random_weights_of_a_named_size(capsys):
     lines = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")]
     assert len(lines) == 2 and all("(length)" in l and len(l.split(")")[1].split()) == 6 for l in lines)
 
+
+
+def test_command_line_with_a_text_prompt_and_a_tokenizer_in_the_model_folder(capsys, tmp_path):
+    """--prompt TEXT goes through the tokenizer files of the model folder, as the reference's entry script
+    does (pico_vllm/run_single.py:15,31); the answer is the decoded prompt + generated tokens
+    (pico_vllm/engine.py:385); the end-of-sequence token comes from the tokenizer when config.json names none
+    (engine.py:48)."""
+    import json
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import WhitespaceSplit
+    from pico_vllm_amd import run
+    from pico_vllm_amd.weights.random_init import write_random_model
+    folder = str(tmp_path / "model")
+    config = {k: v for k, v in TINY_A.items() if k not in ("model_type", "eos_token_id")}
+    write_random_model(folder, config, 0)
+    tok = Tokenizer(WordLevel({f"w{i}": i for i in range(config["vocab_size"])}, unk_token="w0"))
+    tok.pre_tokenizer = WhitespaceSplit()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    common = ["--model", folder, "--max-new-tokens", "8", "--dtype", "float32", "--num-gpu-blocks", "16", "--max-seq-len", "64"]
+    with open(os.path.join(folder, "tokenizer_config.json"), "w") as f:
+        json.dump({"tokenizer_class": "PreTrainedTokenizerFast"}, f)
+    assert run.main(common + ["--prompt-ids", "5,17,3"]) == 0
+    ids = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")][0].split(")")[1].split()
+    assert len(ids) == 8
+    assert run.main(common + ["--prompt", "w5 w17 w3"]) == 0
+    text = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")][0].split(")", 1)[1].strip()
+    assert text == " ".join(["w5", "w17", "w3"] + [f"w{i}" for i in ids])
+    # the tokenizer names the third generated token as the end of a sequence: generation stops there and keeps it
+    with open(os.path.join(folder, "tokenizer_config.json"), "w") as f:
+        json.dump({"tokenizer_class": "PreTrainedTokenizerFast", "eos_token": f"w{ids[2]}"}, f)
+    assert run.main(common + ["--prompt", "w5 w17 w3"]) == 0
+    line = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")][0]
+    first = ids.index(ids[2])
+    assert "(eos)" in line and line.split(")", 1)[1].split() == ["w5", "w17", "w3"] + [f"w{i}" for i in ids[:first + 1]]
