@@ -146,3 +146,71 @@ extern "C" int pico_sample(const float* logits, int ld, int R, int V, const floa
   PICO_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Greedy rows only: the argmax in two launches.  One workgroup per row reads the row no faster than
+// one compute unit takes data in (19 us for 151,936 logits); ARGMAX_CHUNKS workgroups per row find the
+// first maximum of a chunk each, a second launch picks among them (the lowest index on a tie, as above).
+// ---------------------------------------------------------------------------
+#define ARGMAX_CHUNKS 32
+
+__device__ __forceinline__ void keep_first_max(float& mx, int& mi, float ov, int oi) {
+  if (ov > mx || (ov == mx && oi < mi)) { mx = ov; mi = oi; }
+}
+
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits, int ld, int V,
+                                                          float* __restrict__ part_val, int* __restrict__ part_idx) {
+  __shared__ float vals[4];
+  __shared__ int idxs[4];
+  const int row = blockIdx.x, c = blockIdx.y, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * ld;
+  const int len = (V + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+  const int begin = min(V, c * len), end = min(V, begin + len);
+  float mx = -INFINITY;
+  int mi = 0x7fffffff;
+  // four loads in flight per thread; indices rise within a thread, so ">" keeps the first maximum
+  for (int i0 = begin + tid; i0 < end; i0 += 4 * 256) {
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int i = i0 + j * 256;
+      v[j] = i < end ? x[i] : -INFINITY;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (v[j] > mx) { mx = v[j]; mi = i0 + j * 256; }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) keep_first_max(mx, mi, __shfl_xor(mx, off, 64), __shfl_xor(mi, off, 64));
+  if ((tid & 63) == 0) { vals[tid >> 6] = mx; idxs[tid >> 6] = mi; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 4; w++) keep_first_max(mx, mi, vals[w], idxs[w]);
+    part_val[row * ARGMAX_CHUNKS + c] = mx;
+    part_idx[row * ARGMAX_CHUNKS + c] = mi;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx,
+                                                          int* __restrict__ out) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  float mx = lane < ARGMAX_CHUNKS ? part_val[row * ARGMAX_CHUNKS + lane] : -INFINITY;
+  int mi = lane < ARGMAX_CHUNKS ? part_idx[row * ARGMAX_CHUNKS + lane] : 0x7fffffff;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) keep_first_max(mx, mi, __shfl_xor(mx, off, 64), __shfl_xor(mi, off, 64));
+  if (lane == 0) out[row] = mi;
+}
+
+// part_val, part_idx: workspace of R * pico_argmax_chunks() entries each
+extern "C" int pico_argmax_chunks() { return ARGMAX_CHUNKS; }
+
+extern "C" int pico_argmax(const float* logits, int ld, int R, int V, float* part_val, int* part_idx, int* out,
+                           hipStream_t stream) {
+  PICO_REQUIRE(R >= 0 && V > 0 && ld >= V, "pico_argmax: bad sizes R=%d V=%d ld=%d", R, V, ld);
+  PICO_REQUIRE(R <= 65535, "pico_argmax: too many rows");
+  if (R == 0) return 0;
+  argmax_part_kernel<<<dim3(R, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, ld, V, part_val, part_idx);
+  argmax_final_kernel<<<R, 64, 0, stream>>>(part_val, part_idx, out);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

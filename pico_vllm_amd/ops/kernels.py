@@ -381,3 +381,28 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     _check(lib, lib.pico_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature),
                                 _ptr(top_p), _ptr(u), _ptr(out), _stream()))
     return out
+
+
+def argmax_workspace(rows: int, device) -> tuple:
+    """What ``argmax`` needs beside its output: the maxima of the chunks of every row and where they are."""
+    n = rows * int(library.core().pico_argmax_chunks())
+    return torch.empty(n, dtype=torch.float32, device=device), torch.empty(n, dtype=torch.int32, device=device)
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, work: tuple) -> torch.Tensor:
+    """The index of the first maximum of every row of float32 logits (what ``sample`` gives for
+    temperature 0), several workgroups a row."""
+    _gpu(logits, out, *work)
+    R, V = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("argmax: logits must be float32 with unit stride along the vocabulary")
+    if out.dtype != torch.int32 or out.numel() < R or not out.is_contiguous():
+        raise KernelError("argmax: out must be contiguous int32 with one entry per row")
+    lib = library.core()
+    need = R * int(lib.pico_argmax_chunks())
+    val, idx = work
+    if val.dtype != torch.float32 or idx.dtype != torch.int32 or val.numel() < need or idx.numel() < need \
+            or not val.is_contiguous() or not idx.is_contiguous():
+        raise KernelError("argmax: the workspace must come from argmax_workspace for at least as many rows")
+    _check(lib, lib.pico_argmax(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(val), _ptr(idx), _ptr(out), _stream()))
+    return out

@@ -41,8 +41,8 @@ class Sampler:
         self._host = [torch.zeros(3, max_rows, dtype=torch.float32, pin_memory=torch.cuda.is_available()) for _ in range(2)]
         self._dev = torch.zeros(3, max_rows, dtype=torch.float32, device=device)
         self._out = torch.zeros(max_rows, dtype=torch.int32, device=device)
+        self._argmax_work = kernels.argmax_workspace(max_rows, device) if torch.cuda.is_available() else None
         self._host_np = [h.numpy() for h in self._host]
-        self._zeroed = True
         self._landing = [torch.zeros(max_rows, dtype=torch.int32, pin_memory=torch.cuda.is_available()) for _ in range(2)]
         self._landed = [torch.cuda.Event() if torch.cuda.is_available() else None for _ in range(2)]
         self._turn = 0
@@ -77,18 +77,15 @@ class Sampler:
         if R == 0:
             return (0, 0)
         if not any(temperatures):
-            # all rows greedy: temperatures of zero are already on the device, nothing to upload
-            if not self._zeroed:
-                self._dev.zero_()
-                self._zeroed = True
+            # all rows greedy: nothing to upload, and the argmax alone spreads a row over several workgroups
+            kernels.argmax(logits, self._out, self._argmax_work)
         else:
             h = self._host_np[self._turn]
             h[0, :R] = temperatures
             h[1, :R] = top_ps
             h[2, :R] = [uniform(s, i) if t > 0 else 0.0 for s, i, t in zip(seeds, indices, temperatures)]
             self._dev.copy_(self._host[self._turn], non_blocking=True)
-            self._zeroed = False
-        kernels.sample(logits, self._dev[0], self._dev[1], self._dev[2], self._out)
+            kernels.sample(logits, self._dev[0], self._dev[1], self._dev[2], self._out)
         turn = self._turn
         self._turn ^= 1
         self._landing[turn][:R].copy_(self._out[:R], non_blocking=True)

@@ -234,6 +234,27 @@ def test_sampling_greedy_and_ties(K):
     assert out.tolist() == want and want[1] == 7 and want[2] == 999
 
 
+@pytest.mark.parametrize("R,V", [(1, 17), (5, 1000), (8, 151936), (64, 4099)])
+def test_argmax_in_two_launches_is_the_greedy_sample(K, R, V):
+    g = torch.Generator().manual_seed(V)
+    logits = torch.randn(R, V, generator=g)
+    logits[0, V // 3] = logits[0, V - 1] = 40.0                  # a tie across chunks: the lower index wins
+    if R > 1:
+        logits[1, V - 1] = 50.0                                  # the last element of the last chunk
+        logits[R - 1, 0] = 50.0
+    dev = logits.to(DEV)
+    out = torch.full((R,), -1, dtype=torch.int32, device=DEV)
+    K.argmax(dev, out, K.argmax_workspace(R, DEV))
+    z = torch.zeros(R, device=DEV)
+    assert out.tolist() == [P.sample_greedy(l) for l in logits] == K.sample(dev, z, z + 1, z).tolist()
+    assert out[0] == V // 3
+    wide = torch.randn(R, V + 5, generator=g).to(DEV)            # rows with a stride of their own
+    K.argmax(wide[:, :V], out, K.argmax_workspace(R + 3, DEV))
+    assert out.tolist() == wide[:, :V].argmax(1).tolist()
+    with pytest.raises(K.KernelError):
+        K.argmax(dev, out, K.argmax_workspace(max(R - 1, 0), DEV))
+
+
 @pytest.mark.parametrize("V", [301, 5000, 151936])
 def test_sampling_temperature_follows_the_inverse_cdf(K, V):
     g = torch.Generator().manual_seed(V)
