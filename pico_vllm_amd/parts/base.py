@@ -7,7 +7,7 @@ constants.  ``load`` receives the part's CPU tensors by name (relative to the
 part's prefix) and puts what it needs on the device; ``forward`` runs on the
 GPU.
 
-Interfaces (see also DESIGN.md):
+Interfaces:
   Norm.add_norm(resid, delta, rows=None) -> normed
   PositionEncoding.rotate_and_store(qkv, ctx, kv, block_table, nq, nkv, d)
   Mixer.cache_spec() -> CacheSpec;  Mixer.forward(x, ctx, cache) -> y

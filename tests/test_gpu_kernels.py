@@ -449,6 +449,26 @@ def test_fast_kernels_find_one_far_key_among_hundreds(K):
             close(out, want, torch.bfloat16, scale=100)
 
 
+@pytest.mark.parametrize("far", [2, 9000, 20470])
+def test_fast_attention_finds_a_far_key_among_twenty_thousand(K, far):
+    # 20,480 cached keys (1,280 pages) and one key that matters: every split of decode, and a portion of a
+    # prompt after that prefix, reach it through the block table
+    def boost(qs, ks, vs, far=far):
+        for q in qs:
+            ks[0][far] = q[-1, 0:1, :] * 3.0
+        vs[0][far] = 100.0
+    for nsplit in (1, 7, 32):
+        out, want = _fast_case([1], [20480], 4, 2, 64, 16, seed=far, boost=boost, decode=True, nsplit=nsplit)
+        assert float(want[-1, 0].mean()) > 50
+        close(out, want, torch.bfloat16, scale=100)
+    out, want = _fast_case([1], [20480], 4, 2, 64, 16, seed=far, boost=boost, as_step=True)
+    close(out, want, torch.bfloat16, scale=100)
+    for teams in (0, 1, 3):
+        out, want = _fast_case([70], [20411], 4, 2, 64, 16, seed=far, boost=boost, teams=teams)
+        assert float(want[-1, 0].mean()) > 50
+        close(out, want, torch.bfloat16, scale=100)
+
+
 def test_fast_kernels_refuse_what_they_cannot_do(K):
     from pico_vllm_amd.ops.attention_fast import choose, supported
     assert choose(4, 2, 24, 0) is None and choose(4, 2, 512, 0) is None and choose(4, 2, 64, 16) is None

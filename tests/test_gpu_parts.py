@@ -280,3 +280,133 @@ def test_a_toy_mixer_with_state_of_its_own_registers_builds_and_steps(dtype):
         for rid in toks:
             close(torch.cat(got[rid]), whole[rid], dtype, scale=float(whole[rid].std()) * 3)
         assert whole["a"].shape == (29, 100) and float(whole["a"].std()) > 0.01
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(dtype):
+    """Two more toy parts, defined and registered here: a feed-forward that sends every token to the
+    one of three small experts whose router logit is largest (router in float32), and a position
+    encoding that multiplies the entries of q and k by cosines of the position.  Layer 0 has the
+    routed feed-forward, layer 1 the framework's dense one; both use the framework's attention with the toy
+    encoding.  The engine's whole prompt equals a plain computation written out below, and portions
+    equal the whole."""
+    import tempfile
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.ops import kernels
+    from pico_vllm_amd.parts.base import FeedForward, PositionEncoding
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import LayerSpec, ModelSpec, ParamSpec, PartSpec, RunEntry
+    from pico_vllm_amd.weights.random_init import write_random_model
+
+    H, V, NQ, NKV, D, E, I = 40, 90, 3, 1, 16, 3, 24
+
+    def gate_of(positions, d, base):
+        return torch.cos(positions.float()[:, None] / (base ** (torch.arange(d, device=positions.device).float() / d)))
+
+    @register_part("position", "toy_cosine_gate")
+    class CosineGate(PositionEncoding):
+        def __init__(self, base, act_dtype=torch.bfloat16):
+            self.base = base
+
+        def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d):
+            T = qkv.shape[0]
+            qk = qkv[:, :(nq + nkv) * d].view(T, nq + nkv, d)
+            qk.copy_((qk.float() * gate_of(ctx.positions[:T], d, self.base)[:, None, :]).to(qkv.dtype))
+            kernels.rope_kv_store(qkv, None, ctx.slot_mapping[kv.group], kv.k, kv.v, nq, nkv, d, 0)
+
+    @register_part("feed_forward", "toy_top1_experts")
+    class Top1Experts(FeedForward):
+        def __init__(self, hidden_size, num_experts, expert_size, act_dtype=torch.bfloat16):
+            self.H, self.E, self.I = hidden_size, num_experts, expert_size
+
+        def param_specs(self):
+            out = [ParamSpec("router.weight", (self.E, self.H), std=1.0)]
+            for e in range(self.E):
+                out += [ParamSpec(f"experts.{e}.in.weight", (self.I, self.H), std=0.3),
+                        ParamSpec(f"experts.{e}.out.weight", (self.H, self.I), std=0.3)]
+            return out
+
+        def load(self, tensors, device, dtype):
+            self.router = tensors["router.weight"].to(device).float()
+            self.w_in = [tensors[f"experts.{e}.in.weight"].to(device) for e in range(self.E)]
+            self.w_out = [tensors[f"experts.{e}.out.weight"].to(device) for e in range(self.E)]
+
+        def forward(self, x, ctx):
+            choice = (x.float() @ self.router.T).argmax(-1)            # router logits in float32
+            out = torch.zeros_like(x)
+            for e in range(self.E):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    h = torch.relu(x[rows] @ self.w_in[e].T)
+                    out[rows] = h @ self.w_out[e].T
+            return out
+
+    def toy_spec(cfg):
+        norm = PartSpec("rms_norm", {"size": H, "eps": 1e-5})
+        attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": D, "qkv_bias": False,
+                                          "window": 0, "position": PartSpec("toy_cosine_gate", {"base": 50.0})})
+        ffs = [PartSpec("toy_top1_experts", {"hidden_size": H, "num_experts": E, "expert_size": I}),
+               PartSpec("swiglu_mlp", {"hidden_size": H, "intermediate_size": I})]
+        layers = [LayerSpec(f"toy.layers.{i}", "prenorm", {"norm1": ("ln1", norm), "mixer": ("attn", attn), "norm2": ("ln2", norm),
+                                                          "ff": ("ff", ffs[i])}) for i in range(2)]
+        return ModelSpec(H, V, "toy.embed.weight", layers, [RunEntry(0), RunEntry(1)], norm, "toy.norm", None)
+
+    register_architecture("ToyRoutedLM", lambda raw: raw, toy_spec)
+    cfg = {"architectures": ["ToyRoutedLM"]}
+    rnd = P._same if dtype == torch.float32 else P.to_bf16
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=4, std_overrides={"attn": 0.4, "embed": 0.5, "ff.gate": 0.3, "ff.up": 0.3, "ff.down": 0.3})
+        w = {k: v.float() for k, v in P.read_weights(d).items()}
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        r = ModelRunner(model, 8, 16, 3, 64, 64)
+        toks = torch.randint(0, V, (43,), generator=torch.Generator().manual_seed(1)).tolist()
+
+        # the plain computation, whole sequence, no cache
+        def plain(rnd):
+            pos = torch.arange(len(toks))
+            x = w["toy.embed.weight"][toks]
+            margins = []
+            for i in range(2):
+                p = f"toy.layers.{i}"
+                h = rnd(P.rms_norm(x, w[f"{p}.ln1.weight"], 1e-5))
+                W = torch.cat([w[f"{p}.attn.{n}_proj.weight"] for n in "qkv"], 0)
+                q, k, v = P.split_qkv(rnd(h @ W.T), NQ, NKV, D)
+                g = gate_of(pos, D, 50.0)[:, None, :]
+                o = rnd(P.causal_attention(rnd(q * g), rnd(k * g), v))
+                x = x + rnd(o.reshape(len(toks), NQ * D) @ w[f"{p}.attn.o_proj.weight"].T)
+                h = rnd(P.rms_norm(x, w[f"{p}.ln2.weight"], 1e-5))
+                if i == 0:
+                    logits = h @ w[f"{p}.ff.router.weight"].T
+                    top = logits.topk(2, -1).values
+                    margins.append(float((top[:, 0] - top[:, 1]).min()))
+                    f = torch.zeros_like(h)
+                    for t, e in enumerate(logits.argmax(-1).tolist()):
+                        f[t] = rnd(rnd(torch.relu(h[t] @ w[f"{p}.ff.experts.{e}.in.weight"].T)) @ w[f"{p}.ff.experts.{e}.out.weight"].T)
+                    assert len(set(logits.argmax(-1).tolist())) == E          # every expert has tokens
+                else:
+                    gu = torch.cat([w[f"{p}.ff.gate_proj.weight"], w[f"{p}.ff.up_proj.weight"]], 0)
+                    f = rnd(rnd(P.swiglu(rnd(h @ gu.T))) @ w[f"{p}.ff.down_proj.weight"].T)
+                x = x + f
+            return rnd(P.rms_norm(x, w["toy.norm.weight"], 1e-5)) @ w["toy.embed.weight"].T, min(margins)
+
+        want, margin = plain(P._same)
+        assert margin > 0.05, "a token sits between two experts: take another seed"
+        r.manager.add_request("w")
+        assert r.manager.grow("w", len(toks))
+        whole_logits = r.step([SeqStep("w", toks, list(range(len(toks))))])
+        r.manager.free_request("w")
+        close_to_plain(whole_logits, want, plain(rnd)[0], dtype)
+        # in portions, a second request beside it
+        r.manager.add_request("a")
+        r.manager.add_request("b")
+        got, fed = [], 0
+        for n, nb in ((9, 2), (1, 1), (2, 5), (24, 1), (7, 1)):
+            assert r.manager.grow("a", fed + n) and r.manager.grow("b", r.manager.num_computed("b") + nb)
+            seqs = [SeqStep("b", toks[:nb], []), SeqStep("a", toks[fed:fed + n], list(range(n)))]
+            got.append(r.step(seqs))
+            r.advance(seqs)
+            fed += n
+        close(torch.cat(got), whole_logits, dtype, scale=float(whole_logits.std()) * 3)
