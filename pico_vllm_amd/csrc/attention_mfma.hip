@@ -1025,45 +1025,63 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 #endif
 
 // out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s; one workgroup per (sequence,
-// head).  Every wave weighs all splits (lane s holds split s) and sums a quarter of them for all
-// head dimensions, all loads issued together; wave 0 adds the four quarters.
+// head).  Every wave weighs all splits (lane s % 64 holds split s, up to four of them) and sums a
+// quarter of each 64 splits for all head dimensions, the loads of a quarter issued together; wave 0
+// adds the four quarters.
+constexpr int MERGE_MAX_SPLITS = 256;
 __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
                                                            bf16_t* __restrict__ out, int nq) {
   constexpr int DPL = (D + 63) / 64;                        // head dimensions per lane
+  constexpr int CH = MERGE_MAX_SPLITS / 64;
   __shared__ float quarter[3][DPL * 64];
   const int b = blockIdx.x, head = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float* p = part + ((size_t)b * nq + head) * nsplit * (D + 2);
-  const bool mine = lane < nsplit;                         // nsplit <= 64
-  const float m = mine ? p[lane * (D + 2) + D] : -INFINITY;
-  const float l = mine ? p[lane * (D + 2) + D + 1] : 0.f;
-  const float M = wave_max(m);
+  float m[CH], l[CH], wt[CH];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < CH; c++) {
+    const bool mine = 64 * c + lane < nsplit;
+    m[c] = mine ? p[(64 * c + lane) * (D + 2) + D] : -INFINITY;
+    l[c] = mine ? p[(64 * c + lane) * (D + 2) + D + 1] : 0.f;
+    mx = fmaxf(mx, m[c]);
+  }
+  const float M = wave_max(mx);
   bf16_t* o = out + ((size_t)b * nq + head) * D;
   if (M == -INFINITY) {   // an empty row (padding of a captured batch)
     if (wave == 0)
       for (int dim = lane; dim < D; dim += 64) o[dim] = 0;
     return;
   }
-  const float wt = mine ? __expf(m - M) : 0.f;
-  const float L = wave_sum(wt * l);
+  float lsum = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; c++) {
+    wt[c] = 64 * c + lane < nsplit ? __expf(m[c] - M) : 0.f;
+    lsum += wt[c] * l[c];
+  }
+  const float L = wave_sum(lsum);
   float acc[DPL];
 #pragma unroll
   for (int i = 0; i < DPL; i++) acc[i] = 0.f;
-  const int s0 = wave * 16;
-  float v[16][DPL];
 #pragma unroll
-  for (int j = 0; j < 16; j++) {
-    const int s = min(s0 + j, nsplit - 1);
+  for (int c = 0; c < CH; c++) {
+    if (64 * c >= nsplit) break;
+    const int s0 = 64 * c + wave * 16;
+    float v[16][DPL];
 #pragma unroll
-    for (int i = 0; i < DPL; i++) {
-      const int dim = lane + 64 * i;
-      v[j][i] = dim < D ? p[s * (D + 2) + dim] : 0.f;
+    for (int j = 0; j < 16; j++) {
+      const int s = min(s0 + j, nsplit - 1);
+#pragma unroll
+      for (int i = 0; i < DPL; i++) {
+        const int dim = lane + 64 * i;
+        v[j][i] = dim < D ? p[s * (D + 2) + dim] : 0.f;
+      }
     }
-  }
 #pragma unroll
-  for (int j = 0; j < 16; j++) {
-    const float ws = (s0 + j < nsplit) ? __shfl(wt, s0 + j, 64) : 0.f;
+    for (int j = 0; j < 16; j++) {
+      const float ws = (s0 + j < nsplit) ? __shfl(wt[c], wave * 16 + j, 64) : 0.f;
 #pragma unroll
-    for (int i = 0; i < DPL; i++) acc[i] += ws * v[j][i];
+      for (int i = 0; i < DPL; i++) acc[i] += ws * v[j][i];
+    }
   }
   if (wave > 0) {
 #pragma unroll
@@ -1144,7 +1162,7 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
                                 float scale, hipStream_t stream) {
   if (check_common("pico_attn_decode", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
   PICO_REQUIRE(nq / nkv <= 32, "pico_attn_decode: %d query heads per kv head are more than 32", nq / nkv);
-  PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= 64 && nkv <= 65535, "pico_attn_decode: bad sizes (1 to 64 splits)");
+  PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= MERGE_MAX_SPLITS && nkv <= 65535, "pico_attn_decode: bad sizes (1 to %d splits)", MERGE_MAX_SPLITS);
   PICO_REQUIRE(((uintptr_t)q % 16 == 0), "pico_attn_decode: misaligned queries");
   dim3 grid(num_seqs, nkv, nsplit);
   bool direct = false;

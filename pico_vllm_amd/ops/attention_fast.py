@@ -26,10 +26,13 @@ class FastAttention:
 
     def num_splits(self, num_seqs: int, max_context: int) -> int:
         """Enough workgroups to fill the chip (256 CUs, two workgroups each), no split shorter
-        than one 64-key tile, at most 64 splits (one lane of the merging wave each)."""
+        than one 64-key tile (or, beyond 64 splits, than two), at most 256 splits (what the merging kernel takes):
+        a single request with 32,768 tokens behind it is read by 512 workgroups, not by 128."""
         by_fill = max(1, 512 // max(1, num_seqs * self.nkv))
         by_len = max(1, -(-max_context // 64))
-        return max(1, min(by_fill, by_len, 64))
+        if by_len > 64:
+            by_len = max(64, -(-max_context // 128))
+        return max(1, min(by_fill, by_len, 256))
 
     def prefill_teams(self, new_lens, context_lens) -> int:
         """The shape of the prefill workgroups.  1 to 3: teams of four waves that share the key loop of a

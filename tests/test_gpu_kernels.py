@@ -429,7 +429,7 @@ def test_fast_prefill_with_a_cache_of_4_gib(K):
 
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(4, 1, 16, 16), (6, 3, 32, 8), (5, 5, 48, 16), (3, 1, 80, 32), (8, 2, 256, 64),
                                         (12, 2, 128, 16), (32, 1, 64, 16)])
-@pytest.mark.parametrize("nsplit", [1, 3, 8])
+@pytest.mark.parametrize("nsplit", [1, 3, 8, 65, 256])
 def test_fast_decode(K, nq, nkv, d, Pg, nsplit):
     out, want = _fast_case([1, 1, 1, 1, 1], [0, 70, 45, 129, 1000], nq, nkv, d, Pg, seed=4, decode=True, nsplit=nsplit)
     close(out, want, torch.bfloat16)
@@ -457,7 +457,7 @@ def test_fast_attention_finds_a_far_key_among_twenty_thousand(K, far):
         for q in qs:
             ks[0][far] = q[-1, 0:1, :] * 3.0
         vs[0][far] = 100.0
-    for nsplit in (1, 7, 32):
+    for nsplit in (1, 7, 32, 100, 256):
         out, want = _fast_case([1], [20480], 4, 2, 64, 16, seed=far, boost=boost, decode=True, nsplit=nsplit)
         assert float(want[-1, 0].mean()) > 50
         close(out, want, torch.bfloat16, scale=100)
