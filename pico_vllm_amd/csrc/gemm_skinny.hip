@@ -317,19 +317,20 @@ __device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile
   }
 }
 
-template <int MT, int EPI, bool TAIL, int NX>
+// FEW: the grid has at most one workgroup per compute unit; the whole LDS is that workgroup's, for more slices in flight
+template <int MT, int EPI, bool TAIL, int NX, bool FEW = false>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias, void* __restrict__ out,
                                                           int ldo, long long slab_stride, int M, int N, int K,
                                                           int k_per_wg, int rows) {
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, false>()];
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, FEW>()];
   const int wave = threadIdx.x >> 6;
   const int tile = blockIdx.x;
   const int m0 = blockIdx.z * 32 * MT;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, false>(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
-  constexpr int NWV = sk_waves<MT, NX, false>();
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, FEW>(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
+  constexpr int NWV = sk_waves<MT, NX, FEW>();
   for (int a = wave; a < 4; a += NWV) skinny_finish<MT, EPI>(red, tile, rows, a, m0, M, N, bias, out, ldo, slab_stride);
 }
 
@@ -540,21 +541,26 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
     PICO_LAUNCH_CHECK();
     return 0;
   }
-#define LAUNCH3(MT, EPI, TAIL, NX) \
-  gemm_skinny_kernel<MT, EPI, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, false>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
+  // 33 to 64 tokens and at most one workgroup per compute unit (the O and down projections): four waves and
+  // three slices each in flight instead of two and two (19.9 against 19.5 thousand tokens a second at batch
+  // 64); with fewer tokens the same made the step slower (707 against 721 tokens a second at batch 1)
+  const bool few = nx == 8 && (long long)grid.x * grid.y * grid.z <= SK_COMPUTE_UNITS;
+#define LAUNCH4(MT, EPI, TAIL, NX, FEW) \
+  gemm_skinny_kernel<MT, EPI, TAIL, NX, FEW><<<grid, 64 * sk_waves<MT, NX, FEW>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
 #define LAUNCH(EPI)                                               \
   do {                                                            \
-    if (nx == 1) LAUNCH3(1, EPI, false, 1);                       \
-    else if (nx == 2) LAUNCH3(1, EPI, false, 2);                  \
-    else if (nx == 4) LAUNCH3(1, EPI, false, 4);                  \
-    else if (nx == 8) LAUNCH3(2, EPI, false, 8);                  \
-    else if (mt == 1) LAUNCH3(1, EPI, true, 0);                   \
-    else LAUNCH3(2, EPI, true, 0);                                \
+    if (nx == 1) LAUNCH4(1, EPI, false, 1, false);                \
+    else if (nx == 2) LAUNCH4(1, EPI, false, 2, false);           \
+    else if (nx == 4) LAUNCH4(1, EPI, false, 4, false);           \
+    else if (nx == 8 && few) LAUNCH4(2, EPI, false, 8, true);     \
+    else if (nx == 8) LAUNCH4(2, EPI, false, 8, false);           \
+    else if (mt == 1) LAUNCH4(1, EPI, true, 0, false);            \
+    else LAUNCH4(2, EPI, true, 0, false);                         \
   } while (0)
   if (epilogue == EPI_BF16) LAUNCH(EPI_BF16);
   else if (epilogue == EPI_F32) LAUNCH(EPI_F32);
   else LAUNCH(EPI_SWIGLU);
-#undef LAUNCH3
+#undef LAUNCH4
 #undef LAUNCH
   PICO_LAUNCH_CHECK();
   return 0;
