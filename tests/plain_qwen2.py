@@ -27,6 +27,12 @@ from safetensors import safe_open
 # configuration and weights (read with the safetensors package, not with the
 # engine's own reader)
 # --------------------------------------------------------------------------
+def f32(x: torch.Tensor) -> torch.Tensor:
+    """At least float32: what is float64 stays so.  With float64 weights the whole computation runs in
+    float64, which tells the engine's rounding from this implementation's own."""
+    return x if x.dtype == torch.float64 else x.float()
+
+
 @dataclass
 class PlainConfig:
     vocab_size: int
@@ -75,18 +81,19 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """y = x * 1/sqrt(mean(x^2) + eps) * w   (RMSNorm.py:22-31; eager twin
     model.py:63-66).  eps sits inside the square root; the weight multiplies
     (it is not 1+w)."""
-    x = x.float()
+    x = f32(x)
     var = (x * x).sum(dim=-1, keepdim=True) / x.shape[-1]
-    return x * (1.0 / torch.sqrt(var + eps)) * weight.float()
+    return x * (1.0 / torch.sqrt(var + eps)) * f32(weight).to(x.dtype)
 
 
-def rope_tables(positions: torch.Tensor, head_dim: int, theta: float):
+def rope_tables(positions: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype = torch.float32):
     """cos/sin rows for the given absolute positions (model.py:80-90).
 
     f_j = 1 / theta^(2j/d), j < d/2; angle = p * f_j in float32; each table
-    row is the half-row repeated twice."""
+    row is the half-row repeated twice.  The angle is the float32 product by
+    definition; ``dtype`` is that of its cosine and sine."""
     freqs = 1.0 / (theta ** (torch.arange(0, head_dim, 2).float() / head_dim))
-    angles = torch.outer(positions.float(), freqs)
+    angles = torch.outer(positions.float(), freqs).to(dtype)
     cos = torch.cat([angles.cos(), angles.cos()], dim=-1)
     sin = torch.cat([angles.sin(), angles.sin()], dim=-1)
     return cos, sin
@@ -130,19 +137,19 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     if q_positions is None:
         q_positions = torch.arange(N - M, N)
     scale = 1.0 / math.sqrt(d)
-    out = torch.empty(M, nq, d, dtype=torch.float32)
+    out = torch.empty(M, nq, d, dtype=f32(q).dtype)
     k_pos = torch.arange(N)
     visible = k_pos[None, :] <= q_positions[:, None]
     if window > 0:
         visible &= k_pos[None, :] > (q_positions[:, None] - window)
     for h in range(nq):
         g = h // G
-        s = (q[:, h, :].float() @ k[:, g, :].float().T) * scale
+        s = (f32(q[:, h, :]) @ f32(k[:, g, :]).T) * scale
         s = s.masked_fill(~visible, float("-inf"))
         p = torch.softmax(s, dim=-1)
         if rnd_p is not None:
             p = rnd_p(p)
-        out[:, h, :] = p @ v[:, g, :].float()
+        out[:, h, :] = p @ f32(v[:, g, :])
     return out
 
 
@@ -150,7 +157,7 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """gate = first half, up = second half of the last dim (weights.py:58);
     out = gate * sigmoid(gate) * up  (kernels/swiglu.py:36-41, model.py:318)."""
     I = gate_up.shape[-1] // 2
-    gate, up = gate_up[..., :I].float(), gate_up[..., I:].float()
+    gate, up = f32(gate_up[..., :I]), f32(gate_up[..., I:])
     return gate * torch.sigmoid(gate) * up
 
 
@@ -176,7 +183,7 @@ def attention_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
                    w[f"{prefix}.self_attn.v_proj.bias"]], dim=0)
     qkv = rnd(h @ W.T + b)
     q, k, v = split_qkv(qkv, nq, nkv, d)
-    cos, sin = rope_tables(positions, d, cfg.rope_theta)
+    cos, sin = rope_tables(positions, d, cfg.rope_theta, qkv.dtype)
     q, k = rnd(apply_rope(q, cos, sin)), rnd(apply_rope(k, cos, sin))
     o = rnd(causal_attention(q, k, v, q_positions=positions - positions[0], rnd_p=None if rnd is _same else rnd))
     return rnd(o.reshape(h.shape[0], nq * d) @ w[f"{prefix}.self_attn.o_proj.weight"].T)
@@ -210,21 +217,22 @@ def forward(tokens: Sequence[int], w: Dict[str, torch.Tensor], cfg: PlainConfig,
     bfloat16 storage of activations moves the logits of this model, which is
     the yardstick for the bfloat16 engine's tolerance."""
     ids = torch.as_tensor(list(tokens), dtype=torch.long)
-    x = w["model.embed_tokens.weight"][ids].float()
+    x = f32(w["model.embed_tokens.weight"][ids])
     positions = torch.arange(first_position, first_position + len(ids))
     for i in range(cfg.num_hidden_layers):
         x = block(x, w, i, cfg, positions, rnd)
     x = rnd(rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps))
     out_w = w["model.embed_tokens.weight"] if cfg.tie_word_embeddings else w["lm_head.weight"]
-    return x @ out_w.float().T
+    return x @ f32(out_w).T
 
 
 class PlainModel:
     """A model folder read once; ``logits(tokens)`` runs the whole sequence."""
 
-    def __init__(self, model_dir: str):
+    def __init__(self, model_dir: str, dtype: torch.dtype = torch.float32):
+        """``dtype`` float64: the same weights (they are exact in float64) and every sum in float64."""
         self.cfg = read_config(model_dir)
-        self.w = read_weights(model_dir)
+        self.w = {k: v.to(dtype) for k, v in read_weights(model_dir).items()}
 
     def logits(self, tokens: Sequence[int], rnd=_same) -> torch.Tensor:
         with torch.no_grad():

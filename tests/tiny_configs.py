@@ -23,6 +23,35 @@ TINY_C = {   # head size 48 given explicitly (hidden != heads * head), 5 heads w
 PAGE_SIZE = {"A": 16, "B": 8, "C": 16}
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 
+
+def drawn(seed: int):
+    """A configuration drawn at random (the same for a seed on every machine): head sizes in steps of 16,
+    any number of heads and groups, a width, an intermediate size and a vocabulary that are no powers of
+    two, with or without a head size of its own, tied or not; and a page size."""
+    import random
+    rng = random.Random(1000 + seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 128])
+    nkv = rng.choice([1, 2, 3, 4])
+    nq = nkv * rng.choice([1, 2, 3, 5, 7])
+    while nq * d > 1024:
+        nq -= nkv
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu",
+           "num_attention_heads": nq, "num_key_value_heads": nkv,
+           "num_hidden_layers": rng.choice([1, 2, 3]), "vocab_size": rng.randrange(200, 700) | 1,
+           "intermediate_size": 8 * rng.randrange(9, 50), "rms_norm_eps": rng.choice([1e-6, 3e-6, 1e-5]),
+           "rope_theta": rng.choice([1e4, 5e4, 1e6]), "tie_word_embeddings": rng.random() < 0.5,
+           "max_position_embeddings": 2048}
+    if rng.random() < 0.5:
+        cfg["hidden_size"] = nq * d
+    else:
+        cfg["hidden_size"] = 8 * rng.randrange(9, 40)
+        cfg["head_dim"] = d
+    return cfg, rng.choice([8, 16, 32])
+
+
+for _seed in range(10):
+    CONFIGS[f"R{_seed}"], PAGE_SIZE[f"R{_seed}"] = drawn(_seed)
+
 _made = {}
 
 
