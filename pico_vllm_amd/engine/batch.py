@@ -7,7 +7,7 @@ reference builds five tensors per decode step from Python lists and refills a
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Hashable, List, Optional, Sequence
 
 import numpy as np

@@ -9,7 +9,7 @@ build the model, load weights, make the block manager and the engine, then
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple, Union
+from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 

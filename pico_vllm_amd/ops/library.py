@@ -18,7 +18,7 @@ import sys
 import tempfile
 import time
 from concurrent.futures import ThreadPoolExecutor
-from typing import Dict, Iterable, List, Optional, Sequence, Tuple
+from typing import Dict, Iterable, List, Sequence
 
 CSRC = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "csrc"))
 ARCH = "gfx950"

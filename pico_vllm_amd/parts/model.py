@@ -10,7 +10,7 @@ from ..ops import kernels
 from ..ops.linear import Linear
 from ..weights.loader import load_checkpoint
 from . import attention, block, mlp, norm, rotary  # noqa: F401  (register the parts)
-from .base import Block, Part, StepContext
+from .base import Block, StepContext
 from .registry import build_part, part_class
 from .spec import CacheSpec, ModelSpec, ParamSpec
 

@@ -12,7 +12,7 @@ import json
 import mmap
 import os
 import struct
-from typing import Dict, Iterable, Iterator, List, Tuple
+from typing import Dict, Iterable, List, Tuple
 
 import numpy as np
 import torch

@@ -1,7 +1,6 @@
 """Configuration, registry, safetensors reading and the loader's errors (no GPU)."""
 import json
 import os
-import struct
 
 import pytest
 import torch
@@ -15,7 +14,7 @@ from pico_vllm_amd.parts.spec import ParamSpec
 from pico_vllm_amd.weights.loader import WeightsError, load_checkpoint
 from pico_vllm_amd.weights.random_init import write_random_model
 from pico_vllm_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
-from tiny_configs import CONFIGS, TINY_A, TINY_B, TINY_C, model_dir
+from tiny_configs import CONFIGS, TINY_A, TINY_B, model_dir
 
 
 def test_config_reads_every_key_and_has_no_size_defaults():

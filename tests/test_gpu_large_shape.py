@@ -7,7 +7,6 @@ slow here, so the yardstick is the engine's own true 32-bit path, which the othe
 plain implementation; the bfloat16 engine must follow it within bfloat16 rounding, whole, in
 portions, and token by token.
 """
-import os
 import random
 import tempfile
 

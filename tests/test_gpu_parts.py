@@ -1,14 +1,13 @@
 """Each part alone against the plain function of the same part, a model whose run order names a
 layer twice, and a toy mixer with state of its own that the test registers without touching the
 framework."""
-import math
 
 import pytest
 import torch
 
 import plain_qwen2 as P
 from gpu_util import DEV, DTYPES, tol
-from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
+from tiny_configs import PAGE_SIZE, model_dir
 
 pytestmark = pytest.mark.gpu
 

@@ -1,12 +1,10 @@
 """Trace replay against the plain implementation: the same requests whole, with the last 32
 tokens one by one, in portions of changing size, and mixed with other requests in a pool so small
 that pages are used again; in 32-bit and in bfloat16."""
-import io
 import json
 import os
 import random
 import subprocess
-import sys
 import tempfile
 
 import numpy as np

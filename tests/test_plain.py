@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 import plain_qwen2 as P
-from tiny_configs import CONFIGS, model_dir
+from tiny_configs import model_dir
 
 torch.manual_seed(0)
 

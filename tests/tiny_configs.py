@@ -1,5 +1,4 @@
 """The small configurations the tests run: they differ in every size and option."""
-import os
 import tempfile
 
 TINY_A = {   # MQA, tied, head 16
