@@ -481,7 +481,10 @@ def test_fast_kernels_refuse_what_they_cannot_do(K):
                                    (32, 301, 256), (9, 1000, 8960),
                                    # more than 32 tokens and many tiles: two tiles a workgroup (an odd number of tiles,
                                    # an odd number of slices, a single slice)
-                                   (50, 10270, 192), (40, 10400, 64), (64, 10240, 320)])
+                                   (50, 10270, 192), (40, 10400, 64), (64, 10240, 320),
+                                   # more than 64 tokens of a small matrix: blocks of 64 tokens, the last one partial
+                                   # (with 1 to 32 and with more than 32 tokens)
+                                   (65, 301, 136), (100, 1536, 1536), (130, 2048, 1536), (256, 1000, 264), (200, 90, 8960)])
 def test_gemm_skinny_epilogues(K, M, N, K_):
     g = torch.Generator().manual_seed(M * N)
     a = torch.randn(M, K_, generator=g).bfloat16()
@@ -523,7 +526,10 @@ def test_gemm_skinny_epilogues(K, M, N, K_):
 @pytest.mark.parametrize("M,nq,nkv,d,H,Pg,bias", [(1, 12, 2, 128, 1536, 16, True), (8, 12, 2, 128, 1536, 16, True),
                                                   (64, 6, 3, 32, 192, 8, True), (37, 3, 1, 64, 136, 32, False),
                                                   (5, 2, 2, 96, 264, 16, True), (13, 4, 2, 64, 320, 16, True),
-                                                  (29, 2, 1, 128, 128, 8, False)])
+                                                  (29, 2, 1, 128, 128, 8, False),
+                                                  # several blocks of 64 tokens
+                                                  (70, 12, 2, 128, 1536, 16, True), (256, 6, 3, 32, 192, 8, True),
+                                                  (150, 3, 1, 64, 136, 32, False)])
 def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias):
     # projection + bias + rotate-half + store in one kernel against the plain steps one after the other
     theta = 1e6
@@ -566,4 +572,11 @@ def test_gemm_skinny_refuses_misaligned_operands(K):
     assert not K.skinny_ok(a, w)
     with pytest.raises(K.KernelError):
         K.gemm_skinny(a, w)
-    assert not K.skinny_ok(torch.randn(65, 64).bfloat16().to(DEV), torch.randn(64, 64).bfloat16().to(DEV))
+    # more than 64 rows: small matrices only, and never more than 256
+    small, large = torch.randn(64, 64).bfloat16().to(DEV), torch.zeros(4104, 1024, dtype=torch.bfloat16, device=DEV)
+    assert K.skinny_ok(torch.randn(65, 64).bfloat16().to(DEV), small)
+    assert K.skinny_ok(torch.randn(64, 1024).bfloat16().to(DEV), large)
+    assert not K.skinny_ok(torch.randn(65, 1024).bfloat16().to(DEV), large)
+    assert not K.skinny_ok(torch.randn(257, 64).bfloat16().to(DEV), small)
+    with pytest.raises(K.KernelError):
+        K.gemm_skinny(torch.randn(257, 64).bfloat16().to(DEV), small)
