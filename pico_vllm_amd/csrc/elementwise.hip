@@ -340,6 +340,83 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float2* __restrict_
   }
 }
 
+// The same for bfloat16 with 16-byte accesses (d and rot / 2 multiples of 8).  A unit of work is 8 consecutive
+// head dimensions of one token: a rotated pair of such runs of a q or k head, a run of k that is not rotated,
+// or a run of v; every thread takes one unit, so that all loads of the launch are on their way at once (a
+// thread that loops over units waits for each one's loads in turn, because its stores may alias the next loads).
+// Grid x: blocks of RS_TOK consecutive tokens, grid y: the units of such a block in workgroups of 256.  The
+// units of v are numbered with the token fastest, so that the eight 2-byte stores of neighbouring lanes, which
+// go to neighbouring slots of a page when the tokens follow one another in a sequence, fall into one 16-byte
+// piece of V^T instead of eight 32-byte sectors.
+constexpr int RS_TOK = 8;
+typedef uint32_t rs_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void rope_store_bf16x8_kernel(bf16_t* __restrict__ qkv, const float2* __restrict__ cos_sin,
+                                                                const int* __restrict__ slots, bf16_t* __restrict__ k_cache,
+                                                                bf16_t* __restrict__ v_cache, int T, int nq, int nkv, int d,
+                                                                int rot, int P, int num_pages) {
+  const int t0 = blockIdx.x * RS_TOK;
+  const int half = rot >> 1, hc = half >> 3;                 // 8-wide runs in half the rotated part
+  const int row_len = (nq + 2 * nkv) * d;
+  const int u_rot = (nq + nkv) * hc, u_copy = nkv * ((d - rot) >> 3), u_v = nkv * (d >> 3);
+  const int u_qk = RS_TOK * (u_rot + u_copy);
+  int u = blockIdx.y * blockDim.x + threadIdx.x;
+  if (u < u_qk) {                                            // rotated pairs and the rest of k: token-major
+    const int i = u / (u_rot + u_copy), w = u - i * (u_rot + u_copy);
+    const int t = t0 + i;
+    if (t >= T) return;
+    bf16_t* row = qkv + (size_t)t * row_len;
+    const int slot = slots[t];
+    const int page = slot / P, off = slot % P;
+    const bool store = slot >= 0 && page < num_pages;         // not a padding row; the host has checked the rest
+    if (w < u_rot) {
+      const int head = w / hc, j = (w - head * hc) << 3;
+      const bf16_t* x = row + (size_t)head * d;
+      bf16_t* o;
+      if (head < nq) {
+        o = row + (size_t)head * d;
+      } else {
+        if (!store) return;
+        o = k_cache + (((size_t)page * nkv + (head - nq)) * P + off) * d;
+      }
+      const rs_u32x4 lo = *reinterpret_cast<const rs_u32x4*>(x + j), hi = *reinterpret_cast<const rs_u32x4*>(x + j + half);
+      const float4* cs = reinterpret_cast<const float4*>(cos_sin + (size_t)t * half + j);   // (cos, sin) of two dimensions each
+      rs_u32x4 olo, ohi;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float4 c2 = cs[e];
+        const float a0 = __uint_as_float(lo[e] << 16), a1 = __uint_as_float(lo[e] & 0xffff0000u);
+        const float b0 = __uint_as_float(hi[e] << 16), b1 = __uint_as_float(hi[e] & 0xffff0000u);
+        olo[e] = pack2_bf16(a0 * c2.x - b0 * c2.y, a1 * c2.z - b1 * c2.w);
+        ohi[e] = pack2_bf16(b0 * c2.x + a0 * c2.y, b1 * c2.z + a1 * c2.w);
+      }
+      *reinterpret_cast<rs_u32x4*>(o + j) = olo;
+      *reinterpret_cast<rs_u32x4*>(o + j + half) = ohi;
+    } else if (store) {
+      const int w2 = w - u_rot, per = (d - rot) >> 3;
+      const int g = w2 / per, j = rot + ((w2 - g * per) << 3);
+      *reinterpret_cast<rs_u32x4*>(k_cache + (((size_t)page * nkv + g) * P + off) * d + j) =
+          *reinterpret_cast<const rs_u32x4*>(row + (size_t)(nq + g) * d + j);
+    }
+    return;
+  }
+  u -= u_qk;                                                 // v: token fastest
+  if (u >= RS_TOK * u_v) return;
+  const int i = u % RS_TOK, w = u / RS_TOK;
+  const int t = t0 + i;
+  if (t >= T) return;
+  const int slot = slots[t];
+  const int page = slot / P, off = slot % P;
+  if (slot < 0 || page >= num_pages) return;
+  const int g = w / (d >> 3), j = (w - g * (d >> 3)) << 3;
+  const rs_u32x4 v = *reinterpret_cast<const rs_u32x4*>(qkv + (size_t)t * row_len + (size_t)(nq + nkv + g) * d + j);
+  bf16_t* o = v_cache + (((size_t)page * nkv + g) * d + j) * P + off;
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    o[(size_t)(2 * e) * P] = (bf16_t)(v[e] & 0xffffu);
+    o[(size_t)(2 * e + 1) * P] = (bf16_t)(v[e] >> 16);
+  }
+}
+
 extern "C" int pico_rope_kv_store(void* qkv, int dtype, const float* cos_sin, const int* slots,
                                   void* k_cache, void* v_cache, int T, int nq, int nkv, int d,
                                   int rot, int P, int num_pages, hipStream_t stream) {
@@ -352,6 +429,11 @@ extern "C" int pico_rope_kv_store(void* qkv, int dtype, const float* cos_sin, co
   if (dtype == PICO_DTYPE_F32)
     rope_store_kernel<float><<<grid, threads, 0, stream>>>((float*)qkv, (const float2*)cos_sin, slots, (float*)k_cache,
                                                       (float*)v_cache, nq, nkv, d, rot, P, num_pages);
+  else if (dtype == PICO_DTYPE_BF16 && T >= RS_TOK && d % 8 == 0 && rot % 16 == 0 && (uintptr_t)qkv % 16 == 0 &&
+           (uintptr_t)k_cache % 16 == 0 && (rot == 0 || (uintptr_t)cos_sin % 16 == 0))
+    rope_store_bf16x8_kernel<<<dim3((T + RS_TOK - 1) / RS_TOK, (RS_TOK * ((nq + nkv) * (rot / 16) + nkv * ((d - rot) / 8) + nkv * (d / 8)) + 255) / 256),
+                               256, 0, stream>>>(
+        (bf16_t*)qkv, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, T, nq, nkv, d, rot, P, num_pages);
   else if (dtype == PICO_DTYPE_BF16)
     rope_store_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)qkv, (const float2*)cos_sin, slots, (bf16_t*)k_cache,
                                                        (bf16_t*)v_cache, nq, nkv, d, rot, P, num_pages);

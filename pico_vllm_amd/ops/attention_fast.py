@@ -114,13 +114,18 @@ class FastAttention:
         if ctx.all_decode and grouped:
             return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, B, scale,
                                self.num_splits(B, ctx.max_context))
-        teams, lead = 0, 0
-        if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
-            cu = ctx.host["cu_seqlens"]
-            lens = cu[1:B + 1] - cu[:B]
-            while lead < B and lens[lead] == 1:
-                lead += 1
-            teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
+        # what the host decides from the shape of the batch is the same for every layer of the step
+        plan = ("fast_attention", self.nq, self.nkv, self.d)
+        if plan not in ctx.shared:
+            teams, lead = 0, 0
+            if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
+                cu = ctx.host["cu_seqlens"]
+                lens = cu[1:B + 1] - cu[:B]
+                while lead < B and lens[lead] == 1:
+                    lead += 1
+                teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
+            ctx.shared[plan] = (teams, lead)
+        teams, lead = ctx.shared[plan]
         if lead == 0 or not grouped:
             return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, scale, teams=teams)
         # A mixed step: the scheduler puts the decoding requests first.  Their tokens (one row each, rows
