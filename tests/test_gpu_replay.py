@@ -249,7 +249,7 @@ def test_mixed_with_pages_used_again(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", [f"R{i}" for i in range(10)])
+@pytest.mark.parametrize("name", [f"R{i}" for i in range(10)] + ["D"])
 def test_configurations_drawn_at_random_whole_and_mixed(name, dtype):
     # sizes nobody picked by hand: whole requests, and the same requests mixed in a small pool
     reqs = make_requests(name, [40, 77, 33, 60], seed=7)

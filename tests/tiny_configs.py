@@ -19,8 +19,14 @@ TINY_C = {   # head size 48 given explicitly (hidden != heads * head), 5 heads w
     "num_key_value_heads": 5, "head_dim": 48, "intermediate_size": 200, "rms_norm_eps": 1e-6,
     "rope_theta": 50000.0, "tie_word_embeddings": True, "max_position_embeddings": 1024, "hidden_act": "silu",
 }
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+TINY_D = {   # sizes that no vector access divides: a width of 100, an odd intermediate size and vocabulary
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 257, "hidden_size": 100, "num_hidden_layers": 2, "num_attention_heads": 4,
+    "num_key_value_heads": 2, "head_dim": 16, "intermediate_size": 123, "rms_norm_eps": 1e-6,
+    "rope_theta": 10000.0, "tie_word_embeddings": False, "max_position_embeddings": 1024, "hidden_act": "silu",
+}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def drawn(seed: int):
