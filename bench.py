@@ -32,8 +32,8 @@ MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 from pico_vllm_amd.config.presets import preset   # noqa: E402  (needs ROOT on the path)
 
-CONFIG_1P5B = preset("1.5b")       # BASELINE.json configs[2]: Qwen2.5-1.5B
-CONFIG_7B = preset("7b")           # BASELINE.json configs[3]: Qwen2.5-7B (measured with fewer layers when asked: --layers)
+CONFIG_1P5B = preset("1.5b")       # the default run: the Qwen2.5-1.5B shape
+CONFIG_7B = preset("7b")           # the Qwen2.5-7B shape (measured with fewer layers when asked: --layers)
 SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", CONFIG_1P5B), "7b": ("Qwen2.5-7B shape", CONFIG_7B),
           "32b": ("Qwen2.5-32B shape", preset("32b"))}
 CONFIG = CONFIG_1P5B         # the shape being measured (set in main)
@@ -131,7 +131,7 @@ def prefill_point(model_dir, model, dtype, reps=3):
 
 
 def serve_point(model_dir, dtype, requests, max_new):
-    """BASELINE.json's mixed workload: `requests` requests with prompt lengths uniform in 128..4096 (seeded) and
+    """The mixed workload: `requests` requests with prompt lengths uniform in 128..4096 (seeded) and
     `max_new` new tokens each, all submitted at once; the scheduler admits, cuts prompts into portions of at most
     2,048 tokens beside the decoding requests, decodes, finishes and frees."""
     import torch
