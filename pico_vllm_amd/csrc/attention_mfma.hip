@@ -849,9 +849,12 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(c
 // blocks of 32 keys: two 16-key tiles of S^T = K Q^T (the 16 columns are the query heads of the
 // group), then O^T += V^T P^T with the 32 keys as the contraction; as in the other kernels the
 // contraction order is the order in which the registers hold the keys, so P never moves.
-// Operands come straight from the pages: lane (key, kq) reads the 64 contiguous bytes
-// K[key][32 kq ..] (the contraction over the head dimension runs in that permuted order for K
-// and Q alike), and lane (dim, kq) reads the 8 bytes V^T[dim][4 kq .. 4 kq + 3] of each tile.
+// Operands come straight from the pages, in the order of memory: in step st the four lanes (a, 0..3) of
+// row a read the 64 contiguous bytes K[key of row a][32 st ..] (a load instruction touches 16 cache
+// lines; with a lane reading its own 64 bytes it touched 32), and lane (dim, kq) reads the 16 bytes
+// V^T[dim][8 kq .. 8 kq + 7] of the block.  Which key is row a of tile t is free; it is key
+// 8 (a / 4) + 4 t + a % 4 of the block, so that the registers of lane quarter kq hold the scores of the
+// eight consecutive keys 8 kq + 0..7, which is the contraction order of the V^T operand.
 // The loads of a wave's next block are issued while the current block is computed.
 #if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -879,11 +882,11 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 
   bf16x8 qf[KS16];
   {
-    const bf16_t* qrow = q + (size_t)b * q_stride + (size_t)head * D + (D / 4) * kq;
+    const bf16_t* qrow = q + (size_t)b * q_stride + (size_t)head * D + 8 * kq;
 #pragma unroll
     for (int st = 0; st < KS16; st++) {
       uint4 v = make_uint4(0, 0, 0, 0);
-      if (col_ok) v = *reinterpret_cast<const uint4*>(qrow + 8 * st);
+      if (col_ok) v = *reinterpret_cast<const uint4*>(qrow + 32 * st);
       qf[st] = __builtin_bit_cast(bf16x8, v);
     }
   }
@@ -896,29 +899,28 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
   const int pshift = 31 - __clz(P);                             // page sizes are powers of two
   if (first < k_end) {
     const int last = first + (k_end - 1 - first) / 128 * 128;   // this wave's last block
-    const int last_key = k_end - 1, last_group = last_key / 4 * 4;
+    const int last_key = k_end - 1, last_group = last_key / 8 * 8;
+    const int row_key = 8 * (col >> 2) + (col & 3);             // key of this lane's row in tile 0; tile 1: 4 more
     uint4 kr[2][KS16];
-    uint2 vr[DT16][2];
-    // positions beyond the split are clamped to its last key (group): the pages exist, the scores are masked
+    uint4 vr[DT16];
+    // positions beyond the split are clamped to its last key (group of 8, which lies in one page as pages hold
+    // at least 8 keys): the pages exist, the scores are masked
     auto load_k = [&](int key0) {
 #pragma unroll
       for (int t = 0; t < 2; t++) {
-        const int pos = min(key0 + 16 * t + col, last_key);
+        const int pos = min(key0 + row_key + 4 * t, last_key);
         const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
-        const bf16_t* kp = k_cache + ((((size_t)page * nkv + g) << pshift) + (pos & (P - 1))) * D + (D / 4) * kq;
+        const bf16_t* kp = k_cache + ((((size_t)page * nkv + g) << pshift) + (pos & (P - 1))) * D + 8 * kq;
 #pragma unroll
-        for (int st = 0; st < KS16; st++) kr[t][st] = *reinterpret_cast<const uint4*>(kp + 8 * st);
+        for (int st = 0; st < KS16; st++) kr[t][st] = *reinterpret_cast<const uint4*>(kp + 32 * st);
       }
     };
     auto load_v = [&](int key0) {
+      const int pos = min(key0 + 8 * kq, last_group);
+      const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
+      const bf16_t* vp = v_cache + ((((size_t)page * nkv + g) * D + col) << pshift) + (pos & (P - 1));
 #pragma unroll
-      for (int t = 0; t < 2; t++) {
-        const int pos = min(key0 + 16 * t + 4 * kq, last_group);
-        const int page = min(max(bt[pos >> pshift], 0), num_pages - 1);
-        const bf16_t* vp = v_cache + ((((size_t)page * nkv + g) * D + col) << pshift) + (pos & (P - 1));
-#pragma unroll
-        for (int tt = 0; tt < DT16; tt++) vr[tt][t] = *reinterpret_cast<const uint2*>(vp + ((size_t)tt * 16 << pshift));
-      }
+      for (int tt = 0; tt < DT16; tt++) vr[tt] = *reinterpret_cast<const uint4*>(vp + ((size_t)tt * 16 << pshift));
     };
     load_k(first);
     __builtin_amdgcn_sched_barrier(0);       // keys before values, as in the loop, so the waits there stay partial
@@ -941,7 +943,7 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 #pragma unroll
       for (int r = 0; r < 8; r++) {
         float v = (r < 4 ? s0[r & 3] : s1[r & 3]) * scale;
-        if (tail && key0 + 16 * (r >> 2) + 4 * kq + (r & 3) >= k_end) v = -INFINITY;
+        if (tail && key0 + 8 * kq + r >= k_end) v = -INFINITY;
         sv[r] = v;
         mx = fmaxf(mx, v);
       }
@@ -962,25 +964,22 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
       const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack2_bf16(sv[0], sv[1]), pack2_bf16(sv[2], sv[3]),
                                                                pack2_bf16(sv[4], sv[5]), pack2_bf16(sv[6], sv[7])));
       if (tail) {   // values of keys beyond the split hold whatever the page held before: make them zero
+        const int left = k_end - (key0 + 8 * kq);               // keys of this lane's eight that exist
+        uint32_t keep[4];
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-          const int pos = key0 + 16 * t + 4 * kq;
+        for (int w = 0; w < 4; w++) keep[w] = left >= 2 * w + 2 ? 0xffffffffu : left == 2 * w + 1 ? 0x0000ffffu : 0u;
 #pragma unroll
-          for (int tt = 0; tt < DT16; tt++) {
-            if (pos >= k_end) vr[tt][t] = make_uint2(0, 0);
-            else {
-              if (pos + 1 >= k_end) vr[tt][t].x &= 0x0000ffffu;
-              if (pos + 2 >= k_end) vr[tt][t].y = 0;
-              else if (pos + 3 >= k_end) vr[tt][t].y &= 0x0000ffffu;
-            }
-          }
+        for (int tt = 0; tt < DT16; tt++) {
+          vr[tt].x &= keep[0];
+          vr[tt].y &= keep[1];
+          vr[tt].z &= keep[2];
+          vr[tt].w &= keep[3];
         }
       }
 #pragma unroll
       for (int tt = 0; tt < DT16; tt++) {
         o[tt] *= alpha;
-        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vr[tt][0].x, vr[tt][0].y, vr[tt][1].x, vr[tt][1].y));
-        o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[tt], 0, 0, 0);
+        o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vr[tt]), pb, o[tt], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
       if (key0 >= last) break;
