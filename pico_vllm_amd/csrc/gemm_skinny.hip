@@ -50,6 +50,7 @@ struct TileRows {
 #define EPI_BF16 0     // out bf16 [M, N]
 #define EPI_F32 1      // out float32 [M, N] (slab `blockIdx.y` when the k range is split over the grid)
 #define EPI_SWIGLU 2   // W = [gate rows; up rows], out bf16 [M, N / 2]
+#define MAX_SK_SLABS 8 // partial sums that a norm in front of a projection adds up
 
 // The sums of one output tile when K is no multiple of 64 (any multiple of 8): operands go through
 // registers, lane (i, h) reads W[row i][k0 + 32 h ..] and the activations alike; k beyond the range
@@ -131,11 +132,21 @@ constexpr int sk_smem_bytes() {
 // holds the slices k_begin + 64 (v + 4 i) whatever the number of waves (a wave of a two-wave
 // workgroup keeps two sets of sums), so that a row's result does not depend on how many rows came
 // with it.
-template <int MT, int NX, int NWV, int DEPTH>
+//
+// XS: the activations, one row, do not travel with the slices.  The row lies in LDS already, bfloat16 [k_end] at xs
+// (the caller's `between`, which every wave runs after the first copies of W have been issued, puts it there;
+// its `before` runs ahead of those copies, for loads that should not queue behind them); a stage then holds
+// W only, and every column of the product is the row's.
+struct SkNothing {
+  __device__ __forceinline__ void operator()() const {}
+};
+template <int MT, int NX, int NWV, int DEPTH, bool XS = false, typename Before = SkNothing, typename Between = SkNothing>
 __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W,
                                                   int ldw, TileRows tr, int m0, int M, int k_begin,
-                                                  int k_end, char* smem) {
-  constexpr int STAGE = sk_stage_bytes<NX>(), LOADS = 4 + NX;
+                                                  int k_end, char* smem, const char* xs = nullptr,
+                                                  Before before = Before(), Between between = Between()) {
+  constexpr int STAGE = XS ? 4 * SK_GROUP : sk_stage_bytes<NX>(), LOADS = XS ? 4 : 4 + NX;
+  static_assert(!XS || (MT == 1 && NX == 1), "activations that stay in LDS: one row");
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int col = lane & 31, h = lane >> 5, rho = lane >> 3, pos = lane & 7;
   // sources of this lane's 16 bytes in each group, at k = 0
@@ -144,7 +155,7 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
   for (int g = 0; g < 4; g++) wsrc[g] = W + (size_t)tr.row(8 * g + rho) * ldw + 8 * (pos ^ rho);
   const bf16_t* xsrc[NX];
 #pragma unroll
-  for (int g = 0; g < NX; g++) xsrc[g] = X + (size_t)min(m0 + 8 * g + rho, M - 1) * ldx + 8 * (pos ^ rho);
+  for (int g = 0; g < NX; g++) xsrc[g] = XS ? nullptr : X + (size_t)min(m0 + 8 * g + rho, M - 1) * ldx + 8 * (pos ^ rho);
   // where lane (col, h) finds chunk 4 h + s of tile row (or token) col, relative to the slice
   int rd[4];
 #pragma unroll
@@ -162,38 +173,50 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
 
   constexpr int STRIDE = 64 * NWV;             // this wave's slices start at k_begin + 64 (wave + NWV i)
   const int first = k_begin + 64 * wave;
-  if (first < k_end) {
-    const int n_slices = (k_end - first + STRIDE - 1) / STRIDE;
-    const int rounds = (n_slices + DEPTH - 1) / DEPTH;
-    const int last = first + (n_slices - 1) * STRIDE;
-    auto issue = [&](int d, int slice) {       // beyond the wave's last slice the last one is copied again
-      const int k0 = min(first + STRIDE * slice, last);
-      char* dst = mine + d * NWV * STAGE;
+  const bool any = first < k_end;
+  const int n_slices = any ? (k_end - first + STRIDE - 1) / STRIDE : 0;
+  const int rounds = (n_slices + DEPTH - 1) / DEPTH;
+  const int last = first + (n_slices - 1) * STRIDE;
+  auto issue = [&](int d, int slice) {         // beyond the wave's last slice the last one is copied again
+    const int k0 = min(first + STRIDE * slice, last);
+    char* dst = mine + d * NWV * STAGE;
 #pragma unroll
-      for (int g = 0; g < 4; g++) __builtin_amdgcn_global_load_lds(GPTR(wsrc[g] + k0), LPTR(dst + g * SK_GROUP), 16, 0, 0);
+    for (int g = 0; g < 4; g++) __builtin_amdgcn_global_load_lds(GPTR(wsrc[g] + k0), LPTR(dst + g * SK_GROUP), 16, 0, 0);
+    if (!XS) {
 #pragma unroll
       for (int g = 0; g < NX; g++)
         __builtin_amdgcn_global_load_lds(GPTR(xsrc[g] + k0), LPTR(dst + (4 + g) * SK_GROUP), 16, 0, 0);
-    };
-    auto multiply = [&](int d) {
-      const char* src = mine + d * NWV * STAGE;
-      u32x4 a[4], b[MT][4];
+    }
+  };
+  auto multiply = [&](int d, int slice) {
+    const char* src = mine + d * NWV * STAGE;
+    u32x4 a[4], b[MT][4];
 #pragma unroll
-      for (int s = 0; s < 4; s++) {
-        a[s] = *reinterpret_cast<const u32x4*>(src + rd[s]);
+    for (int s = 0; s < 4; s++) {
+      a[s] = *reinterpret_cast<const u32x4*>(src + rd[s]);
+      if (XS) {   // the one row, for every column alike (only column 0 is stored)
+        b[0][s] = *reinterpret_cast<const u32x4*>(xs + 2 * (first + STRIDE * slice) + ((4 * h + s) << 4));
+      } else {
 #pragma unroll
         for (int t = 0; t < MT; t++) b[t][s] = *reinterpret_cast<const u32x4*>(src + (4 + 4 * t) * SK_GROUP + rd[s]);
       }
+    }
 #pragma unroll
-      for (int s = 0; s < 4; s++)
+    for (int s = 0; s < 4; s++)
 #pragma unroll
-        for (int t = 0; t < MT; t++)
-          acc[t][d % VW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[s]),
-                                                                   __builtin_bit_cast(bf16x8, b[t][s]), acc[t][d % VW], 0, 0, 0);
-    };
+      for (int t = 0; t < MT; t++)
+        acc[t][d % VW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[s]),
+                                                                 __builtin_bit_cast(bf16x8, b[t][s]), acc[t][d % VW], 0, 0, 0);
+  };
+  before();
+  __builtin_amdgcn_sched_barrier(0);
+  if (any) {
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) issue(d, d);
     __builtin_amdgcn_sched_barrier(0);
+  }
+  between();                                   // every wave, with its first copies on their way
+  if (any) {
     for (int r = 0; r + 1 < rounds; r++) {     // every slice of these rounds exists
 #pragma unroll
       for (int d = 0; d < DEPTH; d++) {
@@ -202,7 +225,7 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
         // these copies by itself.
         __builtin_amdgcn_s_waitcnt(sk_vmcnt((DEPTH - 1) * LOADS));
         __builtin_amdgcn_sched_barrier(0);
-        multiply(d);                            // its operand reads are complete when the products have issued
+        multiply(d, r * DEPTH + d);             // its operand reads are complete when the products have issued
         __builtin_amdgcn_sched_barrier(0);
         issue(d, (r + 1) * DEPTH + d);
         __builtin_amdgcn_sched_barrier(0);
@@ -213,7 +236,7 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
     const int left = n_slices - (rounds - 1) * DEPTH;            // 1..DEPTH slices in the last round
 #pragma unroll
     for (int d = 0; d < DEPTH; d++)
-      if (d < left) multiply(d);
+      if (d < left) multiply(d, (rounds - 1) * DEPTH + d);
   }
   __syncthreads();                             // every wave is done with its stages: the sums take their place
   float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
@@ -332,6 +355,102 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, FEW>(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
   constexpr int NWV = sk_waves<MT, NX, FEW>();
   for (int a = wave; a < 4; a += NWV) skinny_finish<MT, EPI>(red, tile, rows, a, m0, M, N, bias, out, ldo, slab_stride);
+}
+
+// ---- one token: the norm in front of the projection inside the projection's launch -------------------
+// A decode step of one request is a chain of launches of which each costs about 4.5 us before it has
+// streamed a byte, the add + norm kernels in front of the q/k/v and gate/up projections among them.  With
+// one row every workgroup of the projection can do that norm itself: it reads the row of the
+// residual stream, the partial sums that the projection before left (pico_vllm/RMSNorm.py:22-31 for the
+// norm, the sums in slab order as pico_add_rmsnorm forms them), reduces, and writes the normed row as
+// bfloat16 into LDS, where it stays for all slices; only W streams.  Workgroup 0 also writes the new residual stream, to another buffer than the one the other
+// workgroups still read.
+struct SkNormIn {
+  const float* resid;        // [M, K] float32, the residual stream before the sum
+  const float* delta;        // `slabs` partial sums [M, K] float32, slab s at delta + s * slab_stride; null: nothing to add
+  int slabs;
+  long long slab_stride;
+  const float* weight;       // [K] float32
+  float eps;
+  float* resid_out;          // [M, K] float32: resid + the slabs, written by workgroup 0
+};
+constexpr int SK_NORM_VPT = 2;                         // groups of four elements a thread: K <= 256 * 4 * 2
+constexpr int SK_NORM_MAX_K = 256 * 4 * SK_NORM_VPT;
+#ifndef SK_NORM_DEPTH
+#define SK_NORM_DEPTH 3                                // slices a wave keeps in flight in the projections of many tiles
+#endif
+
+// The one row: `load` requests the row, its partial sums and the norm's weight (before the first copies of W are
+// issued: vector memory returns in order, and behind those copies this small read from the caches would wait
+// for HBM); `finish` sums, norms and writes the row into xs as bfloat16 [K].
+// All 256 threads of the workgroup take part in both.
+struct SkNormRow {
+  float4 v[SK_NORM_VPT], g[SK_NORM_VPT], d[SK_NORM_VPT][MAX_SK_SLABS];
+
+  __device__ __forceinline__ void load(const SkNormIn& in, int K) {
+#pragma unroll
+    for (int j = 0; j < SK_NORM_VPT; j++) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+      v[j] = g[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int sl = 0; sl < MAX_SK_SLABS; sl++) d[j][sl] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < K) {
+        v[j] = *reinterpret_cast<const float4*>(in.resid + i);
+        g[j] = *reinterpret_cast<const float4*>(in.weight + i);
+#pragma unroll
+        for (int sl = 0; sl < MAX_SK_SLABS; sl++)
+          if (sl < in.slabs) d[j][sl] = *reinterpret_cast<const float4*>(in.delta + sl * in.slab_stride + i);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void finish(const SkNormIn& in, int K, char* xs, float* scratch, bool writer) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < SK_NORM_VPT; j++) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+#pragma unroll
+      for (int sl = 0; sl < MAX_SK_SLABS; sl++) { v[j].x += d[j][sl].x; v[j].y += d[j][sl].y; v[j].z += d[j][sl].z; v[j].w += d[j][sl].w; }
+      if (i < K) {
+        if (writer) *reinterpret_cast<float4*>(in.resid_out + i) = v[j];
+        ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+      }
+    }
+    ss = block_sum(ss, scratch);
+    const float r = 1.0f / sqrtf(ss / (float)K + in.eps);
+#pragma unroll
+    for (int j = 0; j < SK_NORM_VPT; j++) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+      if (i < K) {
+        *reinterpret_cast<uint2*>(xs + 2 * i) = make_uint2(pack2_bf16(v[j].x * r * g[j].x, v[j].y * r * g[j].y),
+                                                   pack2_bf16(v[j].z * r * g[j].z, v[j].w * r * g[j].w));
+      }
+    }
+    // workgroup 0 has stores on their way besides the copies: the counts that the stream waits with assume copies only
+    if (writer) __builtin_amdgcn_s_waitcnt(sk_vmcnt(0));
+    __syncthreads();
+  }
+};
+
+// stages of the stream (4 waves, W only), then the normed rows
+template <int DEPTH> constexpr int sk_xs_offset() { return DEPTH * 4 * 4 * SK_GROUP; }
+static int sk_xs_smem_bytes(int depth, int K) { return depth * 4 * 4 * SK_GROUP + 2 * K; }
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_skinny_norm_kernel(SkNormIn in, const bf16_t* __restrict__ W, int ldw,
+                                                               void* __restrict__ out, int ldo, int M, int N, int K,
+                                                               int rows) {
+  constexpr int DEPTH = SK_NORM_DEPTH;
+  extern __shared__ __attribute__((aligned(16))) char dsmem[];
+  __shared__ float scratch[16];
+  char* xs = dsmem + sk_xs_offset<DEPTH>();
+  const int wave = threadIdx.x >> 6, tile = blockIdx.x;
+  SkNormRow row;
+  skinny_stream_lds<1, 1, 4, DEPTH, true>(nullptr, 0, W, ldw, skinny_rows<EPI>(tile, rows, N), 0, M, 0, K, dsmem, xs,
+                                          [&]() { row.load(in, K); },
+                                          [&]() { row.finish(in, K, xs, scratch, blockIdx.x == 0); });
+  float(*red)[1][16][64] = reinterpret_cast<float(*)[1][16][64]>(dsmem);
+  skinny_finish<1, EPI>(red, tile, rows, wave, 0, M, N, nullptr, out, ldo, 0);
 }
 
 // ---- 33 to 64 tokens, large grids: two tiles of W share the activations ---------------------------
@@ -566,6 +685,58 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   return 0;
 }
 
+static int sk_check_norm(const char* who, const float* resid, const float* delta, int slabs, long long slab_stride,
+                         const float* norm_w, float eps, const float* resid_out, int M, int K) {
+  PICO_REQUIRE(M == 1, "%s: one row, got %d", who, M);
+  PICO_REQUIRE(K > 0 && K % 64 == 0 && K <= SK_NORM_MAX_K, "%s: K = %d must be a multiple of 64 up to %d", who, K, SK_NORM_MAX_K);
+  PICO_REQUIRE(resid && norm_w && resid_out && resid_out != resid, "%s: the residual stream needs a buffer of its own to go to", who);
+  PICO_REQUIRE(eps > 0.f, "%s: eps must be positive", who);
+  PICO_REQUIRE(delta ? (slabs >= 1 && slabs <= MAX_SK_SLABS && slab_stride >= (long long)M * K && slab_stride % 4 == 0) : slabs == 0,
+               "%s: 1 to %d slabs of at least M * K floats each, or none (got %d, stride %lld)", who, MAX_SK_SLABS, slabs, slab_stride);
+  PICO_REQUIRE((uintptr_t)resid % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)norm_w % 16 == 0 && (uintptr_t)resid_out % 16 == 0,
+               "%s: the norm's operands must be 16-byte aligned", who);
+  return 0;
+}
+
+template <typename Kernel>
+static int sk_raise_lds(Kernel kernel, int bytes, const char* who) {
+  PICO_REQUIRE(bytes <= 160 * 1024, "%s: %d bytes of LDS are more than a compute unit has", who, bytes);
+  if (bytes > 48 * 1024 && hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    pico_set_error("%s: %d bytes of LDS refused", who, bytes);
+    return -1;
+  }
+  return 0;
+}
+
+// out = epilogue(norm(resid + slabs) W^T) for one row, the norm as pico_add_rmsnorm
+// computes it; resid_out [M, K] gets resid + slabs.  epilogue: EPI_BF16, EPI_F32 (one slab) or EPI_SWIGLU.
+extern "C" int pico_gemm_skinny_norm(const float* resid, const float* delta, int slabs, long long slab_stride,
+                                     const float* norm_w, float eps, float* resid_out, const void* W, int ldw, void* out,
+                                     int ldo, int epilogue, int M, int N, int K, hipStream_t stream) {
+  if (sk_check_norm("pico_gemm_skinny_norm", resid, delta, slabs, slab_stride, norm_w, eps, resid_out, M, K)) return -1;
+  PICO_REQUIRE(N > 0 && ldw % 8 == 0 && ldw >= K && (uintptr_t)W % 16 == 0, "pico_gemm_skinny_norm: W must be 16-byte aligned with a row stride that is a multiple of 8");
+  PICO_REQUIRE(epilogue >= 0 && epilogue <= 2, "pico_gemm_skinny_norm: unknown epilogue %d", epilogue);
+  PICO_REQUIRE(epilogue != EPI_SWIGLU || N % 2 == 0, "pico_gemm_skinny_norm: SwiGLU needs an even N");
+  const int n_out = epilogue == EPI_SWIGLU ? N / 2 : N;
+  PICO_REQUIRE(ldo >= n_out, "pico_gemm_skinny_norm: output row stride too small");
+  const int unit = epilogue == EPI_SWIGLU ? 2 : 1;
+  const int rows = skinny_tile_height(n_out, unit, 1, 8);
+  const int tiles = (n_out + rows - 1) / rows;
+  const int smem = sk_xs_smem_bytes(SK_NORM_DEPTH, K);
+  const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
+#define LAUNCHN(EPI)                                                                                      \
+  do {                                                                                                    \
+    if (sk_raise_lds(gemm_skinny_norm_kernel<EPI>, smem, "pico_gemm_skinny_norm")) return -1;             \
+    gemm_skinny_norm_kernel<EPI><<<dim3(tiles), 256, smem, stream>>>(in, (const bf16_t*)W, ldw, out, ldo, M, N, K, rows); \
+  } while (0)
+  if (epilogue == EPI_BF16) LAUNCHN(EPI_BF16);
+  else if (epilogue == EPI_F32) LAUNCHN(EPI_F32);
+  else LAUNCHN(EPI_SWIGLU);
+#undef LAUNCHN
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------------------
 // The q/k/v projection of a decode step with everything that follows it before attention:
 // bias, rotate-half position encoding of q and k (pico_vllm/kernels/fused_rope_kvcache_store.py:51-101
@@ -579,14 +750,14 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
 //   K pages [page][kv head][slot][d], V pages [page][kv head][d][slot], P = 1 << pshift slots;
 //   slots[m] = page * P + slot of token m, negative: store nothing.
 // ---------------------------------------------------------------------------
-template <int MT, bool TAIL, int NX>
-__global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
+// XS: the activations are put into LDS at `xs` by `between` (a norm in front of the projection) and stay there.
+template <int MT, bool TAIL, int NX, bool XS = false, typename Before = SkNothing, typename Between = SkNothing>
+__device__ __forceinline__ void skinny_rope_body(
     const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
     bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
     bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
-    int nq, int nkv, int d, int pshift, int num_pages, int pairs) {
-  // the grid of this projection is small (one workgroup per 32 of (nq + 2 nkv) d rows): four waves always
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, true>()];
+    int nq, int nkv, int d, int pshift, int num_pages, int pairs, char* smem, const char* xs = nullptr,
+    Before before = Before(), Between between = Between()) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int half = d >> 1, tiles_per_head = half / pairs;
   const int head = blockIdx.x / tiles_per_head, tp = blockIdx.x % tiles_per_head;
@@ -637,7 +808,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
       }
     }
   }
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, true>(X, ldx, W, ldw, tr, m0, M, 0, K, smem);
+  float(*red)[MT][16][64];
+  if constexpr (XS) {
+    skinny_stream_lds<1, 1, 4, sk_depth<1, true>(), true>(nullptr, 0, W, ldw, tr, m0, M, 0, K, smem, xs, before, between);
+    red = reinterpret_cast<float(*)[MT][16][64]>(smem);
+  } else {
+    red = skinny_tile<MT, TAIL, NX, true>(X, ldx, W, ldw, tr, m0, M, 0, K, smem);
+  }
   if (!mine) return;
 
 #pragma unroll
@@ -681,6 +858,33 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
   }
 }
 
+template <int MT, bool TAIL, int NX>
+__global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
+    const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
+    bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
+    bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
+    int nq, int nkv, int d, int pshift, int num_pages, int pairs) {
+  // the grid of this projection is small (one workgroup per 32 of (nq + 2 nkv) d rows): four waves always
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, true>()];
+  skinny_rope_body<MT, TAIL, NX>(X, ldx, W, ldw, bias, q_out, ldq, cos_sin, slots, k_cache, v_cache, M, K, nq, nkv, d, pshift,
+                                 num_pages, pairs, smem);
+}
+
+// the same with the norm of the one row in front (SkNormIn), the activations staying in LDS
+__global__ __launch_bounds__(256) void gemm_skinny_rope_norm_kernel(
+    SkNormIn in, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
+    bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
+    bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
+    int nq, int nkv, int d, int pshift, int num_pages, int pairs) {
+  extern __shared__ __attribute__((aligned(16))) char dsmem[];
+  __shared__ float scratch[16];
+  char* xs = dsmem + sk_xs_offset<sk_depth<1, true>()>();
+  SkNormRow row;
+  skinny_rope_body<1, false, 1, true>(nullptr, 0, W, ldw, bias, q_out, ldq, cos_sin, slots, k_cache, v_cache, M, K, nq, nkv, d,
+                                      pshift, num_pages, pairs, dsmem, xs, [&]() { row.load(in, K); },
+                                      [&]() { row.finish(in, K, xs, scratch, blockIdx.x == 0); });
+}
+
 extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int ldw, const float* bias, void* q_out,
                                      int ldq, const float* cos_sin, const int* slots,
                                      void* k_cache, void* v_cache, int M, int K, int nq, int nkv, int d, int P,
@@ -714,6 +918,35 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   else if (mt == 1) LAUNCH(1, true, 0);
   else LAUNCH(2, true, 0);
 #undef LAUNCH
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// pico_gemm_skinny_rope with the norm of the rows in front: X = norm(resid + slabs) as pico_add_rmsnorm computes it
+// (one row); resid_out [1, K] gets resid + slabs.
+extern "C" int pico_gemm_skinny_rope_norm(const float* resid, const float* delta, int slabs, long long slab_stride,
+                                          const float* norm_w, float eps, float* resid_out, const void* W, int ldw,
+                                          const float* bias, void* q_out, int ldq, const float* cos_sin, const int* slots,
+                                          void* k_cache, void* v_cache, int M, int K, int nq, int nkv, int d, int P,
+                                          int num_pages, hipStream_t stream) {
+  if (sk_check_norm("pico_gemm_skinny_rope_norm", resid, delta, slabs, slab_stride, norm_w, eps, resid_out, M, K)) return -1;
+  PICO_REQUIRE(cos_sin != nullptr && (uintptr_t)cos_sin % 8 == 0, "pico_gemm_skinny_rope_norm: no table of cosines and sines");
+  PICO_REQUIRE(nq > 0 && nkv > 0 && num_pages > 0, "pico_gemm_skinny_rope_norm: bad sizes");
+  PICO_REQUIRE(d >= 32 && d % 32 == 0, "pico_gemm_skinny_rope_norm: head size %d is not a multiple of 32", d);
+  PICO_REQUIRE(P >= 1 && (P & (P - 1)) == 0, "pico_gemm_skinny_rope_norm: page size %d is not a power of two", P);
+  PICO_REQUIRE(ldw % 8 == 0 && ldw >= K && (uintptr_t)W % 16 == 0, "pico_gemm_skinny_rope_norm: W must be 16-byte aligned with a row stride that is a multiple of 8");
+  PICO_REQUIRE(ldq >= nq * d && ldq % 4 == 0 && (uintptr_t)q_out % 8 == 0 && (uintptr_t)k_cache % 8 == 0,
+               "pico_gemm_skinny_rope_norm: q and the cache must be 8-byte aligned, the q row stride a multiple of 4");
+  int pshift = 0;
+  while ((1 << pshift) < P) pshift++;
+  int pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, 8, nullptr, 1, 4);
+  if (pairs == 12) pairs = 16;
+  const int smem = sk_xs_smem_bytes(sk_depth<1, true>(), K);
+  if (sk_raise_lds(gemm_skinny_rope_norm_kernel, smem, "pico_gemm_skinny_rope_norm")) return -1;
+  const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
+  gemm_skinny_rope_norm_kernel<<<dim3((nq + 2 * nkv) * (d / 2 / pairs)), 256, smem, stream>>>(
+      in, (const bf16_t*)W, ldw, bias, (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K,
+      nq, nkv, d, pshift, num_pages, pairs);
   PICO_LAUNCH_CHECK();
   return 0;
 }

@@ -80,10 +80,17 @@ class Linear:
             return torch.addmm(self.bias, x, self.weight.t())
         return torch.mm(x, self.weight.t())
 
-    def swiglu(self, x: torch.Tensor) -> torch.Tensor:
+    def swiglu(self, x) -> torch.Tensor:
         """silu(gate) * up where [gate; up] = x W^T (W's first half of rows is the gate).  With few
         rows the activation is the epilogue of the weight-streaming kernel and [gate; up] never
-        reaches memory."""
+        reaches memory.  x may be a norm that has not run (``parts.base.DeferredNorm``): with one
+        row it becomes the same kernel's prologue."""
+        if hasattr(x, "resid_in"):
+            if (x.kind == "rms" and self.bias is None and kernels.skinny_norm_ok(x.resid_in, x.delta, self.weight)
+                    and self.out_features % 2 == 0):
+                out, x.resid = kernels.gemm_skinny_norm(x.resid_in, x.delta, x.weight, x.eps, self.weight, kernels.EPI_SWIGLU)
+                return out
+            x = x.run()
         if self.weight.dtype == torch.bfloat16 and self.bias is None and kernels.skinny_ok(x, self.weight):
             return kernels.gemm_skinny(x, self.weight, None, kernels.EPI_SWIGLU)
         return kernels.swiglu(self(x))

@@ -8,7 +8,7 @@ import torch
 
 from ..ops import kernels
 from ..ops.linear import Linear
-from .base import Mixer, StepContext
+from .base import DeferredNorm, Mixer, StepContext
 from .registry import build_part, register_part
 from .spec import CacheSpec, ParamSpec, PartSpec
 
@@ -25,6 +25,8 @@ class GQAAttention(Mixer):
     makes a prompt cut into portions equal the whole prompt.  The checkpoint
     holds q_proj, k_proj and v_proj separately; they are concatenated at load.
     ``window`` > 0 restricts every query to the last ``window`` keys."""
+
+    takes_deferred_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, position: PartSpec, window: int = 0,
@@ -69,6 +71,8 @@ class GQAAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         nq, nkv, d = self.nq, self.nkv, self.d
         bt = ctx.block_tables[cache.group]
+        if isinstance(x, DeferredNorm) and not getattr(self.position, "takes_deferred_norm", False):
+            x = x.run()
         # [T, >= nq d]: the encoded queries first; keys and values are in the cache after this
         qkv = self.position.project_rotate_store(x, self.qkv, ctx, cache, bt, nq, nkv, d)
         if self.fast is not None and cache.k.dtype == torch.bfloat16:

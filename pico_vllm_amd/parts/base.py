@@ -8,7 +8,7 @@ part's prefix) and puts what it needs on the device; ``forward`` runs on the
 GPU.
 
 Interfaces:
-  Norm.add_norm(resid, delta, rows=None) -> normed
+  Norm.add_norm(resid, delta, rows=None) -> normed;  Norm.deferred(resid, delta) -> DeferredNorm or None
   PositionEncoding.rotate_and_store(qkv, ctx, kv, block_table, nq, nkv, d)
   Mixer.cache_spec() -> CacheSpec;  Mixer.forward(x, ctx, cache) -> y
   FeedForward.forward(x, ctx) -> y
@@ -60,7 +60,31 @@ class Part:
         pass
 
 
+class DeferredNorm:
+    """A norm whose operands are known but which has not run: ``resid_in + delta`` normed.  A block hands
+    this, instead of the normed activations, to a consumer that says ``takes_deferred_norm`` and whose first
+    kernel may do the norm itself (one launch less in a step of one token).  The consumer either
+    does so and sets ``resid`` to the residual stream after the sum, or calls ``run()``, which is the
+    norm's own kernel.  ``kind``, ``weight`` and ``eps`` say which norm it is ("rms": RMSNorm)."""
+
+    def __init__(self, norm: "Norm", resid_in: torch.Tensor, delta: Optional[torch.Tensor], kind: str,
+                 weight: torch.Tensor, eps: float):
+        self.norm, self.resid_in, self.delta = norm, resid_in, delta
+        self.kind, self.weight, self.eps = kind, weight, eps
+        self.resid: Optional[torch.Tensor] = None
+
+    def run(self) -> torch.Tensor:
+        h = self.norm.add_norm(self.resid_in, self.delta)
+        self.resid = self.resid_in          # summed in place
+        return h
+
+
 class Norm(Part):
+    def deferred(self, resid: torch.Tensor, delta: Optional[torch.Tensor]) -> Optional[DeferredNorm]:
+        """The norm of ``resid + delta`` as something a consumer may run inside its own first kernel, or
+        None where that cannot pay (the default)."""
+        return None
+
     def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """resid (float32 [T, H]) += delta, returns the normed rows in the activation dtype;
@@ -79,13 +103,18 @@ class PositionEncoding(Part):
     def project_rotate_store(self, x: torch.Tensor, linear, ctx: StepContext, kv, block_table: torch.Tensor,
                              nq: int, nkv: int, d: int) -> torch.Tensor:
         """qkv = linear(x), then ``rotate_and_store``; returns a tensor whose first nq * d columns are
-        the encoded queries.  An encoding may override this to fuse the three steps."""
+        the encoded queries.  An encoding may override this to fuse the three steps; one that sets
+        ``takes_deferred_norm`` may be given a ``DeferredNorm`` as x."""
+        if isinstance(x, DeferredNorm):
+            x = x.run()
         qkv = linear(x)
         self.rotate_and_store(qkv, ctx, kv, block_table, nq, nkv, d)
         return qkv
 
 
 class Mixer(Part):
+    takes_deferred_norm = False      # True: forward may be given a DeferredNorm as x (and must run or fuse it)
+
     def cache_spec(self) -> CacheSpec:
         return CacheSpec("none")
 
@@ -96,6 +125,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_deferred_norm = False      # as for a mixer
+
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 

@@ -18,6 +18,8 @@ class SwiGLUMLP(FeedForward):
     checkpoint holds gate_proj and up_proj separately; they are concatenated
     at load so one GEMM makes both."""
 
+    takes_deferred_norm = True      # Linear.swiglu runs or fuses it
+
     def __init__(self, hidden_size: int, intermediate_size: int, act_dtype: torch.dtype = torch.bfloat16):
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.gate_up: Optional[Linear] = None

@@ -6,7 +6,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..ops import kernels
-from .base import Norm
+from .base import DeferredNorm, Norm
 from .registry import register_part
 from .spec import ParamSpec
 
@@ -27,3 +27,10 @@ class RMSNorm(Norm):
 
     def add_norm(self, resid, delta, rows=None):
         return kernels.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
+
+    def deferred(self, resid, delta):
+        # the one row of a bfloat16 step: the projection behind the norm can norm it itself
+        if (self.act_dtype == torch.bfloat16 and resid.shape[0] <= kernels.SKINNY_NORM_ROWS
+                and (delta is None or delta.dtype == torch.float32)):
+            return DeferredNorm(self, resid, delta, "rms", self.weight, self.eps)
+        return None

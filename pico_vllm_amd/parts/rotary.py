@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import kernels
-from .base import PositionEncoding
+from .base import DeferredNorm, PositionEncoding
 from .registry import register_part
 
 
@@ -38,10 +38,20 @@ class RotaryHalf(PositionEncoding):
     def rotate_and_store(self, qkv, ctx, kv, block_table, nq, nkv, d) -> None:
         kernels.rope_kv_store(qkv, self.table(ctx), ctx.slot_mapping[kv.group], kv.k, kv.v, nq, nkv, d, self.rotary_dim)
 
+    takes_deferred_norm = True
+
     def project_rotate_store(self, x, linear, ctx, kv, block_table, nq, nkv, d) -> torch.Tensor:
+        fusable = (self.rotary_dim == d and d % 32 == 0 and kv.k.dtype == torch.bfloat16
+                   and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0)
+        if isinstance(x, DeferredNorm):
+            # one token: the norm in front rides on the same kernel
+            if fusable and x.kind == "rms" and kernels.skinny_norm_ok(x.resid_in, x.delta, linear.weight):
+                q, x.resid = kernels.gemm_skinny_rope_norm(x.resid_in, x.delta, x.weight, x.eps, linear.weight, linear.bias_f32,
+                                                           self.table(ctx), ctx.slot_mapping[kv.group], kv.k, kv.v, nq, nkv, d)
+                return q
+            x = x.run()
         # few tokens in bfloat16: projection, bias, rotation and cache store are one weight-streaming kernel
-        if (self.rotary_dim == d and d % 32 == 0 and kv.k.dtype == torch.bfloat16
-                and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0 and kernels.skinny_ok(x, linear.weight)):
+        if fusable and kernels.skinny_ok(x, linear.weight):
             return kernels.gemm_skinny_rope(x, linear.weight, linear.bias_f32, self.table(ctx), ctx.slot_mapping[kv.group],
                                             kv.k, kv.v, nq, nkv, d)
         return super().project_rotate_store(x, linear, ctx, kv, block_table, nq, nkv, d)

@@ -569,6 +569,71 @@ def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias
     close(vc, want_v, torch.bfloat16, scale=4)
 
 
+@pytest.mark.parametrize("N,K_,slabs", [(2048, 1536, 5), (17920, 1536, 3), (1000, 320, 1), (90, 64, 0), (640, 2048, 8),
+                                        (2 * 323, 512, -1)])
+def test_gemm_skinny_with_the_norm_in_front(K, N, K_, slabs):
+    # norm(resid + partial sums) W^T of one row in one kernel against the norm kernel followed by the product;
+    # slabs: 0 = nothing to add, -1 = one sum [1, K], else a stack [slabs, 1, K]
+    g = torch.Generator().manual_seed(N + K_)
+    resid = torch.randn(1, K_, generator=g)
+    delta = None if slabs == 0 else torch.randn((1, K_) if slabs < 0 else (slabs, 1, K_), generator=g)
+    nw = 1 + 0.1 * torch.randn(K_, generator=g)
+    w = (torch.randn(N, K_, generator=g) / math.sqrt(K_)).bfloat16().to(DEV)
+    eps = 1e-5
+    d_dev = None if delta is None else delta.to(DEV)
+    assert K.skinny_norm_ok(resid.to(DEV), d_dev, w)
+    assert not K.skinny_norm_ok(torch.randn(2, K_).to(DEV), None, w)
+    r2 = resid.clone().to(DEV)
+    h = K.add_rmsnorm(r2, d_dev, nw.to(DEV), eps, torch.bfloat16)              # the two kernels: r2 is summed in place
+    total = resid.double() + (0 if delta is None else delta.double().reshape(-1, 1, K_).sum(0))
+    for epi in (K.EPI_F32, K.EPI_BF16, K.EPI_SWIGLU):
+        out, r_out = K.gemm_skinny_norm(resid.to(DEV), d_dev, nw.to(DEV), eps, w, epi)
+        assert torch.equal(r_out, r2)                                            # the same sums in the same order
+        want = K.gemm_skinny(h, w, None, epi)
+        scale = float(want.float().abs().max())
+        # the sum of squares is formed by other threads: the normed row may differ in a last bfloat16 bit
+        assert float((out.float() - want.float()).abs().max()) <= 2e-2 * scale, epi
+        assert float((out.float() - want.float()).abs().mean()) <= 1e-3 * scale, epi
+        if epi == K.EPI_F32:
+            close(out, (P.rms_norm(total.float(), nw, eps).bfloat16().double() @ w.cpu().double().T).float(), torch.bfloat16, scale=4)
+    assert torch.allclose(r_out.cpu().double(), total, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("nq,nkv,d,H,Pg,bias,slabs", [(12, 2, 128, 1536, 16, True, 5), (6, 3, 32, 192, 8, True, 0),
+                                                      (3, 1, 64, 128, 32, False, 1), (4, 2, 64, 320, 16, True, 3)])
+def test_gemm_skinny_with_the_norm_in_front_and_rotation_and_cache_store(K, nq, nkv, d, H, Pg, bias, slabs):
+    theta = 1e6
+    g = torch.Generator().manual_seed(d + H)
+    resid = torch.randn(1, H, generator=g)
+    delta = None if slabs == 0 else torch.randn(slabs, 1, H, generator=g)
+    nw = 1 + 0.1 * torch.randn(H, generator=g)
+    N = (nq + 2 * nkv) * d
+    w = (torch.randn(N, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
+    b = torch.randn(N, generator=g).to(DEV) if bias else None
+    pos = torch.randint(0, 5000, (1,), generator=g, dtype=torch.int32)
+    slots = torch.tensor([3 * Pg + 5], dtype=torch.int32, device=DEV)
+    inv = (1.0 / (theta ** (torch.arange(0, d, 2).float() / d))).to(DEV)
+    table = K.rope_table(pos.to(DEV), inv)
+    d_dev = None if delta is None else delta.to(DEV)
+    caches = []
+    for fused in (False, True):
+        kc = torch.full((6, nkv, Pg, d), 7.0, dtype=torch.bfloat16, device=DEV)
+        vc = torch.full((6, nkv, d, Pg), 7.0, dtype=torch.bfloat16, device=DEV)
+        if fused:
+            q, r_out = K.gemm_skinny_rope_norm(resid.to(DEV), d_dev, nw.to(DEV), 1e-6, w, b, table, slots, kc, vc, nq, nkv, d)
+        else:
+            r_out = resid.clone().to(DEV)
+            h = K.add_rmsnorm(r_out, d_dev, nw.to(DEV), 1e-6, torch.bfloat16)
+            q = K.gemm_skinny_rope(h, w, b, table, slots, kc, vc, nq, nkv, d)
+        caches.append((q.float(), r_out, kc.float(), vc.float()))
+    (q0, r0, k0, v0), (q1, r1, k1, v1) = caches
+    assert torch.equal(r0, r1)
+    for a, c in ((q0, q1), (k0, k1), (v0, v1)):
+        scale = float(a.abs().max())
+        assert float((a - c).abs().max()) <= 2e-2 * scale and float((a - c).abs().mean()) <= 1e-3 * scale
+    assert float((k0 == 7.0).float().mean()) > 0.5 and torch.equal(k0 == 7.0, k1 == 7.0)     # only the token's slot was written
+
+
 def test_gemm_skinny_refuses_misaligned_operands(K):
     a = torch.randn(4, 172).bfloat16().to(DEV)          # K = 172 is no multiple of 8
     w = torch.randn(64, 172).bfloat16().to(DEV)
