@@ -374,8 +374,8 @@ struct SkNormIn {
   float eps;
   float* resid_out;          // [M, K] float32: resid + the slabs, written by workgroup 0
 };
-constexpr int SK_NORM_VPT = 2;                         // groups of four elements a thread: K <= 256 * 4 * 2
-constexpr int SK_NORM_MAX_K = 256 * 4 * SK_NORM_VPT;
+constexpr int SK_NORM_MAX_VPT = 4;                     // groups of four elements a thread: K <= 256 * 4 * 4
+constexpr int SK_NORM_MAX_K = 256 * 4 * SK_NORM_MAX_VPT;
 #ifndef SK_NORM_DEPTH
 #define SK_NORM_DEPTH 3                                // slices a wave keeps in flight in the projections of many tiles
 #endif
@@ -384,12 +384,14 @@ constexpr int SK_NORM_MAX_K = 256 * 4 * SK_NORM_VPT;
 // issued: vector memory returns in order, and behind those copies this small read from the caches would wait
 // for HBM); `finish` sums, norms and writes the row into xs as bfloat16 [K].
 // All 256 threads of the workgroup take part in both.
+// VPT: groups of four elements a thread holds (K <= 1024 VPT): what is loaded early waits in registers.
+template <int VPT>
 struct SkNormRow {
-  float4 v[SK_NORM_VPT], g[SK_NORM_VPT], d[SK_NORM_VPT][MAX_SK_SLABS];
+  float4 v[VPT], g[VPT], d[VPT][MAX_SK_SLABS];
 
   __device__ __forceinline__ void load(const SkNormIn& in, int K) {
 #pragma unroll
-    for (int j = 0; j < SK_NORM_VPT; j++) {
+    for (int j = 0; j < VPT; j++) {
       const int i = 4 * threadIdx.x + 1024 * j;
       v[j] = g[j] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
@@ -407,7 +409,7 @@ struct SkNormRow {
   __device__ __forceinline__ void finish(const SkNormIn& in, int K, char* xs, float* scratch, bool writer) {
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < SK_NORM_VPT; j++) {
+    for (int j = 0; j < VPT; j++) {
       const int i = 4 * threadIdx.x + 1024 * j;
 #pragma unroll
       for (int sl = 0; sl < MAX_SK_SLABS; sl++) { v[j].x += d[j][sl].x; v[j].y += d[j][sl].y; v[j].z += d[j][sl].z; v[j].w += d[j][sl].w; }
@@ -419,7 +421,7 @@ struct SkNormRow {
     ss = block_sum(ss, scratch);
     const float r = 1.0f / sqrtf(ss / (float)K + in.eps);
 #pragma unroll
-    for (int j = 0; j < SK_NORM_VPT; j++) {
+    for (int j = 0; j < VPT; j++) {
       const int i = 4 * threadIdx.x + 1024 * j;
       if (i < K) {
         *reinterpret_cast<uint2*>(xs + 2 * i) = make_uint2(pack2_bf16(v[j].x * r * g[j].x, v[j].y * r * g[j].y),
@@ -436,7 +438,7 @@ struct SkNormRow {
 template <int DEPTH> constexpr int sk_xs_offset() { return DEPTH * 4 * 4 * SK_GROUP; }
 static int sk_xs_smem_bytes(int depth, int K) { return depth * 4 * 4 * SK_GROUP + 2 * K; }
 
-template <int EPI>
+template <int EPI, int VPT>
 __global__ __launch_bounds__(256) void gemm_skinny_norm_kernel(SkNormIn in, const bf16_t* __restrict__ W, int ldw,
                                                                void* __restrict__ out, int ldo, int M, int N, int K,
                                                                int rows) {
@@ -445,7 +447,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_norm_kernel(SkNormIn in, cons
   __shared__ float scratch[16];
   char* xs = dsmem + sk_xs_offset<DEPTH>();
   const int wave = threadIdx.x >> 6, tile = blockIdx.x;
-  SkNormRow row;
+  SkNormRow<VPT> row;
   skinny_stream_lds<1, 1, 4, DEPTH, true>(nullptr, 0, W, ldw, skinny_rows<EPI>(tile, rows, N), 0, M, 0, K, dsmem, xs,
                                           [&]() { row.load(in, K); },
                                           [&]() { row.finish(in, K, xs, scratch, blockIdx.x == 0); });
@@ -724,15 +726,21 @@ extern "C" int pico_gemm_skinny_norm(const float* resid, const float* delta, int
   const int tiles = (n_out + rows - 1) / rows;
   const int smem = sk_xs_smem_bytes(SK_NORM_DEPTH, K);
   const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
-#define LAUNCHN(EPI)                                                                                      \
+#define LAUNCHV(EPI, VPT)                                                                                  \
   do {                                                                                                    \
-    if (sk_raise_lds(gemm_skinny_norm_kernel<EPI>, smem, "pico_gemm_skinny_norm")) return -1;             \
-    gemm_skinny_norm_kernel<EPI><<<dim3(tiles), 256, smem, stream>>>(in, (const bf16_t*)W, ldw, out, ldo, M, N, K, rows); \
+    if (sk_raise_lds(gemm_skinny_norm_kernel<EPI, VPT>, smem, "pico_gemm_skinny_norm")) return -1;        \
+    gemm_skinny_norm_kernel<EPI, VPT><<<dim3(tiles), 256, smem, stream>>>(in, (const bf16_t*)W, ldw, out, ldo, M, N, K, rows); \
+  } while (0)
+#define LAUNCHN(EPI)            \
+  do {                          \
+    if (K <= 2048) LAUNCHV(EPI, 2); \
+    else LAUNCHV(EPI, 4);       \
   } while (0)
   if (epilogue == EPI_BF16) LAUNCHN(EPI_BF16);
   else if (epilogue == EPI_F32) LAUNCHN(EPI_F32);
   else LAUNCHN(EPI_SWIGLU);
 #undef LAUNCHN
+#undef LAUNCHV
   PICO_LAUNCH_CHECK();
   return 0;
 }
@@ -871,6 +879,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
 }
 
 // the same with the norm of the one row in front (SkNormIn), the activations staying in LDS
+template <int VPT>
 __global__ __launch_bounds__(256) void gemm_skinny_rope_norm_kernel(
     SkNormIn in, const bf16_t* __restrict__ W, int ldw, const float* __restrict__ bias,
     bf16_t* __restrict__ q_out, int ldq, const float2* __restrict__ cos_sin, const int* __restrict__ slots,
@@ -879,7 +888,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_norm_kernel(
   extern __shared__ __attribute__((aligned(16))) char dsmem[];
   __shared__ float scratch[16];
   char* xs = dsmem + sk_xs_offset<sk_depth<1, true>()>();
-  SkNormRow row;
+  SkNormRow<VPT> row;
   skinny_rope_body<1, false, 1, true>(nullptr, 0, W, ldw, bias, q_out, ldq, cos_sin, slots, k_cache, v_cache, M, K, nq, nkv, d,
                                       pshift, num_pages, pairs, dsmem, xs, [&]() { row.load(in, K); },
                                       [&]() { row.finish(in, K, xs, scratch, blockIdx.x == 0); });
@@ -942,11 +951,17 @@ extern "C" int pico_gemm_skinny_rope_norm(const float* resid, const float* delta
   int pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, 8, nullptr, 1, 4);
   if (pairs == 12) pairs = 16;
   const int smem = sk_xs_smem_bytes(sk_depth<1, true>(), K);
-  if (sk_raise_lds(gemm_skinny_rope_norm_kernel, smem, "pico_gemm_skinny_rope_norm")) return -1;
   const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
-  gemm_skinny_rope_norm_kernel<<<dim3((nq + 2 * nkv) * (d / 2 / pairs)), 256, smem, stream>>>(
-      in, (const bf16_t*)W, ldw, bias, (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K,
-      nq, nkv, d, pshift, num_pages, pairs);
+#define LAUNCHR(VPT)                                                                                              \
+  do {                                                                                                            \
+    if (sk_raise_lds(gemm_skinny_rope_norm_kernel<VPT>, smem, "pico_gemm_skinny_rope_norm")) return -1;           \
+    gemm_skinny_rope_norm_kernel<VPT><<<dim3((nq + 2 * nkv) * (d / 2 / pairs)), 256, smem, stream>>>(            \
+        in, (const bf16_t*)W, ldw, bias, (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache,    \
+        (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages, pairs);                                            \
+  } while (0)
+  if (K <= 2048) LAUNCHR(2);
+  else LAUNCHR(4);
+#undef LAUNCHR
   PICO_LAUNCH_CHECK();
   return 0;
 }

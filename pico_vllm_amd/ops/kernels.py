@@ -347,7 +347,7 @@ def gemm_skinny_rope(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
 
 # The norm in front of a projection inside the projection's launch: every workgroup norms the row itself, which
 # pays for a single row (a decode step of one request: a launch of 4.5 us saved, some reading added).
-SKINNY_NORM_ROWS, SKINNY_NORM_MAX_K, SKINNY_NORM_SLABS = 1, 2048, 8
+SKINNY_NORM_ROWS, SKINNY_NORM_MAX_K, SKINNY_NORM_SLABS = 1, 4096, 8
 
 
 def skinny_norm_ok(resid: torch.Tensor, delta: Optional[torch.Tensor], w: torch.Tensor) -> bool:

@@ -570,7 +570,7 @@ def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias
 
 
 @pytest.mark.parametrize("N,K_,slabs", [(2048, 1536, 5), (17920, 1536, 3), (1000, 320, 1), (90, 64, 0), (640, 2048, 8),
-                                        (2 * 323, 512, -1)])
+                                        (2 * 323, 512, -1), (1000, 3584, 6), (512, 4096, 8), (384, 2112, 0)])
 def test_gemm_skinny_with_the_norm_in_front(K, N, K_, slabs):
     # norm(resid + partial sums) W^T of one row in one kernel against the norm kernel followed by the product;
     # slabs: 0 = nothing to add, -1 = one sum [1, K], else a stack [slabs, 1, K]
@@ -600,7 +600,8 @@ def test_gemm_skinny_with_the_norm_in_front(K, N, K_, slabs):
 
 
 @pytest.mark.parametrize("nq,nkv,d,H,Pg,bias,slabs", [(12, 2, 128, 1536, 16, True, 5), (6, 3, 32, 192, 8, True, 0),
-                                                      (3, 1, 64, 128, 32, False, 1), (4, 2, 64, 320, 16, True, 3)])
+                                                      (3, 1, 64, 128, 32, False, 1), (4, 2, 64, 320, 16, True, 3),
+                                                      (28, 4, 128, 3584, 16, True, 5)])
 def test_gemm_skinny_with_the_norm_in_front_and_rotation_and_cache_store(K, nq, nkv, d, H, Pg, bias, slabs):
     theta = 1e6
     g = torch.Generator().manual_seed(d + H)
