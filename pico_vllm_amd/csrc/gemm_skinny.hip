@@ -363,8 +363,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 // one row every workgroup of the projection can do that norm itself: it reads the row of the
 // residual stream, the partial sums that the projection before left (pico_vllm/RMSNorm.py:22-31 for the
 // norm, the sums in slab order as pico_add_rmsnorm forms them), reduces, and writes the normed row as
-// bfloat16 into LDS, where it stays for all slices; only W streams.  Workgroup 0 also writes the new residual stream, to another buffer than the one the other
-// workgroups still read.
+// bfloat16 into LDS, where it stays for all slices; only W streams.  Workgroup 0 also writes the new
+// residual stream, to another buffer than the one the other workgroups still read.
 struct SkNormIn {
   const float* resid;        // [M, K] float32, the residual stream before the sum
   const float* delta;        // `slabs` partial sums [M, K] float32, slab s at delta + s * slab_stride; null: nothing to add
@@ -376,9 +376,8 @@ struct SkNormIn {
 };
 constexpr int SK_NORM_MAX_VPT = 4;                     // groups of four elements a thread: K <= 256 * 4 * 4
 constexpr int SK_NORM_MAX_K = 256 * 4 * SK_NORM_MAX_VPT;
-#ifndef SK_NORM_DEPTH
-#define SK_NORM_DEPTH 3                                // slices a wave keeps in flight in the projections of many tiles
-#endif
+constexpr int SK_NORM_DEPTH = 3;                       // slices a wave keeps in flight in the projections of many tiles:
+                                                       // 50 KB of stages and the row leave room for three workgroups a compute unit
 
 // The one row: `load` requests the row, its partial sums and the norm's weight (before the first copies of W are
 // issued: vector memory returns in order, and behind those copies this small read from the caches would wait
@@ -434,7 +433,7 @@ struct SkNormRow {
   }
 };
 
-// stages of the stream (4 waves, W only), then the normed rows
+// stages of the stream (4 waves, W only), then the normed row
 template <int DEPTH> constexpr int sk_xs_offset() { return DEPTH * 4 * 4 * SK_GROUP; }
 static int sk_xs_smem_bytes(int depth, int K) { return depth * 4 * 4 * SK_GROUP + 2 * K; }
 
