@@ -409,3 +409,58 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(dtype):
             r.advance(seqs)
             fed += n
         close(torch.cat(got), whole_logits, dtype, scale=float(whole_logits.std()) * 3)
+
+
+def test_a_block_leaves_the_norm_of_a_single_row_to_a_part_that_takes_it():
+    """With one row in bfloat16 the block hands a part that says so the norm's operands instead of
+    normed activations.  A part that runs the norm itself sees what the norm's kernel gives, the
+    residual stream is summed either way, parts that do not say so get tensors, and a part that
+    takes the operands and drops them is caught."""
+    from pico_vllm_amd.parts.base import DeferredNorm, FeedForward, Mixer
+    from pico_vllm_amd.parts.block import PreNormBlock
+    from pico_vllm_amd.parts.norm import RMSNorm
+    H = 128
+    g = torch.Generator().manual_seed(0)
+    seen = []
+
+    class Plain(Mixer):                       # does not take deferred norms
+        def forward(self, x, ctx, cache):
+            seen.append(("mixer", type(x)))
+            return 0.5 * x.float()
+
+    class Runs(FeedForward):
+        takes_deferred_norm = True
+
+        def forward(self, x, ctx):
+            seen.append(("ff", type(x)))
+            h = x.run() if isinstance(x, DeferredNorm) else x
+            return 2.0 * h.float()
+
+    class Drops(FeedForward):
+        takes_deferred_norm = True
+
+        def forward(self, x, ctx):
+            return torch.zeros(x.resid_in.shape, device=DEV)
+
+    def block(ff):
+        norms = [RMSNorm(H, 1e-5, torch.bfloat16) for _ in range(2)]
+        for n in norms:
+            n.load({"weight": 1 + 0.1 * torch.randn(H, generator=g)}, DEV, torch.bfloat16)
+        return PreNormBlock({"norm1": norms[0], "mixer": Plain(), "norm2": norms[1], "ff": ff}), norms
+
+    for T in (1, 3):
+        seen.clear()
+        blk, norms = block(Runs())
+        x0 = torch.randn(T, H, generator=g)
+        pend = torch.randn(T, H, generator=g)
+        resid, out = blk.forward(x0.clone().to(DEV), pend.to(DEV), None, None)
+        assert seen[0] == ("mixer", torch.Tensor)
+        assert seen[1] == ("ff", DeferredNorm if T == 1 else torch.Tensor)
+        r1 = x0 + pend
+        h1 = P.rms_norm(r1, norms[0].weight.cpu(), 1e-5).bfloat16().float()
+        r2 = r1 + 0.5 * h1
+        close(resid, r2, torch.float32, scale=4)
+        close(out, 2.0 * P.rms_norm(r2, norms[1].weight.cpu(), 1e-5), torch.bfloat16, scale=8)
+    blk, _ = block(Drops())
+    with pytest.raises(RuntimeError, match="deferred norm"):
+        blk.forward(torch.randn(1, H).to(DEV), None, None, None)
