@@ -699,13 +699,17 @@ static int sk_check_norm(const char* who, const float* resid, const float* delta
   return 0;
 }
 
+// A kernel may be launched with `bytes` of dynamic LDS once it has been allowed that much; `allowed` is the
+// kernel's own record of it (one per instantiation, at the call site).
 template <typename Kernel>
-static int sk_raise_lds(Kernel kernel, int bytes, const char* who) {
+static int sk_raise_lds(Kernel kernel, int bytes, int* allowed, const char* who) {
   PICO_REQUIRE(bytes <= 160 * 1024, "%s: %d bytes of LDS are more than a compute unit has", who, bytes);
-  if (bytes > 48 * 1024 && hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+  if (bytes <= *allowed) return 0;
+  if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
     pico_set_error("%s: %d bytes of LDS refused", who, bytes);
     return -1;
   }
+  *allowed = bytes;
   return 0;
 }
 
@@ -727,7 +731,8 @@ extern "C" int pico_gemm_skinny_norm(const float* resid, const float* delta, int
   const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
 #define LAUNCHV(EPI, VPT)                                                                                  \
   do {                                                                                                    \
-    if (sk_raise_lds(gemm_skinny_norm_kernel<EPI, VPT>, smem, "pico_gemm_skinny_norm")) return -1;        \
+    static int allowed = 0;                                                                               \
+    if (sk_raise_lds(gemm_skinny_norm_kernel<EPI, VPT>, smem, &allowed, "pico_gemm_skinny_norm")) return -1; \
     gemm_skinny_norm_kernel<EPI, VPT><<<dim3(tiles), 256, smem, stream>>>(in, (const bf16_t*)W, ldw, out, ldo, M, N, K, rows); \
   } while (0)
 #define LAUNCHN(EPI)            \
@@ -953,7 +958,8 @@ extern "C" int pico_gemm_skinny_rope_norm(const float* resid, const float* delta
   const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
 #define LAUNCHR(VPT)                                                                                              \
   do {                                                                                                            \
-    if (sk_raise_lds(gemm_skinny_rope_norm_kernel<VPT>, smem, "pico_gemm_skinny_rope_norm")) return -1;           \
+    static int allowed = 0;                                                                                       \
+    if (sk_raise_lds(gemm_skinny_rope_norm_kernel<VPT>, smem, &allowed, "pico_gemm_skinny_rope_norm")) return -1; \
     gemm_skinny_rope_norm_kernel<VPT><<<dim3((nq + 2 * nkv) * (d / 2 / pairs)), 256, smem, stream>>>(            \
         in, (const bf16_t*)W, ldw, bias, (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache,    \
         (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages, pairs);                                            \
