@@ -109,20 +109,28 @@ __device__ __forceinline__ void skinny_stream(const bf16_t* __restrict__ X, int 
 #define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 constexpr int SK_GROUP = 1024 + 16;
 template <int NX> constexpr int sk_stage_bytes() { return (4 + NX) * SK_GROUP; }
-// slices in flight per wave.  FEW (at most one workgroup per compute unit, the whole LDS is its own): as many
-// as fit, because such a launch is a chain of memory latencies, not a stream
-template <int NX, bool FEW> constexpr int sk_depth() { return FEW ? (NX <= 2 ? 6 : NX == 4 ? 4 : 3) : (NX >= 4 ? 2 : 3); }
+// How full the grid makes the chip (FILL): SK_FEW, at most one workgroup per compute unit; SK_MANY, more than two
+// per unit; 0 otherwise.
+// Slices in flight per wave.  SK_FEW (the whole LDS is the workgroup's own): as many as fit, because such a launch
+// is a chain of memory latencies, not a stream.  SK_MANY, up to 16 tokens: two, so that the stages are 42 to 50 KB
+// and three workgroups share a compute unit instead of two (5,141 against 5,098 tokens a second at batch 8; with
+// the normed row in LDS three workgroups gave 800 tokens a second at batch 1, two gave 747).
+#define SK_FEW 1
+#define SK_MANY 2
+template <int NX, int FILL> constexpr int sk_depth() {
+  return FILL == SK_FEW ? (NX <= 2 ? 6 : NX == 4 ? 4 : 3) : (NX >= 4 || FILL == SK_MANY) ? 2 : 3;
+}
 // waves per workgroup: two when a wave holds two blocks of tokens in LDS and the grid is large, so that
-// three workgroups fit a compute unit; four otherwise (FEW: at most one workgroup per compute unit anyway)
-template <int MT, int NX, bool FEW> constexpr int sk_waves() { return (MT == 2 && NX > 0 && !FEW) ? 2 : 4; }
+// three workgroups fit a compute unit; four otherwise (SK_FEW: at most one workgroup per compute unit anyway)
+template <int MT, int NX, int FILL> constexpr int sk_waves() { return (MT == 2 && NX > 0 && FILL != SK_FEW) ? 2 : 4; }
 // s_waitcnt for "at most n vector memory operations outstanding", nothing else waited for
 constexpr int sk_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
-template <int MT, int NX, bool FEW>
+template <int MT, int NX, int FILL>
 constexpr int sk_smem_bytes() {
   constexpr int red = 4 * MT * 16 * 64 * 4;
   if (NX == 0) return red;
-  constexpr int stages = sk_depth<NX, FEW>() * sk_waves<MT, NX, FEW>() * sk_stage_bytes<NX>();
+  constexpr int stages = sk_depth<NX, FILL>() * sk_waves<MT, NX, FILL>() * sk_stage_bytes<NX>();
   return stages > red ? stages : red;
 }
 
@@ -250,14 +258,14 @@ __device__ __forceinline__ void skinny_stream_lds(const bf16_t* __restrict__ X, 
 }
 
 // The 32 tile rows' sums for this workgroup's tokens, through LDS (NX > 0) or registers (NX == 0).
-template <int MT, bool TAIL, int NX, bool FEW>
+template <int MT, bool TAIL, int NX, int FILL>
 __device__ __forceinline__ float (*skinny_tile(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
                                                TileRows tr, int m0, int M, int k_begin, int k_end,
                                                char* smem))[MT][16][64] {
   float(*red)[MT][16][64] = reinterpret_cast<float(*)[MT][16][64]>(smem);
   if constexpr (NX > 0) {
     static_assert(!TAIL && NX <= 4 * MT, "the stream through LDS takes whole slices");
-    skinny_stream_lds<MT, NX, sk_waves<MT, NX, FEW>(), sk_depth<NX, FEW>()>(X, ldx, W, ldw, tr, m0, M, k_begin, k_end, smem);
+    skinny_stream_lds<MT, NX, sk_waves<MT, NX, FILL>(), sk_depth<NX, FILL>()>(X, ldx, W, ldw, tr, m0, M, k_begin, k_end, smem);
   } else {
     // Only a k tail must read as zero, because it is summed into outputs that are stored.
     skinny_stream<MT>(X, ldx, W + (size_t)tr.row(threadIdx.x & 31) * ldw, m0, M, k_begin, k_end, red);
@@ -340,20 +348,20 @@ __device__ __forceinline__ void skinny_finish(float (*red)[MT][16][64], int tile
   }
 }
 
-// FEW: the grid has at most one workgroup per compute unit; the whole LDS is that workgroup's, for more slices in flight
-template <int MT, int EPI, bool TAIL, int NX, bool FEW = false>
+// FILL: SK_FEW, SK_MANY or 0 (see sk_depth)
+template <int MT, int EPI, bool TAIL, int NX, int FILL = 0>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias, void* __restrict__ out,
                                                           int ldo, long long slab_stride, int M, int N, int K,
                                                           int k_per_wg, int rows) {
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, FEW>()];
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, FILL>()];
   const int wave = threadIdx.x >> 6;
   const int tile = blockIdx.x;
   const int m0 = blockIdx.z * 32 * MT;
   const int k_begin = blockIdx.y * k_per_wg, k_end = min(K, k_begin + k_per_wg);
-  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, FEW>(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
-  constexpr int NWV = sk_waves<MT, NX, FEW>();
+  float(*red)[MT][16][64] = skinny_tile<MT, TAIL, NX, FILL>(X, ldx, W, ldw, skinny_rows<EPI>(tile, rows, N), m0, M, k_begin, k_end, smem);
+  constexpr int NWV = sk_waves<MT, NX, FILL>();
   for (int a = wave; a < 4; a += NWV) skinny_finish<MT, EPI>(red, tile, rows, a, m0, M, N, bias, out, ldo, slab_stride);
 }
 
@@ -664,18 +672,23 @@ extern "C" int pico_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   // 33 to 64 tokens and at most one workgroup per compute unit (the O and down projections): four waves and
   // three slices each in flight instead of two and two (19.9 against 19.5 thousand tokens a second at batch
   // 64); with fewer tokens the same made the step slower (707 against 721 tokens a second at batch 1)
-  const bool few = nx == 8 && (long long)grid.x * grid.y * grid.z <= SK_COMPUTE_UNITS;
-#define LAUNCH4(MT, EPI, TAIL, NX, FEW) \
-  gemm_skinny_kernel<MT, EPI, TAIL, NX, FEW><<<grid, 64 * sk_waves<MT, NX, FEW>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
+  const long long workgroups = (long long)grid.x * grid.y * grid.z;
+  const bool few = nx == 8 && workgroups <= SK_COMPUTE_UNITS;
+  // up to 16 tokens and more than two workgroups per compute unit: shallower stages, three workgroups a unit
+  const bool many = workgroups > 2 * SK_COMPUTE_UNITS;
+#define LAUNCH4(MT, EPI, TAIL, NX, FILL) \
+  gemm_skinny_kernel<MT, EPI, TAIL, NX, FILL><<<grid, 64 * sk_waves<MT, NX, FILL>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, b0, out, ldo, slab_stride, M, N, K, k_per_wg, rows)
 #define LAUNCH(EPI)                                               \
   do {                                                            \
-    if (nx == 1) LAUNCH4(1, EPI, false, 1, false);                \
-    else if (nx == 2) LAUNCH4(1, EPI, false, 2, false);           \
-    else if (nx == 4) LAUNCH4(1, EPI, false, 4, false);           \
-    else if (nx == 8 && few) LAUNCH4(2, EPI, false, 8, true);     \
-    else if (nx == 8) LAUNCH4(2, EPI, false, 8, false);           \
-    else if (mt == 1) LAUNCH4(1, EPI, true, 0, false);            \
-    else LAUNCH4(2, EPI, true, 0, false);                         \
+    if (nx == 1 && many) LAUNCH4(1, EPI, false, 1, SK_MANY);      \
+    else if (nx == 1) LAUNCH4(1, EPI, false, 1, 0);               \
+    else if (nx == 2 && many) LAUNCH4(1, EPI, false, 2, SK_MANY); \
+    else if (nx == 2) LAUNCH4(1, EPI, false, 2, 0);               \
+    else if (nx == 4) LAUNCH4(1, EPI, false, 4, 0);               \
+    else if (nx == 8 && few) LAUNCH4(2, EPI, false, 8, SK_FEW);   \
+    else if (nx == 8) LAUNCH4(2, EPI, false, 8, 0);               \
+    else if (mt == 1) LAUNCH4(1, EPI, true, 0, 0);                \
+    else LAUNCH4(2, EPI, true, 0, 0);                             \
   } while (0)
   if (epilogue == EPI_BF16) LAUNCH(EPI_BF16);
   else if (epilogue == EPI_F32) LAUNCH(EPI_F32);
@@ -788,7 +801,7 @@ __device__ __forceinline__ void skinny_rope_body(
   }
   // What the epilogue needs besides the sums is read now, so that the stream hides the latency: thread
   // (wave a, lane (col, h)) finishes tile rows 8 a + 4 h + 0..3 of token block t's column `col`.
-  static_assert(sk_waves<MT, NX, true>() == 4, "one wave per 8 tile rows");
+  static_assert(sk_waves<MT, NX, SK_FEW>() == 4, "one wave per 8 tile rows");
   const int a = wave, t0 = 8 * a + 4 * h;
   const bool mine = rotated ? (a < 2 && t0 < pairs) : t0 < 2 * pairs;
   const int e0 = rotated ? pairs * tp + t0 : 2 * pairs * tp + t0;      // first of this thread's four head dimensions
@@ -822,10 +835,10 @@ __device__ __forceinline__ void skinny_rope_body(
   }
   float(*red)[MT][16][64];
   if constexpr (XS) {
-    skinny_stream_lds<1, 1, 4, sk_depth<1, true>(), true>(nullptr, 0, W, ldw, tr, m0, M, 0, K, smem, xs, before, between);
+    skinny_stream_lds<1, 1, 4, sk_depth<1, SK_FEW>(), true>(nullptr, 0, W, ldw, tr, m0, M, 0, K, smem, xs, before, between);
     red = reinterpret_cast<float(*)[MT][16][64]>(smem);
   } else {
-    red = skinny_tile<MT, TAIL, NX, true>(X, ldx, W, ldw, tr, m0, M, 0, K, smem);
+    red = skinny_tile<MT, TAIL, NX, SK_FEW>(X, ldx, W, ldw, tr, m0, M, 0, K, smem);
   }
   if (!mine) return;
 
@@ -877,7 +890,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_kernel(
     bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int M, int K,
     int nq, int nkv, int d, int pshift, int num_pages, int pairs) {
   // the grid of this projection is small (one workgroup per 32 of (nq + 2 nkv) d rows): four waves always
-  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, true>()];
+  __shared__ __attribute__((aligned(16))) char smem[sk_smem_bytes<MT, NX, SK_FEW>()];
   skinny_rope_body<MT, TAIL, NX>(X, ldx, W, ldw, bias, q_out, ldq, cos_sin, slots, k_cache, v_cache, M, K, nq, nkv, d, pshift,
                                  num_pages, pairs, smem);
 }
@@ -891,7 +904,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_rope_norm_kernel(
     int nq, int nkv, int d, int pshift, int num_pages, int pairs) {
   extern __shared__ __attribute__((aligned(16))) char dsmem[];
   __shared__ float scratch[16];
-  char* xs = dsmem + sk_xs_offset<sk_depth<1, true>()>();
+  char* xs = dsmem + sk_xs_offset<sk_depth<1, SK_FEW>()>();
   SkNormRow<VPT> row;
   skinny_rope_body<1, false, 1, true>(nullptr, 0, W, ldw, bias, q_out, ldq, cos_sin, slots, k_cache, v_cache, M, K, nq, nkv, d,
                                       pshift, num_pages, pairs, dsmem, xs, [&]() { row.load(in, K); },
@@ -922,7 +935,7 @@ extern "C" int pico_gemm_skinny_rope(const void* X, int ldx, const void* W, int 
   const bool tail = K % 64 != 0;
   const int nx = tail ? 0 : (mt == 2 ? 8 : M <= 8 ? 1 : M <= 16 ? 2 : 4);
 #define LAUNCH(MT, TAIL, NX) \
-  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, true>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
+  gemm_skinny_rope_kernel<MT, TAIL, NX><<<grid, 64 * sk_waves<MT, NX, SK_FEW>(), 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, \
       (bf16_t*)q_out, ldq, (const float2*)cos_sin, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, M, K, nq, nkv, d, pshift, num_pages, pairs)
   if (nx == 1) LAUNCH(1, false, 1);
   else if (nx == 2) LAUNCH(1, false, 2);
@@ -954,7 +967,7 @@ extern "C" int pico_gemm_skinny_rope_norm(const float* resid, const float* delta
   while ((1 << pshift) < P) pshift++;
   int pairs = skinny_tile_height((long long)(nq + 2 * nkv) * (d / 2), 2, 1, 8, nullptr, 1, 4);
   if (pairs == 12) pairs = 16;
-  const int smem = sk_xs_smem_bytes(sk_depth<1, true>(), K);
+  const int smem = sk_xs_smem_bytes(sk_depth<1, SK_FEW>(), K);
   const SkNormIn in = {resid, delta, slabs, slab_stride, norm_w, eps, resid_out};
 #define LAUNCHR(VPT)                                                                                              \
   do {                                                                                                            \
