@@ -68,6 +68,11 @@ class ModelRunner:
             logits = self._step_graph(seqs, device_tokens)
         else:
             ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size)
+            if decode_only:
+                # the kernel choices of a recorded decode step (how the context is split over workgroups) hold for
+                # any context; a decode step that is not replayed makes the same ones, so that a request gets the
+                # same tokens with and without graphs
+                ctx.max_context = self.max_seq_len
             if device_tokens is not None:
                 ctx.token_ids[:len(seqs)].copy_(device_tokens[:len(seqs)])
             logits = self.model.forward(ctx, self.storage)

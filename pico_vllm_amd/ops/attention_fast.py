@@ -28,7 +28,12 @@ class FastAttention:
         """Enough workgroups to fill the chip (256 CUs, two workgroups each), no split shorter
         than one 64-key tile (or, beyond 64 splits, than two), at most 256 splits (what the merging kernel takes):
         a single request with 32,768 tokens behind it is read by 512 workgroups, not by 128."""
-        by_fill = max(1, 512 // max(1, num_seqs * self.nkv))
+        # the number of sequences counts as the power of two that a recorded step of them is padded to, so that
+        # a step splits its contexts alike whether it is replayed from a graph or not
+        padded = 1
+        while padded < num_seqs:
+            padded *= 2
+        by_fill = max(1, 512 // max(1, padded * self.nkv))
         by_len = max(1, -(-max_context // 64))
         if by_len > 64:
             by_len = max(64, -(-max_context // 128))

@@ -107,8 +107,8 @@ def test_decode_steps_replayed_from_a_graph_give_the_same_tokens(dtype):
     graph_llm = llm("A", dtype, num_gpu_blocks=128, use_cuda_graph=True, max_batch_size=4)
     graphed = graph_llm.generate(prompts, sp)
     assert graph_llm.engine.runner._graphs, "no decode step went through a graph"
-    if dtype == "float32":
-        assert [o.token_ids for o in graphed] == [o.token_ids for o in eager]
+    # the same kernels with the same choices on the same inputs: the same tokens, in bfloat16 too
+    assert [o.token_ids for o in graphed] == [o.token_ids for o in eager]
     check_greedy("A", dtype, prompts, graphed)
     # a second batch on the same engine replays the graphs captured by the first
     more = graph_llm.generate(prompts[:2], sp)
