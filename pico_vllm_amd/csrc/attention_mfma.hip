@@ -675,7 +675,11 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   // addresses from what init() has prepared.  The last tiles and other pages go the long way.  Two loops
   // and no branch inside them: a branch between the loads would force a wait for the ones before it.
   const uint32_t page_bytes = ((uint32_t)nkv << pshift) * (2 * D);
-  const int n_full = (pshift <= 4 && page_bytes < (1u << 24) && num_pages < (1 << 24)) ? kv_end / PF_TK : 0;
+  // ... and only where a thread's chunks of K are a whole number of pages apart (PfFetch::init): head sizes
+  // whose chunks per key do not divide the workgroup's threads, or pages larger than that distance, go the long way
+  constexpr int K_APART = PfFetch<KT>::PF_NT / PfFetch<KT>::KCH;            // keys between a thread's chunks
+  const bool apart_ok = PfFetch<KT>::PF_NT % PfFetch<KT>::KCH == 0 && ((K_APART >> pshift) << pshift) == K_APART;
+  const int n_full = (apart_ok && pshift <= 4 && page_bytes < (1u << 24) && num_pages < (1 << 24)) ? kv_end / PF_TK : 0;
   regs.init(g, nkv, pshift);
   regs.load_pages(bt, pshift, num_pages, 0, kv_end);
   regs.fetch(k_cache, v_cache, g, nkv, pshift, 0, kv_end);

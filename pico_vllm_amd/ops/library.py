@@ -139,7 +139,7 @@ def attention_library(head_dim: int) -> ctypes.CDLL:
     return load_library(f"pico_attn_d{head_dim}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={head_dim}",))
 
 
-def build_all(head_dims: Iterable[int] = (16, 32, 48, 64, 80, 96, 128, 256), force: bool = True) -> List[str]:
+def build_all(head_dims: Iterable[int] = (16, 32, 48, 64, 80, 96, 128, 160, 192, 224, 256), force: bool = True) -> List[str]:
     """Compile everything (used by the build check); returns the paths."""
     out = [build_library("pico_core", CORE_SOURCES, force=force)]
     if os.path.isfile(os.path.join(CSRC, "attention_mfma.hip")):

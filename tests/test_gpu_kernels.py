@@ -358,13 +358,28 @@ def test_fast_prefill_other_sizes_and_long_portions(K, nq, nkv, d, Pg):
 
 
 @pytest.mark.parametrize("teams", [1, 2, 3, 4])
-@pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64), (4, 1, 96, 32)])
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64), (4, 1, 96, 32),
+                                        (4, 1, 96, 16), (4, 1, 96, 8), (8, 2, 256, 16), (2, 1, 160, 8)])
 def test_fast_prefill_with_every_shape_of_workgroup(K, nq, nkv, d, Pg, teams):
     # the shape of the workgroups (1 to 3 teams on a 64-query tile, 4: two query blocks a wave, 128-query tiles)
     # is a hint: every value gives the same attention; lengths around the 64- and 128-query tiles and the
     # 64-, 128- and 192-key tiles of one to three teams; pages of 8 and 16 keys take the short way in whole tiles
     out, want = _fast_case([63, 1, 65, 130, 2, 200, 193, 127, 257], [0, 127, 1, 62, 191, 129, 383, 1, 64], nq, nkv, d, Pg, seed=5,
                            teams=teams)
+    close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("Pg", [8, 16, 32])
+@pytest.mark.parametrize("d", [32, 64, 96, 128, 160, 192, 224, 256])
+def test_fast_prefill_whole_key_tiles_at_every_head_size_and_page_size(K, d, Pg):
+    # contexts of three and more whole key tiles: where a thread's chunks of K are a whole number of pages
+    # apart the kernel prepares its addresses once per tile, elsewhere it must not; queries are scaled up so
+    # that a few keys carry each row's weight and a wrong key or row part shows
+    def boost(qs, ks, vs):
+        for q in qs:
+            q *= 3.0
+    out, want = _fast_case([200, 70, 3], [0, 330, 400], 2, 1, d, Pg, seed=17 + d + Pg, boost=boost)
+    assert float(want.abs().mean()) > 0.3
     close(out, want, torch.bfloat16)
 
 

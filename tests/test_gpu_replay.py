@@ -260,6 +260,19 @@ def test_configurations_drawn_at_random_whole_and_mixed(name, dtype):
     compare(name, dtype, reqs, got, "mixed")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompts_of_several_whole_key_tiles_at_head_size_96(dtype):
+    # contexts beyond three whole 64-key tiles at a head size whose rows no workgroup's threads divide evenly:
+    # whole, in portions (large ones after a long prefix) and with the tail decoded token by token
+    reqs = make_requests("E", [260, 213], seed=11)
+    got, _ = replay("E", dtype, whole(reqs))
+    compare("E", dtype, reqs, got, "whole")
+    got, _ = replay("E", dtype, portions(reqs, sizes=(70, 2, 130, 3, 40)))
+    compare("E", dtype, reqs, got, "portions")
+    got, _ = replay("E", dtype, tail_one_by_one(reqs, tail=8))
+    compare("E", dtype, reqs, got, "tail")
+
+
 def test_float32_does_not_depend_on_the_cut_at_all():
     # every reduction of the 32-bit path has a fixed order per output element: bitwise equal
     reqs = make_requests("B", [77, 40], seed=5)

@@ -25,8 +25,14 @@ TINY_D = {   # sizes that no vector access divides: a width of 100, an odd inter
     "num_key_value_heads": 2, "head_dim": 16, "intermediate_size": 123, "rms_norm_eps": 1e-6,
     "rope_theta": 10000.0, "tie_word_embeddings": False, "max_position_embeddings": 1024, "hidden_act": "silu",
 }
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+TINY_E = {   # head size 96 (three chunks of 32; its 12 chunks of 16 bytes a key divide no workgroup), groups of 3
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 333, "hidden_size": 168, "num_hidden_layers": 2, "num_attention_heads": 6,
+    "num_key_value_heads": 2, "head_dim": 96, "intermediate_size": 232, "rms_norm_eps": 3e-6,
+    "rope_theta": 100000.0, "tie_word_embeddings": True, "max_position_embeddings": 2048, "hidden_act": "silu",
+}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
 
 
 def drawn(seed: int):
