@@ -214,3 +214,63 @@ extern "C" int pico_argmax(const float* logits, int ld, int R, int V, float* par
   PICO_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// The same two launches with the chunk maxima in memory of the library's own (no_alloc.h).
+// ---------------------------------------------------------------------------
+#include "no_alloc.h"
+
+#include <mutex>
+
+#define NOALLOC_ENTRIES (PICO_NOALLOC_MAX_ROWS * ARGMAX_CHUNKS)
+#define NOALLOC_MAX_DEVICES 64
+
+// [values: NOALLOC_ENTRIES floats][indices: NOALLOC_ENTRIES ints].  In host code this name is only a handle
+// for hipGetSymbolAddress; the address that kernels and copies take is g_scratch_ptr[device].
+static __device__ __align__(256) unsigned char scratch[NOALLOC_ENTRIES * (sizeof(float) + sizeof(int))];
+
+static void* g_scratch_ptr[NOALLOC_MAX_DEVICES];     // per device: where that GPU's copy of the array lies
+static std::mutex g_scratch_mutex;
+
+// The address of the current device's copy, looked up once per device with that device current.
+static int noalloc_scratch(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  PICO_REQUIRE(e == hipSuccess, "pico_noalloc: hipGetDevice failed: %s", hipGetErrorString(e));
+  PICO_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, "pico_noalloc: device %d is beyond the %d this library keeps", dev,
+               NOALLOC_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    PICO_REQUIRE(e == hipSuccess && p != nullptr, "pico_noalloc: hipGetSymbolAddress failed on device %d: %s", dev,
+                 hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int pico_noalloc_max_rows() { return PICO_NOALLOC_MAX_ROWS; }
+
+extern "C" int pico_noalloc_init() {
+  void* p = nullptr;
+  return noalloc_scratch(&p);
+}
+
+extern "C" int pico_argmax_noalloc(const float* logits, int ld, int R, int V, int* out, hipStream_t stream) {
+  PICO_REQUIRE(R >= 0 && V > 0 && ld >= V, "pico_argmax_noalloc: bad sizes R=%d V=%d ld=%d", R, V, ld);
+  PICO_REQUIRE(R <= PICO_NOALLOC_MAX_ROWS, "pico_argmax_noalloc: %d rows, the library's own memory holds %d; "
+               "use pico_argmax with a workspace", R, PICO_NOALLOC_MAX_ROWS);
+  PICO_REQUIRE(logits != nullptr && out != nullptr, "pico_argmax_noalloc: null pointer");
+  if (R == 0) return 0;
+  void* base = nullptr;
+  if (noalloc_scratch(&base) != 0) return -1;
+  float* part_val = reinterpret_cast<float*>(base);
+  int* part_idx = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(base) + NOALLOC_ENTRIES * sizeof(float));
+  // the first launch writes entries [0, R * ARGMAX_CHUNKS), the second reads exactly those: nothing to clear
+  argmax_part_kernel<<<dim3(R, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, ld, V, part_val, part_idx);
+  argmax_final_kernel<<<R, 64, 0, stream>>>(part_val, part_idx, out);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
