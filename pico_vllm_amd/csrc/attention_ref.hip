@@ -51,8 +51,9 @@ __global__ __launch_bounds__(64) void paged_attention_ref_kernel(
     __syncthreads();
     ps[lane] = p;
     __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 4; i++) acc[i] *= alpha;
+    // the block's part of P V is summed on its own and then joins the running sum: two short sums instead of one
+    // over the whole context
+    float blk[4] = {0.f, 0.f, 0.f, 0.f};
     const int kend = min(64, pos - c0 + 1);
     for (int kk = max(0, lo - c0); kk < kend; kk++) {
       const int kpos = c0 + kk;
@@ -63,9 +64,11 @@ __global__ __launch_bounds__(64) void paged_attention_ref_kernel(
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int dim = lane + 64 * i;
-        if (dim < d) acc[i] = fmaf(pk, load_f32(vp + (size_t)dim * P), acc[i]);
+        if (dim < d) blk[i] = fmaf(pk, load_f32(vp + (size_t)dim * P), blk[i]);
       }
     }
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = fmaf(acc[i], alpha, blk[i]);
     m = m_new;
   }
   T* o = out + ((size_t)t * nq + h) * d;

@@ -1,6 +1,11 @@
 // True float32 matrix product C = A W^T (+ bias): plain FMA, no matrix-core reduced
-// precision.  Every output element is accumulated over k = 0..K-1 in that order by one
-// thread, so a row's result does not depend on how many other rows the call has.
+// precision.  Every output element is accumulated by one thread in an order that depends
+// on K alone, so a row's result does not depend on how many other rows the call has.
+// The sum is a tree of radix 16 over k: 16 products are added up one after the other, 16
+// such sums likewise, and so on for four levels (the last takes what is left), so the
+// rounding error of a sum grows like the square root of the number of levels times 16
+// rather than like the square root of K: with one running sum over K = 8,960 terms the
+// error of a product was twenty times that of storing its result in float32.
 // It is the GEMM of the 32-bit engine (the reference uses the library through nn.Linear,
 // pico_vllm/model.py:200,225,316,318,445); speed is secondary.
 #include "common.h"
@@ -19,8 +24,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const TA* __restrict__ A,
   __shared__ float Ws[BK][BN + 1];
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  float acc[4][4] = {};
-  for (int k0 = 0; k0 < K; k0 += BK) {
+  // lvl[0]: the running sum of the current 16 products; lvl[i]: of up to 16 finished sums of level i - 1
+  // (level 3 of all of them)
+  float lvl[4][4][4] = {};
+  int tile = 0;
+  for (int k0 = 0; k0 < K; k0 += BK, tile++) {
     // 64 x 16 elements per tile, 256 threads: 4 each
     for (int i = threadIdx.x; i < BM * BK; i += 256) {
       const int r = i / BK, c = i % BK;
@@ -39,10 +47,29 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const TA* __restrict__ A,
 #pragma unroll
       for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; j++) lvl[0][i][j] = fmaf(a[i], b[j], lvl[0][i][j]);
+    }
+    // carry: after every tile level 0 goes up; after every 16th tile level 1 does, after every 256th level 2
+    // (the same for all threads: no divergence)
+#pragma unroll
+    for (int L = 0; L < 3; L++) {
+      if (((tile + 1) & ((1 << (4 * L)) - 1)) != 0) break;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          lvl[L + 1][i][j] += lvl[L][i][j];
+          lvl[L][i][j] = 0.f;
+        }
     }
     __syncthreads();
   }
+  // what the lower levels still hold goes up in the same fixed order
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = ((lvl[0][i][j] + lvl[1][i][j]) + lvl[2][i][j]) + lvl[3][i][j];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int m = m0 + ty * 4 + i;

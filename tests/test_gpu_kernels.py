@@ -98,6 +98,24 @@ def test_gemm_f32(K, M, N, K_):
     assert torch.allclose(out3.cpu().double(), ab.double() @ w.double().T, rtol=1e-5, atol=1e-4)
 
 
+@pytest.mark.parametrize("K_", [64, 1000, 1536, 3584, 5120, 8960, 18944, 27648])
+def test_gemm_f32_rounding_does_not_grow_with_the_inner_size(K, K_):
+    # The sums are trees of radix 16 with L = ceil(log16 K) levels (at most 4).  An addition rounds its partial sum
+    # by up to eps = 2^-24 of it, 0.58 eps rms; the partial sums of a group of 16 have on average 8.5 / 16 of the
+    # group's mean square, and the groups' mean squares add up to the result's (random signs): every level adds
+    # (0.58 eps)^2 * 8.5 to the relative mean square error, so rms error <= 0.58 sqrt(8.5 L) eps = 1.69 sqrt(L) eps
+    # of the result's rms at ANY inner size.  One running sum over K terms would give 0.2 sqrt(K) eps: 19 eps at 8,960.
+    g = torch.Generator().manual_seed(K_)
+    a, w = torch.randn(8, K_, generator=g), torch.randn(96, K_, generator=g)
+    want = a.double() @ w.double().T
+    err = K.gemm_f32(a.to(DEV), w.to(DEV)).cpu().double() - want
+    eps, levels = 2.0 ** -24, min(4, math.ceil(math.log(K_, 16)))
+    rms = float(err.pow(2).mean().sqrt() / want.pow(2).mean().sqrt())
+    print(f"[gemm_f32] K={K_}: rms error {rms / eps:.2f} eps, bound {1.69 * math.sqrt(levels):.2f} eps")
+    assert rms <= 1.69 * math.sqrt(levels) * eps
+    assert float(err.abs().max() / want.pow(2).mean().sqrt()) <= 5 * 1.69 * math.sqrt(levels) * eps     # 768 outputs: five sigma
+
+
 @pytest.mark.parametrize("M,N,K_", [(1, 301, 136), (3, 256, 64), (8, 384, 192), (33, 130, 172), (64, 1000, 1536),
                                    (100, 77, 40)])
 @pytest.mark.parametrize("out_dtype", DTYPES)
@@ -502,7 +520,11 @@ def test_fast_kernels_refuse_what_they_cannot_do(K):
                                    (50, 10270, 192), (40, 10400, 64), (64, 10240, 320),
                                    # more than 64 tokens of a small matrix: blocks of 64 tokens, the last one partial
                                    # (with 1 to 32 and with more than 32 tokens)
-                                   (65, 301, 136), (100, 1536, 1536), (130, 2048, 1536), (256, 1000, 264), (200, 90, 8960)])
+                                   (65, 301, 136), (100, 1536, 1536), (130, 2048, 1536), (256, 1000, 264), (200, 90, 8960),
+                                   # the four projections at the 7B sizes (hidden 3584, 28 + 2 * 4 heads of 128, 18944) ...
+                                   (1, 4608, 3584), (64, 3584, 3584), (40, 37888, 3584), (8, 3584, 18944),
+                                   # ... and at the 32B sizes (hidden 5120, 40 + 2 * 8 heads of 128, 27648)
+                                   (3, 7168, 5120), (1, 5120, 5120), (64, 55296, 5120), (17, 5120, 27648)])
 def test_gemm_skinny_epilogues(K, M, N, K_):
     g = torch.Generator().manual_seed(M * N)
     a = torch.randn(M, K_, generator=g).bfloat16()
@@ -585,7 +607,8 @@ def test_gemm_skinny_with_rotation_and_cache_store(K, M, nq, nkv, d, H, Pg, bias
 
 
 @pytest.mark.parametrize("N,K_,slabs", [(2048, 1536, 5), (17920, 1536, 3), (1000, 320, 1), (90, 64, 0), (640, 2048, 8),
-                                        (2 * 323, 512, -1), (1000, 3584, 6), (512, 4096, 8), (384, 2112, 0)])
+                                        (2 * 323, 512, -1), (1000, 3584, 6), (512, 4096, 8), (384, 2112, 0),
+                                        (4608, 3584, 7), (37888, 3584, 5)])
 def test_gemm_skinny_with_the_norm_in_front(K, N, K_, slabs):
     # norm(resid + partial sums) W^T of one row in one kernel against the norm kernel followed by the product;
     # slabs: 0 = nothing to add, -1 = one sum [1, K], else a stack [slabs, 1, K]
@@ -648,6 +671,15 @@ def test_gemm_skinny_with_the_norm_in_front_and_rotation_and_cache_store(K, nq, 
         scale = float(a.abs().max())
         assert float((a - c).abs().max()) <= 2e-2 * scale and float((a - c).abs().mean()) <= 1e-3 * scale
     assert float((k0 == 7.0).float().mean()) > 0.5 and torch.equal(k0 == 7.0, k1 == 7.0)     # only the token's slot was written
+
+
+def test_the_norm_in_front_is_refused_beyond_its_widest_row(K):
+    # a width of 5,120 (the 32B size) does not fit the kernel's row buffer: the caller is told so and runs the norm itself
+    w = torch.zeros(256, 5120, dtype=torch.bfloat16, device=DEV)
+    resid = torch.zeros(1, 5120, device=DEV)
+    assert not K.skinny_norm_ok(resid, None, w)
+    with pytest.raises(K.KernelError):
+        K.gemm_skinny_norm(resid, None, torch.ones(5120, device=DEV), 1e-6, w)
 
 
 def test_gemm_skinny_refuses_misaligned_operands(K):

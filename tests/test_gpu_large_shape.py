@@ -1,11 +1,17 @@
-"""The kernels at the sizes of a real model: two layers of the Qwen2.5-1.5B shape with random weights.
+"""The engine at the layer sizes of real models, with random weights.
 
 The tiny configurations of the other tests never reach the paths that only large sizes take (two key
 teams over a 2,048-token triangle, the 8960-wide contraction cut into seven ranges, a vocabulary of
-151,936, the library's matrix products for many rows).  The plain implementation on the CPU is too
-slow here, so the yardstick is the engine's own true 32-bit path, which the other tests pin to the
-plain implementation; the bfloat16 engine must follow it within bfloat16 rounding, whole, in
-portions, and token by token.
+151,936, the library's matrix products for many rows, groups of 5 and 7 query heads of size 128, a width
+beyond what the fused norm takes).
+
+Against the plain implementation in float64: two layers of the Qwen2.5-1.5B sizes and one layer each of
+the 7B and 32B sizes with a vocabulary cut to a few thousand, a prompt of 200 tokens whole, in portions
+of changing size and with its tail token by token, in 32-bit and in bfloat16, with the bounds of the
+replay tests (the reference's own bar is equality of generations with an outside model at the real
+size, pico_vllm/tests/test_engine.py:59-93).
+With the whole vocabulary of 151,936 and a prompt beyond one 2,048-token portion the plain implementation
+is too slow; there the yardstick is the engine's own 32-bit path, which the tests above pin.
 """
 import random
 import tempfile
@@ -133,4 +139,29 @@ def test_decoding_40_requests_together_gives_what_each_gives_alone(folder):
         print(f"[large] 40 together, decode step {k}: rms difference {rms:.2e} of the spread, argmax equal in {same}/{R} rows")
         assert rms < 5e-3 and same >= R - 2, (k, rms, same)
     del rep
+    torch.cuda.empty_cache()
+
+
+# ---- against the plain implementation ----------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["L1.5B", "L7B", "L32B"])
+def test_real_layer_sizes_against_the_plain_implementation(name, dtype):
+    import test_gpu_replay as R
+    reqs = R.make_requests(name, [200], seed=21)
+    print(f"[real sizes] {name} {dtype}", flush=True)
+    for label, trace in (("whole", R.whole(reqs)), ("portions", R.portions(reqs)), ("tail", R.tail_one_by_one(reqs))):
+        got, _ = R.replay(name, dtype, trace)
+        R.compare(name, dtype, reqs, got, f"real {label}")
+    torch.cuda.empty_cache()
+
+
+def test_real_layer_sizes_mixed_in_a_small_pool():
+    # seven requests of the 7B sizes, three live at a time, portions of some beside single tokens of others, pages used again
+    import test_gpu_replay as R
+    reqs = R.make_requests("L7B", [90, 70, 120, 64, 100, 80, 75], seed=22)
+    trace = R.mixed(reqs, seed=5, max_live=3)
+    for dtype in ("float32", "bfloat16"):
+        got, pool = R.replay("L7B", dtype, trace)
+        assert pool.reuse_count > 0
+        R.compare("L7B", dtype, reqs, got, "real mixed")
     torch.cuda.empty_cache()

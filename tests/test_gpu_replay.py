@@ -24,6 +24,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # is the rounding noise of this model at this length.  The engine must stay within a small
 # multiple of it; a fault larger than the rounding noise fails, whatever the model's sensitivity.
 F32_REL_MAX, F32_REL_MEAN = 2e-5, 4e-6
+# The yardstick that adapts to the model, as for bfloat16: the plain implementation itself in float32 (torch on the
+# CPU, its own summation orders) against the same in float64 shows what float32 arithmetic costs THIS request of THIS
+# model.  The engine's sums are trees of radix 16 (2 half-units in the last place rms for any K, against 4 to 5 for
+# the CPU library's), so it stays below the plain float32 run's own error; a fault does not.
+F32_VS_PLAIN32_RMS, F32_VS_PLAIN32_MAX = 1.25, 2.0
 BF16_RMS_FACTOR, BF16_MAX_FACTOR = 1.5, 2.0
 # The engine stores bfloat16 where the rounded plain computation rounds (activations between parts,
 # probabilities before P.V), so it follows THAT computation at least as closely as the exact one:
@@ -175,6 +180,19 @@ def bf16_noise(name, tokens):
     return _noise_cache[key]
 
 
+_noise32_cache = {}
+
+
+def f32_noise(name, tokens):
+    """(rms, max) of the logit error of the plain implementation run in float32 against float64."""
+    key = (name, tuple(tokens))
+    if key not in _noise32_cache:
+        ref = plain_logits(name, tokens)
+        err = np.abs(_plain_cache[name].logits(tokens).numpy().astype(np.float64) - ref)
+        _noise32_cache[key] = (float(np.sqrt((err ** 2).mean())), float(err.max()))
+    return _noise32_cache[key]
+
+
 def compare(name, dtype, reqs, got, label):
     worst = 0.0
     for rid, toks in reqs.items():
@@ -189,6 +207,13 @@ def compare(name, dtype, reqs, got, label):
             assert rel.max() <= F32_REL_MAX, (f"{label} {name} {dtype}: request {rid} first wrong position "
                                               f"{int(np.argmax(rel > F32_REL_MAX))}, worst {rel.max():.3e} at {int(rel.argmax())}")
             assert err.mean() / spread <= F32_REL_MEAN, f"{label} {name}: mean error {err.mean() / spread:.3e}"
+            n_rms, n_max = f32_noise(name, toks)
+            rms = float(np.sqrt((err.astype(np.float64) ** 2).mean()))
+            print(f"[replay] {label} {name} f32 {rid}: rms {rms / n_rms:.2f}x max {err.max() / n_max:.2f}x of the plain float32 "
+                  f"run's own error (max {n_max / spread:.2e} of the spread)")
+            assert rms <= F32_VS_PLAIN32_RMS * n_rms and err.max() <= F32_VS_PLAIN32_MAX * n_max, \
+                (f"{label} {name} float32: request {rid}: {rms / n_rms:.2f}x (rms) {err.max() / n_max:.2f}x (max) the error of "
+                 f"the plain implementation in float32")
         else:
             noise_rms, noise_max, rounded = bf16_noise(name, toks)
             rms = float(np.sqrt((err ** 2).mean()))
@@ -271,6 +296,23 @@ def test_prompts_of_several_whole_key_tiles_at_head_size_96(dtype):
     compare("E", dtype, reqs, got, "portions")
     got, _ = replay("E", dtype, tail_one_by_one(reqs, tail=8))
     compare("E", dtype, reqs, got, "tail")
+
+
+def test_fifty_more_drawn_configurations_in_every_way_of_cutting():
+    # a sweep over sizes nobody looked at, in both precisions, whole, with the tail token by token and mixed in a
+    # small pool; it stops at the first configuration that fails and names it
+    import tiny_configs as TC
+    for seed in range(10, 60):
+        name = f"S{seed}"
+        TC.CONFIGS[name], TC.PAGE_SIZE[name] = TC.drawn(seed)
+        for dtype in ("bfloat16", "float32"):
+            reqs = make_requests(name, [40, 77, 33, 60], seed=seed)
+            for label, trace in (("whole", whole(reqs)), ("tail", tail_one_by_one(reqs)),
+                                 ("mixed", mixed(reqs, seed=seed, max_live=3))):
+                got, _ = replay(name, dtype, trace)
+                compare(name, dtype, reqs, got, f"sweep {label}")
+        for key in [k for k in _plain_cache if k == name or (isinstance(k, tuple) and k[0] == name)]:
+            del _plain_cache[key]           # the weights of fifty models need not stay in memory
 
 
 def test_float32_does_not_depend_on_the_cut_at_all():

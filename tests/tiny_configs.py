@@ -63,6 +63,32 @@ def drawn(seed: int):
 for _seed in range(10):
     CONFIGS[f"R{_seed}"], PAGE_SIZE[f"R{_seed}"] = drawn(_seed)
 
+
+
+def _real(hidden, heads, kv_heads, inter, layers, vocab, tied):
+    return {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": vocab, "hidden_size": hidden,
+            "num_hidden_layers": layers, "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+            "intermediate_size": inter, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "tie_word_embeddings": tied,
+            "max_position_embeddings": 32768, "hidden_act": "silu"}
+
+
+# Layers of the sizes of real models (the vocabulary cut down so that the plain implementation stays quick): two
+# layers of Qwen2.5-1.5B, one each of 7B (groups of 7 heads) and 32B (groups of 5, a width beyond 4,096)
+REAL = {"L1.5B": _real(1536, 12, 2, 8960, 2, 20011, True), "L7B": _real(3584, 28, 4, 18944, 1, 4099, False),
+        "L32B": _real(5120, 40, 8, 27648, 1, 3001, False)}
+for _name, _cfg in REAL.items():
+    CONFIGS[_name], PAGE_SIZE[_name] = _cfg, 16
+
+
+def balanced(config) -> dict:
+    """Standard deviations for the real sizes: every part changes the residual stream by about as much as it
+    holds (rows of unit length into unit-variance activations), and attention scores have a spread of about 3."""
+    H, I = config["hidden_size"], config["intermediate_size"]
+    return {"q_proj.weight": (3.0 / H) ** 0.5, "k_proj.weight": (3.0 / H) ** 0.5, "v_proj.weight": H ** -0.5,
+            "o_proj.weight": H ** -0.5, "gate_proj": 1.5 * H ** -0.5, "up_proj": H ** -0.5, "down_proj": 2.0 * I ** -0.5,
+            "_proj.bias": 0.2, "embed_tokens": 1.0, "lm_head": H ** -0.5}
+
+
 _made = {}
 
 
@@ -86,6 +112,7 @@ def model_dir(name: str, seed: int = 0, strong: bool = True) -> str:
     key = (name, seed, strong)
     if key not in _made:
         d = tempfile.mkdtemp(prefix=f"pico_tiny_{name}_")
-        write_random_model(d, CONFIGS[name], seed, globals()['strong'](CONFIGS[name]) if strong else None)
+        stds = (balanced if name in REAL else globals()['strong'])(CONFIGS[name]) if strong else None
+        write_random_model(d, CONFIGS[name], seed, stds)
         _made[key] = d
     return _made[key]
