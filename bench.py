@@ -62,7 +62,7 @@ def make_engine(model_dir, dtype, batch, layers_model=None):
     args = EngineArgs(model=model_dir, dtype=dtype, block_size=block,
                       num_gpu_blocks=batch * (CONTEXT // block + 1) + 8, max_seq_len=CONTEXT + 16,
                       max_num_seqs=batch, max_num_batched_tokens=max(PREFILL_TOKENS, batch),
-                      use_cuda_graph=True, max_batch_size=64)
+                      use_cuda_graph=True, max_batch_size=64, tune_library_gemm=True)
     return LLMEngine(args, model=layers_model)
 
 
@@ -146,7 +146,7 @@ def serve_point(model_dir, dtype, requests, max_new):
     pages = sum(-(-(n + max_new) // block) for n in lens) + 8
     eng = LLMEngine(EngineArgs(model=model_dir, dtype=dtype, block_size=block, num_gpu_blocks=pages, max_seq_len=CONTEXT,
                                max_num_seqs=requests, max_num_batched_tokens=PREFILL_TOKENS, use_cuda_graph=True,
-                               max_batch_size=64))
+                               max_batch_size=64, tune_library_gemm=True))
     V = CONFIG["vocab_size"]
     # a short run first: kernels built and tuned, graphs captured for the batch sizes of the run's tail
     for n in (PREFILL_TOKENS, 300):

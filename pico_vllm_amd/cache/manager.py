@@ -80,6 +80,9 @@ class CacheManager:
                 raise ValueError(f"layer {layer}: unknown cache kind {spec.kind!r}")
         self.slots = StateSlots(max_seqs)
         self.requests: Dict[Hashable, RequestCache] = {}
+        # slots handed out since the storage last cleared any: a request's state starts from zero, whoever held
+        # the slot before (``take_fresh_slots``; the step function clears them before the model runs)
+        self._fresh_slots: List[int] = []
 
     # ---- requests -------------------------------------------------------
     def add_request(self, req: Hashable) -> bool:
@@ -91,7 +94,15 @@ class CacheManager:
             return False
         self.requests[req] = RequestCache(slot, [[] for _ in self.groups], 0, [0] * len(self.groups),
                                           [np.full(16, -1, dtype=np.int32) for _ in self.groups])
+        if self.state_layers:
+            self._fresh_slots.append(slot)
         return True
+
+    def take_fresh_slots(self) -> List[int]:
+        """The state slots given to new requests since the last call; whoever owns the state tensors sets them
+        to zero before the next step reads them, so that no mixer has to find out by itself that a request is new."""
+        out, self._fresh_slots = self._fresh_slots, []
+        return out
 
     def free_request(self, req: Hashable) -> None:
         rc = self.requests.pop(req)
@@ -149,6 +160,10 @@ class CacheManager:
         engine.py:265)."""
         if num_tokens % self.page_size:
             raise ValueError("only whole pages can be shared")
+        if self.state_layers:
+            # a fixed-size state exists only as of the source's last token, not as of the end of the prefix
+            raise PagePoolError("a model with per-request state cannot share a prefix: the state at the end of the "
+                                "prefix is not kept")
         s, d = self.requests[src], self.requests[dst]
         if d.num_computed or any(d.tables):
             raise PagePoolError("the receiving request must be empty")

@@ -29,7 +29,7 @@ class PagedKVLayer:
 
 @dataclass
 class StateLayer:
-    state: torch.Tensor        # [slots, *state_shape]
+    state: torch.Tensor        # [slots + 1, *state_shape]; the last slot belongs to padding rows
     group: int = -1
 
 
@@ -48,13 +48,33 @@ class CacheStorage:
                 self._layers[layer] = PagedKVLayer(k, v, gi, P)
             elif spec.kind == "state":
                 sdt = getattr(torch, spec.state_dtype)
+                # one slot more than requests can hold: the padding rows of a recorded decode batch write there
                 self._layers[layer] = StateLayer(
-                    torch.zeros(manager.slots.num_slots, *spec.state_shape, dtype=sdt, device=device))
+                    torch.zeros(manager.slots.num_slots + 1, *spec.state_shape, dtype=sdt, device=device))
             else:
                 self._layers[layer] = None
 
     def layer(self, index: int):
         return self._layers.get(index)
+
+    def save_state(self):
+        """Copies of every per-request state tensor (for ``restore_state``)."""
+        return {i: l.state.clone() for i, l in self._layers.items() if isinstance(l, StateLayer)}
+
+    def restore_state(self, saved) -> None:
+        for i, t in saved.items():
+            self._layers[i].state.copy_(t)
+
+    def reset_state(self, slots) -> None:
+        """Zero the state of these slots in every layer that keeps one (a new request took them)."""
+        if not slots:
+            return
+        idx = None
+        for l in self._layers.values():
+            if isinstance(l, StateLayer):
+                if idx is None:
+                    idx = torch.tensor(sorted(set(slots)), dtype=torch.long, device=l.state.device)
+                l.state.index_fill_(0, idx, 0)
 
     def num_bytes(self) -> int:
         total = 0

@@ -28,6 +28,7 @@ class EngineArgs:
     max_batch_size: int = 8              # largest decode batch that has a graph
     manual_seed: int = 42
     pipeline_decode: bool = True         # keep one decode step in flight while the host prepares the next
+    tune_library_gemm: bool = False      # let the library time its solutions for whole prompt portions (stalls the first such step)
     device: str = "cuda:0"
 
     def validate(self) -> None:

@@ -43,6 +43,8 @@ def qwen2_spec(cfg: Qwen2Config) -> ModelSpec:
         head_name=None if cfg.tie_word_embeddings else "lm_head.weight",
         eos_token_id=cfg.eos_token_id,
         max_position=cfg.max_position_embeddings,
+        # a tied model's file may still hold the output matrix; the reference never reads it (weights.py:67-68)
+        ignored_tensors=("lm_head.weight",) if cfg.tie_word_embeddings else (),
     )
 
 

@@ -6,29 +6,29 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------
-// embedding: out[t, :] = table[ids[t], :] as float32.  An id outside [0, V) gives a
+// embedding: out[t, :] = table[ids[t], :] * scale as float32.  An id outside [0, V) gives a
 // row of zeros (the host checks ids before a step; this only keeps the kernel in bounds).
 // Reference: nn.Embedding lookup, pico_vllm/model.py:427.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embedding_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                 float* __restrict__ out, int H, int V) {
+                                 float* __restrict__ out, int H, int V, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   const bool ok = id >= 0 && id < V;
   const T* row = table + (size_t)(ok ? id : 0) * H;
   float* o = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ok ? load_f32(row + i) : 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ok ? load_f32(row + i) * scale : 0.f;
 }
 
 extern "C" int pico_embedding(const void* table, int table_dtype, const int* ids, float* out, int T, int H,
-                              int V, hipStream_t stream) {
+                              int V, float scale, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && H > 0 && V > 0, "pico_embedding: bad sizes T=%d H=%d V=%d", T, H, V);
   if (T == 0) return 0;
   if (table_dtype == PICO_DTYPE_F32)
-    embedding_kernel<float><<<T, 256, 0, stream>>>((const float*)table, ids, out, H, V);
+    embedding_kernel<float><<<T, 256, 0, stream>>>((const float*)table, ids, out, H, V, scale);
   else if (table_dtype == PICO_DTYPE_BF16)
-    embedding_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V);
+    embedding_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V, scale);
   else
     PICO_REQUIRE(false, "pico_embedding: unknown dtype %d", table_dtype);
   PICO_LAUNCH_CHECK();
@@ -439,6 +439,25 @@ extern "C" int pico_rope_kv_store(void* qkv, int dtype, const float* cos_sin, co
                                                        (bf16_t*)v_cache, nq, nkv, d, rot, P, num_pages);
   else
     PICO_REQUIRE(false, "pico_rope_kv_store: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+
+// ---------------------------------------------------------------------------
+// soft cap of logits in place: x = cap * tanh(x / cap), float32 (not used by the reference's model; a model
+// description may ask for it)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, long long n, float cap, float inv_cap) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    x[i] = cap * tanhf(x[i] * inv_cap);
+}
+
+extern "C" int pico_softcap(float* x, long long n, float cap, hipStream_t stream) {
+  PICO_REQUIRE(n >= 0 && cap > 0.f, "pico_softcap: bad arguments n=%lld cap=%g", n, (double)cap);
+  if (n == 0) return 0;
+  const long long blocks = (n + 255) / 256;
+  softcap_kernel<<<(int)(blocks < 4096 ? blocks : 4096), 256, 0, stream>>>(x, n, cap, 1.0f / cap);
   PICO_LAUNCH_CHECK();
   return 0;
 }

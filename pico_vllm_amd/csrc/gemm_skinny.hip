@@ -593,16 +593,29 @@ __global__ __launch_bounds__(256) void gemm_skinny_pair_kernel(const bf16_t* __r
 // 32 rows, whose blocks share the activations, would read less still, but left with one workgroup of few
 // slices in flight per compute unit it measured slower); ties go to the taller tile.  total: rows (pairs) of the matrix; k_splits: ranges
 // of k, each a workgroup of its own; x_rows: rows of activations a workgroup fetches per slice.
-static const int SK_COMPUTE_UNITS = 256;
+// Compute units of the current device, asked once per device; 256 (an MI355X) where no device answers (a build
+// check without a GPU).
+static int sk_compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+#define SK_COMPUTE_UNITS sk_compute_units()
 static int skinny_tile_height(long long total, int unit, int k_splits, int x_rows, double* cost_out = nullptr,
                               int tiles_per_wg = 1, int step = 1) {
   int best = 0;
   double best_cost = 0;
+  const int cus = SK_COMPUTE_UNITS;
   for (int h = 32 / unit; h >= 1; h -= step) {       // rows or pairs per tile
     const long long wgs = (total + h * tiles_per_wg - 1) / (h * tiles_per_wg) * k_splits;
     // whole rounds of workgroups while they are few; many rounds run into one another
-    const double rounds = wgs <= 4 * SK_COMPUTE_UNITS ? (double)((wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS)
-                                                      : (double)wgs / SK_COMPUTE_UNITS;
+    const double rounds = wgs <= 4 * cus ? (double)((wgs + cus - 1) / cus) : (double)wgs / cus;
     const double cost = rounds * (h * unit * tiles_per_wg + x_rows);
     if (best == 0 || cost < best_cost) best = h, best_cost = cost;
   }

@@ -52,7 +52,8 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
 
     ``pad_to``: pad a pure-decode batch with empty rows up to that many
     sequences (for replaying a graph captured at that size); a padded row has a
-    block table of -1, so nothing is written for it, and its output is ignored.
+    block table of -1 and a context of 0, so nothing is written for it, its state slot is
+    the spare one behind the requests' slots, and its output is ignored.
     """
     B = len(seqs)
     if B == 0:
@@ -129,7 +130,7 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         t += 1
         h_cu[b + 1] = t
         h_ctx[b] = 0
-        h_slot[b] = 0
+        h_slot[b] = manager.slots.num_slots       # the spare slot that no request ever holds
     width = buf.max_pages if pad_to else need_pages
     if width > buf.max_pages:
         raise BatchError(f"a sequence needs {width} pages, the buffers hold {buf.max_pages} per sequence")

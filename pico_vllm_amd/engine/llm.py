@@ -14,6 +14,7 @@ from typing import Dict, List, Optional, Sequence, Union
 import torch
 
 from ..config.engine_args import EngineArgs
+from ..ops import linear
 from ..parts.model import DecoderModel, load_model
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
@@ -46,6 +47,10 @@ class LLMEngine:
             raise RuntimeError("pico_vllm_amd runs on an AMD GPU only; no GPU is visible to torch")
         self.args = args
         self.model = model if model is not None else load_model(args.model, args.dtype, args.device)
+        if args.max_seq_len > self.model.spec.max_position:
+            raise ValueError(f"max_seq_len = {args.max_seq_len} exceeds the model's max_position_embeddings = "
+                             f"{self.model.spec.max_position}")
+        linear.set_library_tuning(args.tune_library_gemm)
         num_pages = args.num_gpu_blocks
         if num_pages is None:
             num_pages = args.max_num_seqs * (-(-args.max_seq_len // args.block_size))
@@ -190,6 +195,9 @@ class LLMEngine:
         return [int(t) for t in prompt]
 
     def _output(self, r: Request) -> RequestOutput:
+        # a finished request leaves the engine's books with its report (the reference keeps every request
+        # for the life of the engine, pico_vllm/engine.py:262)
+        self.requests.pop(r.request_id, None)
         text = None
         if self.tokenizer is not None:
             text = self.tokenizer.decode(r.input_ids + r.generated_ids)     # prompt + generated, engine.py:385

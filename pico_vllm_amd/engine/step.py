@@ -43,7 +43,8 @@ class ModelRunner:
         rows = max(max_seqs, _bucket(min(max_seqs, max_graph_batch))) if use_graph else max_seqs
         self.buffers = BatchBuffers(self.device, max(max_tokens_per_step, rows), rows, self.max_pages,
                                     max(1, len(self.manager.groups)))
-        self.use_graph = use_graph
+        # a part that decides on the host per step (``Part.graph_safe`` False) keeps the whole model out of graphs
+        self.use_graph = use_graph and model.is_graph_safe()
         self.max_graph_batch = max_graph_batch
         self._graphs: Dict[int, tuple] = {}
         self.steps = 0
@@ -63,6 +64,8 @@ class ModelRunner:
         for s in seqs:
             if self.manager.num_computed(s.req) + len(s.tokens) > self.max_seq_len:
                 raise BatchError(f"request {s.req!r} would grow beyond max_seq_len={self.max_seq_len}")
+        # state slots that new requests took start from zero; outside any graph
+        self.storage.reset_state(self.manager.take_fresh_slots())
         decode_only = all(len(s.tokens) == 1 and list(s.want) == [0] for s in seqs)
         if self.use_graph and decode_only and len(seqs) <= self.max_graph_batch:
             logits = self._step_graph(seqs, device_tokens)
@@ -98,11 +101,13 @@ class ModelRunner:
         return out[:B]
 
     def _capture(self, size: int, seqs: List[SeqStep]) -> None:
-        """Warm up on the real batch (which also writes this step's keys; the replay
-        that follows writes the same values again), then record the graph."""
+        """Warm up on the real batch, then record the graph.  The warm-up runs write this step's keys and
+        values, which the replay that follows writes again with the same values; per-request state, which
+        a run changes from what it was, is put back afterwards so that only the replay counts."""
         ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
                             pad_to=size)
         ctx.max_context = self.max_seq_len          # kernel choices must hold for every later replay
+        saved = self.storage.save_state()
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -113,6 +118,7 @@ class ModelRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             out = self.model.forward(ctx, self.storage)
+        self.storage.restore_state(saved)
         self._graphs[size] = (graph, out)
 
     # ---- sizes for reports ----------------------------------------------

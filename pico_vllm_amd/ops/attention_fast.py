@@ -12,6 +12,16 @@ from .kernels import KernelError, _check, _check_cache, _ptr, _stream
 c_float = ctypes.c_float
 
 
+_cus = {}
+
+
+def compute_units(device: int = 0) -> int:
+    """Compute units of the GPU, asked once (256 on an MI355X); the cost models below count workgroups against it."""
+    if device not in _cus:
+        _cus[device] = torch.cuda.get_device_properties(device).multi_processor_count if torch.cuda.is_available() else 256
+    return _cus[device]
+
+
 def supported(nq: int, nkv: int, head_dim: int, window: int) -> bool:
     """Head sizes in steps of 16 up to 256, no window; anything else goes to the plain kernel."""
     return head_dim % 16 == 0 and 16 <= head_dim <= 256 and window == 0 and nq % nkv == 0
@@ -23,9 +33,10 @@ class FastAttention:
         self.lib = library.attention_library(head_dim)
         if self.lib.pico_attn_head_dim() != head_dim:
             raise KernelError("attention library was built for another head size")
+        self.cus = compute_units()
 
     def num_splits(self, num_seqs: int, max_context: int) -> int:
-        """Enough workgroups to fill the chip (256 CUs, two workgroups each), no split shorter
+        """Enough workgroups to fill the chip (two workgroups a compute unit), no split shorter
         than one 64-key tile (or, beyond 64 splits, than two), at most 256 splits (what the merging kernel takes):
         a single request with 32,768 tokens behind it is read by 512 workgroups, not by 128."""
         # the number of sequences counts as the power of two that a recorded step of them is padded to, so that
@@ -33,7 +44,7 @@ class FastAttention:
         padded = 1
         while padded < num_seqs:
             padded *= 2
-        by_fill = max(1, 512 // max(1, padded * self.nkv))
+        by_fill = max(1, 2 * self.cus // max(1, padded * self.nkv))
         by_len = max(1, -(-max_context // 64))
         if by_len > 64:
             by_len = max(64, -(-max_context // 128))
@@ -57,9 +68,10 @@ class FastAttention:
             total += tiles * max(1, (2 * c - n) // 128)      # mean key tiles of the portion's query tiles
             tokens += n
             padded += -(-n // 128) * 128
-        if total * self.nq < 256 * longest:
+        cus = getattr(self, "cus", None) or compute_units()
+        if total * self.nq < cus * longest:
             return 3
-        return 4 if total * self.nq >= 256 * 64 and 4 * tokens >= 3 * padded else 1
+        return 4 if total * self.nq >= cus * 64 and 4 * tokens >= 3 * padded else 1
 
     def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
                 scale: float, out: Optional[torch.Tensor] = None, teams: int = 0) -> torch.Tensor:

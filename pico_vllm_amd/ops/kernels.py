@@ -78,8 +78,8 @@ def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
         raise KernelError(f"{name} has {t.numel()} entries, {n} are needed")
 
 
-def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = table[ids[t]] as float32 rows (the residual stream)."""
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale as float32 rows (the residual stream)."""
     _gpu(table, ids)
     V, H = table.shape
     T = ids.numel()
@@ -91,8 +91,18 @@ def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor
     elif out.shape != (T, H) or out.dtype != torch.float32 or not out.is_contiguous():
         raise KernelError("embedding: out must be a contiguous float32 [T, H] tensor")
     lib = library.core()
-    _check(lib, lib.pico_embedding(_ptr(table), _dt(table), _ptr(ids), _ptr(out), T, H, V, _stream()))
+    _check(lib, lib.pico_embedding(_ptr(table), _dt(table), _ptr(ids), _ptr(out), T, H, V, c_float(scale), _stream()))
     return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x = cap * tanh(x / cap) in place, float32."""
+    _gpu(x)
+    if x.dtype != torch.float32 or not x.is_contiguous() or not cap > 0:
+        raise KernelError("softcap: a contiguous float32 tensor and a positive cap")
+    lib = library.core()
+    _check(lib, lib.pico_softcap(_ptr(x), c_ll(x.numel()), c_float(cap), _stream()))
+    return x
 
 
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
@@ -203,6 +213,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
 
 
 EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
+MAX_HEAD_DIM = 256          # the largest head size any attention kernel takes
 
 
 # The weight-streaming kernel takes any number of rows in blocks of 64, each block reading the matrix

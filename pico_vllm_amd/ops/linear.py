@@ -12,29 +12,46 @@ engine) they are widened on load and the result is rounded once.
 from __future__ import annotations
 
 import os
+import tempfile
 from typing import Optional
 
 import torch
 
-from . import kernels, library
+from . import kernels
 
-# The library GEMM is picked by the library's own tuner (PyTorch's TunableOp: it times the rocBLAS and
+# The library GEMM can be picked by the library's own tuner (PyTorch's TunableOp: it times the rocBLAS and
 # hipBLASLt solutions for a shape once and keeps the fastest; on the 1.5B shapes with 2,048 rows that
-# is 91 us against 122 us for the gate/up product).  A step's row count is arbitrary, and tuning every
-# count would stall serving, so only row counts that are multiples of TUNE_ROWS (whole prompt portions)
-# are tuned; every other count takes the library's default choice.  Results are kept beside the built
-# kernels and read back by the next process.
+# is 91 us against 122 us for the gate/up product).  Timing candidates stalls the first step of a shape for
+# up to 30 s and switches a process-wide mode of torch on, so it is off unless ``set_library_tuning(True)``
+# asks for it (``EngineArgs.tune_library_gemm``; the benchmark does).  A step's row count is arbitrary, so only
+# row counts that are multiples of TUNE_ROWS (whole prompt portions) are tuned; every other count takes the
+# library's default choice.  Results are kept in a per-user file under the temp dir and read back by the next process.
 TUNE_ROWS = 512
-_tuner_state = {"ready": False, "tuning": None}
+_tuner_state = {"wanted": False, "ready": False, "tuning": None}
+
+
+def set_library_tuning(on: bool) -> None:
+    """Switch the tuner on or off for this process; off also hands torch's own mode back."""
+    st = _tuner_state
+    st["wanted"] = bool(on)
+    if not on and st["ready"] is True:
+        try:
+            torch.cuda.tunable.tuning_enable(False)
+            torch.cuda.tunable.enable(False)
+        except Exception:
+            pass
+        st["ready"], st["tuning"] = False, None
 
 
 def _library_tuning(rows: int) -> None:
-    tunable = torch.cuda.tunable
     st = _tuner_state
+    if not st["wanted"]:
+        return
+    tunable = torch.cuda.tunable
     if not st["ready"]:
         st["ready"] = True
         try:
-            path = os.path.join(library.build_root(), "tunableop_gemm.csv")
+            path = os.path.join(tempfile.gettempdir(), f"pico_vllm_amd_tunableop_{os.getuid()}.csv")
             tunable.enable(True)
             tunable.set_filename(path)
             tunable.set_max_tuning_duration(30)

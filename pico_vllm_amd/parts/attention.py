@@ -33,6 +33,10 @@ class GQAAttention(Mixer):
                  act_dtype: torch.dtype = torch.bfloat16):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
+        if not 1 <= head_dim <= kernels.MAX_HEAD_DIM:
+            raise ValueError(f"head size {head_dim} is outside what the attention kernels take (1 to {kernels.MAX_HEAD_DIM})")
+        if window < 0:
+            raise ValueError(f"window must not be negative, got {window}")
         self.hidden_size, self.nq, self.nkv, self.d = hidden_size, num_heads, num_kv_heads, head_dim
         self.qkv_bias, self.window, self.act_dtype = qkv_bias, window, act_dtype
         self.scale = 1.0 / math.sqrt(head_dim)          # pico_vllm/kernels/attention.py:92,231

@@ -37,7 +37,7 @@ class StepContext:
     token_seq: torch.Tensor          # int32 [T]   row of the token's sequence in the per-sequence arrays
     cu_seqlens: torch.Tensor         # int32 [B+1]
     context_lens: torch.Tensor       # int32 [B]   cached + new tokens
-    state_slots: torch.Tensor        # int32 [B]   slot of fixed-size state
+    state_slots: torch.Tensor        # int32 [B]   slot of fixed-size state (zeroed when a new request takes it; padding rows: the spare last slot)
     block_tables: List[torch.Tensor]  # per cache group: int32 [B, max_pages]
     slot_mapping: List[torch.Tensor]  # per cache group: int32 [T], page * page size + offset of each token (-1: none)
     want_rows: torch.Tensor          # int32 [R]   flat token indices whose logits are wanted
@@ -51,7 +51,17 @@ class StepContext:
 
 
 class Part:
-    """Common to all parts: declared tensors and loading."""
+    """Common to all parts: declared tensors and loading.
+
+    ``graph_safe``: whether the part's work in a decode step is fixed once the step's shape is (device work only,
+    nothing decided from values on the host, no synchronisation), so that the step may be recorded into a HIP graph
+    and replayed.  A part that reads ``ctx.host`` or copies values to the host per step sets it to False; a model
+    with such a part anywhere never runs from a graph, whatever the engine's options say."""
+    graph_safe = True
+
+    def is_graph_safe(self) -> bool:
+        """This part and the parts it is built from."""
+        return self.graph_safe and all(p.is_graph_safe() for p in vars(self).values() if isinstance(p, Part))
 
     def param_specs(self) -> List[ParamSpec]:
         return []
@@ -138,6 +148,9 @@ class Block(Part):
 
     def __init__(self, parts: Dict[str, Part]):
         self.parts = parts
+
+    def is_graph_safe(self) -> bool:
+        return self.graph_safe and all(p.is_graph_safe() for p in self.parts.values())
 
     @property
     def mixer(self) -> Mixer:

@@ -50,12 +50,15 @@ def model_param_specs(spec: ModelSpec) -> List[ParamSpec]:
     out += [ParamSpec(f"{spec.final_norm_name}.{p.name}", p.shape, p.role, p.std) for p in fn.param_specs()]
     if spec.head_name:
         out.append(ParamSpec(spec.head_name, (spec.vocab_size, spec.hidden_size)))
+    if spec.head_bias_name:
+        out.append(ParamSpec(spec.head_bias_name, (spec.vocab_size,), role="bias"))
     return out
 
 
 class DecoderModel:
-    """embedding -> layers in ``run_order`` -> final norm on the wanted rows ->
-    output matrix (pico_vllm/model.py:427-445).  Logits are float32 and exist
+    """embedding (times ``spec.embed_scale``) -> layers in ``run_order`` -> final norm on the wanted rows ->
+    output matrix (+ ``spec.head_bias_name``, soft cap ``spec.logit_softcap``) (pico_vllm/model.py:427-445; the
+    reference's model has no multiplier, bias or cap: 1, none and 0 here).  Logits are float32 and exist
     only for the wanted rows (the reference computes all rows and keeps the
     last, engine.py:374).  An untied model multiplies by ``lm_head.weight``
     (the reference always uses the embedding matrix, model.py:445)."""
@@ -97,7 +100,12 @@ class DecoderModel:
                 part.load({p.name: tensors[pre + p.name] for p in part.param_specs()}, dev, self.dtype)
         pre = spec.final_norm_name + "."
         self.final_norm.load({p.name: tensors[pre + p.name] for p in self.final_norm.param_specs()}, dev, self.dtype)
-        self.head = Linear(tensors[spec.head_name].to(dev) if spec.head_name else self.embed)
+        self.head = Linear(tensors[spec.head_name].to(dev) if spec.head_name else self.embed,
+                           tensors[spec.head_bias_name].to(dev) if spec.head_bias_name else None)
+
+    def is_graph_safe(self) -> bool:
+        """Whether a decode step of this model may be recorded into a HIP graph: every part says so."""
+        return all(blk.is_graph_safe() for blk in self.layers) and self.final_norm.is_graph_safe()
 
     def num_weight_bytes(self) -> int:
         """Bytes a decode step streams: every matrix once (the embedding table only as the
@@ -117,14 +125,17 @@ class DecoderModel:
 
     def _forward(self, ctx: StepContext, storage) -> torch.Tensor:
         ctx.shared.clear()      # what layers share belongs to this pass (a context may be run again, as at graph capture)
-        resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens])
+        resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens], scale=self.spec.embed_scale)
         pending = None
         for i, e in enumerate(self.spec.run_order):
             resid, pending = self.layers[e.layer].forward(resid, pending, ctx, storage.layer(self.spec.cache_id(i)))
         if ctx.want_rows.numel() == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
         h = self.final_norm.add_norm(resid, pending, rows=ctx.want_rows)
-        return self.head(h, out_dtype=torch.float32)
+        logits = self.head(h, out_dtype=torch.float32)
+        if self.spec.logit_softcap > 0:
+            kernels.softcap(logits, self.spec.logit_softcap)
+        return logits
 
 
 def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> DecoderModel:
@@ -133,8 +144,7 @@ def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") 
         raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
     _, cfg, spec = load_model_description(model_dir)
     model = DecoderModel(spec, _DTYPES[dtype], torch.device(device))
-    optional = ["lm_head.weight"] if spec.head_name is None else []
-    tensors = load_checkpoint(model_dir, model.param_specs(), _DTYPES[dtype], optional=optional)
+    tensors = load_checkpoint(model_dir, model.param_specs(), _DTYPES[dtype], optional=spec.ignored_tensors)
     model.load(tensors)
     model.config = cfg
     return model

@@ -85,6 +85,12 @@ class ModelSpec:
     head_name: Optional[str]          # None: output matrix is the embedding matrix
     eos_token_id: Optional[int] = None
     max_position: int = 131072
+    # names (shell patterns allowed) of tensors a checkpoint may hold that the model does not use: a tied model's
+    # stored output matrix, buffers that another implementation keeps in its files
+    ignored_tensors: Tuple[str, ...] = ()
+    embed_scale: float = 1.0          # the embedding rows are multiplied by this (1: as they are)
+    logit_softcap: float = 0.0        # > 0: logits = cap * tanh(logits / cap)
+    head_bias_name: Optional[str] = None   # a bias [vocab] added to the logits
 
     def cache_id(self, entry_index: int) -> int:
         """The run entry whose cache entry ``entry_index`` uses."""

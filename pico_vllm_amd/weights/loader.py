@@ -12,6 +12,7 @@ keeps everything in float32.  Integer tables become int32.
 """
 from __future__ import annotations
 
+from fnmatch import fnmatchcase
 from typing import Dict, Iterable, List
 
 import torch
@@ -54,10 +55,10 @@ def load_checkpoint(model_dir: str, wanted: Iterable[ParamSpec], engine_dtype: t
                     optional: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
     """CPU tensors for every wanted name, converted to their kept dtype.
 
-    ``optional`` names may be present without being wanted (a tied model's
-    stored ``lm_head.weight``); they are ignored."""
+    ``optional`` names (shell patterns allowed) may be present without being wanted (a tied
+    model's stored ``lm_head.weight``, ``ModelSpec.ignored_tensors``); they are ignored."""
     want: Dict[str, ParamSpec] = {p.name: p for p in wanted}
-    optional = set(optional)
+    optional = tuple(optional)
     files: List[SafetensorsFile] = []
     try:
         paths = list_safetensors(model_dir)
@@ -76,7 +77,7 @@ def load_checkpoint(model_dir: str, wanted: Iterable[ParamSpec], engine_dtype: t
                     other.append(f"tensor {name} is stored twice ({owner[name].path} and {p})")
                 owner[name] = sf
         missing = sorted(n for n in want if n not in owner)
-        unexpected = sorted(n for n in owner if n not in want and n not in optional)
+        unexpected = sorted(n for n in owner if n not in want and not any(fnmatchcase(n, pat) for pat in optional))
         wrong = []
         for n, spec in want.items():
             if n in owner:

@@ -172,3 +172,27 @@ def test_state_slots():
     assert s.acquire() == a
     with pytest.raises(PagePoolError):
         s.release(5)
+
+
+def test_a_slot_taken_by_a_new_request_is_reported_for_clearing():
+    # a state slot is handed out as the last holder left it; the manager tells the owner of the tensors which
+    # slots new requests took, once, so that no mixer has to find out by itself that a request is new
+    m = CacheManager({0: FULL, 1: STATE}, 16, 8, 2)
+    assert m.add_request("a") and m.add_request("b")
+    assert sorted(m.take_fresh_slots()) == [0, 1] and m.take_fresh_slots() == []
+    m.free_request("a")
+    assert m.add_request("c") and m.take_fresh_slots() == [m.slot("c")]
+    # a model without state has nothing to clear
+    plain = CacheManager({0: FULL}, 16, 8, 2)
+    assert plain.add_request("a") and plain.take_fresh_slots() == []
+
+
+def test_a_model_with_state_cannot_share_a_prefix():
+    m = CacheManager({0: FULL, 1: STATE}, 16, 8, 2)
+    m.add_request("a")
+    assert m.grow("a", 32)
+    m.advance("a", 32)
+    m.add_request("b")
+    with pytest.raises(PagePoolError, match="state"):
+        m.fork_prefix("a", "b", 16)
+    m.check()

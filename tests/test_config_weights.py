@@ -168,6 +168,17 @@ def test_tied_model_ignores_a_stored_lm_head_and_untied_needs_it(tmp_path):
     os.makedirs(tmp_path / "m")
     save_file(t, str(tmp_path / "m" / "model.safetensors"))
     load_checkpoint(str(tmp_path / "m"), _specs("A"), torch.bfloat16, optional=["lm_head.weight"])
+    # the model description names what a file may hold unasked: the tied configuration does, by name or by pattern
+    from pico_vllm_amd.config.registry import resolve_architecture
+    arch = resolve_architecture(CONFIGS["A"])
+    assert arch.build_spec(arch.config_from_dict(CONFIGS["A"])).ignored_tensors == ("lm_head.weight",)
+    assert arch.build_spec(arch.config_from_dict(CONFIGS["B"])).ignored_tensors == ()
+    t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(t, str(tmp_path / "m" / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_checkpoint(str(tmp_path / "m"), _specs("A"), torch.bfloat16, optional=["lm_head.weight"])
+    assert e.value.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    load_checkpoint(str(tmp_path / "m"), _specs("A"), torch.bfloat16, optional=["lm_head.weight", "*.rotary_emb.inv_freq"])
     with pytest.raises(WeightsError) as e:
         load_checkpoint(d, _specs("A") + [ParamSpec("lm_head.weight", (256, 64))], torch.bfloat16)
     assert e.value.missing == ["lm_head.weight"]

@@ -245,3 +245,23 @@ def test_command_line_with_a_text_prompt_and_a_tokenizer_in_the_model_folder(cap
     line = [l for l in capsys.readouterr().out.splitlines() if l.startswith("[")][0]
     first = ids.index(ids[2])
     assert "(eos)" in line and line.split(")", 1)[1].split() == ["w5", "w17", "w3"] + [f"w{i}" for i in ids[:first + 1]]
+
+
+def test_what_the_model_cannot_run_is_refused_before_serving_starts():
+    from pico_vllm_amd import EngineArgs
+    from pico_vllm_amd.engine.llm import LLMEngine
+    from pico_vllm_amd.parts.attention import GQAAttention
+    from pico_vllm_amd.parts.spec import PartSpec
+    # a request could reach positions beyond what the model was made for
+    with pytest.raises(ValueError, match="max_position_embeddings"):
+        LLMEngine(EngineArgs(model=model_dir("A"), dtype="float32", max_seq_len=TINY_A["max_position_embeddings"] + 1))
+    # a head size no attention kernel takes: refused when the part is built, not at the first step
+    with pytest.raises(ValueError, match="head size"):
+        GQAAttention(1024, 2, 1, 512, True, PartSpec("none", {}))
+
+
+def test_a_finished_request_leaves_the_engine():
+    from pico_vllm_amd import SamplingParams
+    eng = llm("A", "float32")
+    eng.generate(prompts_for("A", [5, 9, 3]), SamplingParams(max_new_tokens=4, ignore_eos=True))
+    assert eng.engine.requests == {} and not eng.engine.runner.manager.requests

@@ -165,3 +165,41 @@ def test_real_layer_sizes_mixed_in_a_small_pool():
         assert pool.reuse_count > 0
         R.compare("L7B", dtype, reqs, got, "real mixed")
     torch.cuda.empty_cache()
+
+
+def test_graph_replay_and_the_step_in_flight_at_head_size_128():
+    """Decode steps replayed from a HIP graph (recorded with the longest context's kernel choices and padded rows) and the
+    decode step in flight, at the 1.5B layer sizes (heads of 128, groups of 6): batches of 1, 3 (a graph of 4) and 8;
+    the same tokens in all four modes, each the plain implementation's argmax within bfloat16 rounding
+    (the reference's graph path: pico_vllm/engine.py:139-191, its test tests/test_cuda_graph_model.py:64-197)."""
+    import plain_qwen2 as P
+    from tiny_configs import CONFIGS, model_dir
+    from pico_vllm_amd import LLM, SamplingParams
+    name = "L1.5B"
+    V = CONFIGS[name]["vocab_size"]
+    plain = P.PlainModel(model_dir(name))
+    rng = random.Random(5)
+    sp = SamplingParams(max_new_tokens=40, temperature=0.0, ignore_eos=True)
+    for batch in (1, 3, 8):
+        prompts = [[rng.randrange(V) for _ in range(rng.choice([3, 17, 40, 70]))] for _ in range(batch)]
+        seen = {}
+        for graph in (False, True):
+            for pipeline in (False, True):
+                llm = LLM(model=model_dir(name), dtype="bfloat16", block_size=16, num_gpu_blocks=8 * 8, max_seq_len=128,
+                          max_num_seqs=8, max_num_batched_tokens=256, use_cuda_graph=graph, max_batch_size=8,
+                          pipeline_decode=pipeline)
+                outs = llm.generate(prompts, sp)
+                if graph:
+                    assert (1 if batch == 1 else 4 if batch == 3 else 8) in llm.engine.runner._graphs
+                seen[graph, pipeline] = [o.token_ids for o in outs]
+                del llm
+                torch.cuda.empty_cache()
+        first = seen[False, False]
+        assert all(len(t) == 40 for t in first)
+        for mode, toks in seen.items():
+            assert toks == first, (batch, mode)
+        for p, gen in zip(prompts, first):
+            logits = plain.logits(p + gen)
+            for k, t in enumerate(gen):
+                row = logits[len(p) + k - 1]
+                assert float(row[t]) >= float(row.max()) - 0.05 * float(row.std()), (batch, len(p), k, t, int(row.argmax()))

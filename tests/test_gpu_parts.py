@@ -216,15 +216,22 @@ def test_a_toy_mixer_with_state_of_its_own_registers_builds_and_steps(dtype):
             self.w = tensors["mix.weight"].to(device).float()
 
         def forward(self, x, ctx, cache):
+            H = self.H
+            if ctx.all_decode:
+                # one token a sequence: device work only, so the step may be recorded into a graph and replayed
+                # (padding rows of a recorded batch all point at the spare slot)
+                slots = ctx.state_slots[:ctx.num_seqs].long()
+                st = cache.state.index_select(0, slots)
+                sums = st[:, :H] + x.float()
+                counts = st[:, H] + 1
+                cache.state.index_copy_(0, slots, torch.cat([sums, counts[:, None]], 1))
+                return ((sums / counts[:, None]) @ self.w.T).to(x.dtype)
             out = torch.empty_like(x)
             cu = ctx.host["cu_seqlens"]
             slots = ctx.state_slots.tolist()
-            ctxl = ctx.host["context_lens"]
             for b in range(ctx.num_seqs):
                 lo, hi = int(cu[b]), int(cu[b + 1])
-                st = cache.state[slots[b]]
-                if int(ctxl[b]) - (hi - lo) == 0:
-                    st.zero_()                                  # a new request starts from empty state
+                st = cache.state[slots[b]]                      # zero when the request is new: the framework sees to it
                 xs = x[lo:hi].float()
                 sums = st[:self.H] + torch.cumsum(xs, 0)
                 counts = st[self.H] + torch.arange(1, hi - lo + 1, device=x.device)
@@ -279,6 +286,60 @@ def test_a_toy_mixer_with_state_of_its_own_registers_builds_and_steps(dtype):
         for rid in toks:
             close(torch.cat(got[rid]), whole[rid], dtype, scale=float(whole[rid].std()) * 3)
         assert whole["a"].shape == (29, 100) and float(whole["a"].std()) > 0.01
+        del r, model
+
+        # through the entry point, with graphs: five requests through two state slots (every slot is taken again by a
+        # later request and must start from zero), decode steps replayed from graphs; the same tokens as without graphs
+        # and as each request alone in an engine of its own
+        from pico_vllm_amd import LLM, SamplingParams
+        prompts = [list(range(1, 12)), [7, 3], list(range(40, 70)), [9], list(range(80, 97))]
+        sp = SamplingParams(max_new_tokens=12, temperature=0.0, ignore_eos=True)
+        kind = "float32" if dtype == torch.float32 else "bfloat16"
+
+        def run(ps, **kw):
+            llm = LLM(model=d, dtype=kind, block_size=16, num_gpu_blocks=8, max_seq_len=64, max_num_batched_tokens=64, **kw)
+            outs = [o.token_ids for o in llm.generate(ps, sp)]
+            return outs, llm.engine.runner
+        graphed, runner = run(prompts, max_num_seqs=2, use_cuda_graph=True, max_batch_size=2)
+        assert runner.use_graph and runner._graphs, "the toy mixer is graph-safe: decode steps were to be replayed"
+        eager, _ = run(prompts, max_num_seqs=2, use_cuda_graph=False)
+        assert graphed == eager
+        if dtype == torch.float32:          # alone the batch has another shape: in bfloat16 the library's product may round otherwise
+            alone = [run([p], max_num_seqs=1, use_cuda_graph=False)[0][0] for p in prompts]
+            assert eager == alone
+        one_slot, _ = run(prompts, max_num_seqs=1, use_cuda_graph=False)      # every request takes slot 0 after another
+        assert one_slot == eager or dtype != torch.float32
+
+
+def test_a_part_that_decides_on_the_host_keeps_the_model_out_of_graphs():
+    """``graph_safe = False`` on any part: the runner never records a graph, whatever the options say."""
+    import dataclasses
+    from pico_vllm_amd.config.registry import load_model_description
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.base import FeedForward
+    from pico_vllm_amd.parts.model import DecoderModel
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import LayerSpec, PartSpec
+
+    @register_part("feed_forward", "toy_host_decides")
+    class HostDecides(FeedForward):
+        graph_safe = False
+
+        def __init__(self, act_dtype=torch.bfloat16):
+            pass
+
+        def forward(self, x, ctx):
+            return x * float(len(ctx.host["cu_seqlens"]))
+
+    _, cfg, spec = load_model_description(model_dir("A"))
+    safe = DecoderModel(spec, torch.bfloat16, torch.device(DEV))
+    assert safe.is_graph_safe()
+    l0 = spec.layers[0]
+    layers = [LayerSpec(l0.prefix, l0.block, {**l0.slots, "ff": ("mlp", PartSpec("toy_host_decides", {}))})] + list(spec.layers[1:])
+    model = DecoderModel(dataclasses.replace(spec, layers=layers), torch.bfloat16, torch.device(DEV))
+    assert not model.is_graph_safe()
+    assert ModelRunner(safe, 16, 8, 2, 64, 64, use_graph=True).use_graph
+    assert not ModelRunner(model, 16, 8, 2, 64, 64, use_graph=True).use_graph
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -464,3 +525,49 @@ def test_a_block_leaves_the_norm_of_a_single_row_to_a_part_that_takes_it():
     blk, _ = block(Drops())
     with pytest.raises(RuntimeError, match="deferred norm"):
         blk.forward(torch.randn(1, H).to(DEV), None, None, None)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_description_with_an_embedding_multiplier_a_head_bias_and_a_soft_cap(dtype):
+    """What surrounds the layers is data of the model description too: the framework's layers between an embedding
+    times 3, an output matrix with a bias and logits capped at 2 tanh(x / 2), registered here as an architecture of
+    its own, written with random weights, stepped in portions and compared with the plain parts."""
+    import dataclasses
+    import tempfile
+    from pico_vllm_amd.config.model_config import Qwen2Config
+    from pico_vllm_amd.config.qwen2 import qwen2_spec
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.weights.random_init import write_random_model
+    from tiny_configs import TINY_B, strong
+    SCALE, CAP = 3.0, 2.0
+    register_architecture("ToyCappedLM", Qwen2Config.from_dict,
+                          lambda cfg: dataclasses.replace(qwen2_spec(cfg), embed_scale=SCALE, logit_softcap=CAP,
+                                                          head_bias_name="toy_head.bias"))
+    cfg = dict(TINY_B, architectures=["ToyCappedLM"])
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=4, std_overrides=dict(strong(cfg), **{"toy_head.bias": 0.5}))
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        r = ModelRunner(model, 8, 16, 2, 64, 64)
+        plain = P.PlainModel(d)
+        toks = torch.randint(0, 383, (37,), generator=torch.Generator().manual_seed(6)).tolist()
+
+        def want(rnd):
+            x = plain.w["model.embed_tokens.weight"][toks].float() * SCALE
+            for i in range(plain.cfg.num_hidden_layers):
+                x = P.block(x, plain.w, i, plain.cfg, torch.arange(len(toks)), rnd)
+            h = rnd(P.rms_norm(x, plain.w["model.norm.weight"], plain.cfg.rms_norm_eps))
+            return CAP * torch.tanh((h @ plain.w["lm_head.weight"].T + plain.w["toy_head.bias"]) / CAP)
+        exact, rounded = want(lambda x: x), want(P.to_bf16)
+        assert float(plain.w["toy_head.bias"].abs().max()) > 0.5 and float(exact.abs().max()) > 1.5      # bias and cap both bite
+        r.manager.add_request("r")
+        got, i = [], 0
+        for n in (20, 1, 2, 14):
+            assert r.manager.grow("r", i + n)
+            seq = [SeqStep("r", toks[i:i + n], list(range(n)))]
+            got.append(r.step(seq))
+            r.advance(seq)
+            i += n
+        close_to_plain(torch.cat(got), exact, rounded, dtype)
