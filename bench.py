@@ -7,12 +7,20 @@
                                                             (64 requests, prompts of 128..4096 tokens, 256 new tokens each,
                                                              continuous batching with prompts cut into portions)
 
+  python bench.py --workload long --shape 32b --device-weights --context 32768
+                                                            (one 16k-token prompt in portions of 2,048, then decode at
+                                                             batch 1 and 8 with contexts ending at the context length;
+                                                             --device-weights draws the weights on the GPU, no file)
+
 A step is one decode step of the engine (scheduler, model step from a HIP graph, sampling) at
 batch 8 with every request's context ending at 4096 tokens.  One JSON line goes to stdout:
-decoded tokens a second as ``value``; ``prefill`` (one 2,048-token prompt in one step) with its
-fraction of the bf16 matrix-core peak; ``roofline`` (bytes the decode step has to read: every
-weight once plus the cache of the live requests, over its time, against 8 TB/s); ``points``
-with decode at batch 1 and 64.
+decoded tokens a second as ``value`` (K steps between two synchronisations, the contract's clock);
+``ms_per_step_median`` from device events around every step; ``prefill`` (one 2,048-token prompt in one
+step, median of device-event times) with its TFLOP/s and its fraction of the bf16 matrix-core peak;
+``roofline`` (bytes the decode step has to read: every weight once plus the cache of the live requests,
+over its time, against 8 TB/s); ``points`` with decode at batch 1 and 64.  Beside the published peaks
+stand measured ones (``measured_peak``): a read stream over 2 GiB and a loop of matrix-core products, by
+this package's own kernels on the same GPU in the same run.
 """
 from __future__ import annotations
 
@@ -55,6 +63,46 @@ def prefill_flops(cfg, T: int) -> float:
     return per_token * T + attn + 2.0 * H * V
 
 
+def measured_peaks():
+    """(read stream in bytes/s, bf16 matrix-core loop in flop/s) on this GPU, once per run."""
+    global _PEAKS
+    if _PEAKS is None:
+        from pico_vllm_amd.ops import peaks
+        _PEAKS = (peaks.read_bandwidth(), peaks.mfma_peak()[0])
+        log(f"measured peaks: read stream {_PEAKS[0] / 1e12:.2f} TB/s, bf16 matrix cores {_PEAKS[1] / 1e15:.2f} PFLOP/s")
+    return _PEAKS
+
+
+_PEAKS = None
+
+
+def device_model(cfg, dtype, seed=0):
+    """The model of ``cfg`` with random weights drawn on the GPU (same distributions as the random-weights
+    folders: matrices and biases N(0, 0.02), norm weights 1 + U(-0.1, 0.1)): for sizes whose file would take
+    longer to write and read than the measurement."""
+    import torch
+    from pico_vllm_amd.config.registry import resolve_architecture
+    from pico_vllm_amd.parts.model import DecoderModel
+    arch = resolve_architecture(cfg)
+    typed = arch.config_from_dict(cfg)
+    model = DecoderModel(arch.build_spec(typed), {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype],
+                         torch.device("cuda:0"))
+    g = torch.Generator(device="cuda:0").manual_seed(seed)
+    tensors = {}
+    for p in model.param_specs():
+        if p.role == "norm":
+            tensors[p.name] = 1.0 + (torch.rand(p.shape, generator=g, device="cuda:0") * 0.2 - 0.1)
+        elif p.role == "table":
+            tensors[p.name] = torch.zeros(p.shape, dtype=torch.int32, device="cuda:0")
+        else:
+            t = torch.empty(p.shape, dtype=model.dtype, device="cuda:0")
+            t.normal_(0.0, p.std, generator=g)
+            tensors[p.name] = t
+    model.load(tensors)
+    model.config = typed
+    return model
+
+
 def make_engine(model_dir, dtype, batch, layers_model=None):
     from pico_vllm_amd import EngineArgs
     from pico_vllm_amd.engine.llm import LLMEngine
@@ -79,8 +127,12 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
         ids = torch.randint(0, V, (prompt_len,), generator=g).tolist()
         eng.submit(ids, max_new_tokens=warmup + steps + 1 + slack, temperature=0.0, ignore_eos=True)
     t0 = time.time()
+    said = time.time()
     while any(r.num_uncomputed > 1 or not r.generated_ids for r in eng.requests.values()):
         eng.step()                                   # prompt portions (and the first decodes of early requests)
+        if time.time() - said > 20:
+            said = time.time()
+            log(f"batch {batch}: {sum(r.num_computed for r in eng.requests.values())} of {batch * prompt_len} prompt tokens in the cache")
     torch.cuda.synchronize()
     log(f"batch {batch}: prompts of {prompt_len} tokens in the cache after {time.time() - t0:.1f}s")
     # bring every request to the same number of generated tokens is not needed: all decode from here on
@@ -88,25 +140,35 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
         eng.step()
     torch.cuda.synchronize()
     ctx_start = [r.total_len - 1 for r in eng.requests.values()]
+    pool = eng.runner.manager.groups[0].pool
+    pages_in_use = pool.num_used
+    # the contract's clock: K steps between two synchronisations; and an event behind every step's launches, whose
+    # distances are the steps' times on the device
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
         done = eng.step()
+        marks[i + 1].record()
         if done:
             raise RuntimeError("a request finished inside the timed region")
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
     ctx_mean = [c + (steps - 1) / 2 + 1 for c in ctx_start]          # keys read per step, averaged over the region
     nbytes = eng.runner.decode_bytes([int(c) for c in ctx_mean])
     ms = dt / steps * 1e3
     res = {"prompt_len": prompt_len, "tok_s": batch * steps / dt, "ms_per_step": ms, "bytes": nbytes, "gbps": nbytes / (dt / steps) / 1e9,
-           "context": sum(ctx_mean) / batch}
+           "context": sum(ctx_mean) / batch, "ms_median": per_step[len(per_step) // 2], "ms_min": per_step[0],
+           "pages_in_use": pages_in_use, "pages": pool.num_pages}
     model = eng.model
     del eng
     torch.cuda.empty_cache()
     return res, model
 
 
-def prefill_point(model_dir, model, dtype, reps=3):
+def prefill_point(model_dir, model, dtype, reps=7):
     import torch
     from pico_vllm_amd.engine.batch import SeqStep
     eng = make_engine(model_dir, dtype, 1, model)
@@ -119,15 +181,57 @@ def prefill_point(model_dir, model, dtype, reps=3):
         m.add_request(rid)
         assert m.grow(rid, PREFILL_TOKENS)
         seq = [SeqStep(rid, ids, [PREFILL_TOKENS - 1])]
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
+        e0.record()
         eng.runner.step(seq)
+        e1.record()
         torch.cuda.synchronize()
-        times.append(time.perf_counter() - t0)
+        times.append(e0.elapsed_time(e1) * 1e-3)
         m.free_request(rid)
-    dt = min(times[1:])
-    return {"value": PREFILL_TOKENS / dt, "tokens": PREFILL_TOKENS, "ms": dt * 1e3,
-            "frac": prefill_flops(CONFIG, PREFILL_TOKENS) / dt / MFMA_PEAK[dtype]}
+    times = sorted(times[1:])                         # the first run builds, tunes and warms
+    dt = times[len(times) // 2]
+    flops = prefill_flops(CONFIG, PREFILL_TOKENS)
+    out = {"value": PREFILL_TOKENS / dt, "tokens": PREFILL_TOKENS, "ms": dt * 1e3, "ms_min": times[0] * 1e3,
+           "tflops": flops / dt / 1e12, "frac": flops / dt / MFMA_PEAK[dtype]}
+    if dtype == "bfloat16":
+        peak = measured_peaks()[1]
+        out["measured_peak_tflops"] = peak / 1e12
+        out["frac_of_measured"] = flops / dt / peak
+    return out
+
+
+def long_prompt_point(model_dir, model, dtype, prompt_len):
+    """One prompt of ``prompt_len`` tokens through the scheduler, cut into portions of PREFILL_TOKENS; the time
+    until its first token is sampled."""
+    import torch
+    eng = make_engine(model_dir, dtype, 1, model)
+    V = CONFIG["vocab_size"]
+    g = torch.Generator().manual_seed(3)
+    warm = eng.submit(torch.randint(0, V, (PREFILL_TOKENS + 40,), generator=g).tolist(), max_new_tokens=2, ignore_eos=True)
+    while not eng.is_done():
+        eng.step()                                   # kernels built, library products chosen
+    torch.cuda.synchronize()
+    rid = eng.submit(torch.randint(0, V, (prompt_len,), generator=g).tolist(), max_new_tokens=2, temperature=0.0, ignore_eos=True)
+    req = eng.requests[rid]
+    steps = 0
+    t0 = time.perf_counter()
+    while not req.generated_ids:
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    while not eng.is_done():
+        eng.step()
+    model = eng.model
+    del eng
+    torch.cuda.empty_cache()
+    return {"tokens": prompt_len, "portions": steps, "ms": dt * 1e3, "tok_s": prompt_len / dt,
+            "tflops": prefill_flops_long(CONFIG, prompt_len) / dt / 1e12}, model
+
+
+def prefill_flops_long(cfg, T):
+    return prefill_flops(cfg, T)
 
 
 def serve_point(model_dir, dtype, requests, max_new):
@@ -219,8 +323,12 @@ def main() -> int:
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
     ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve"],
-                    help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long"],
+                    help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once; "
+                         "long: one prompt of --prompt tokens in portions, then decode at batch 1 and 8 at the context length")
+    ap.add_argument("--prompt", type=int, default=16384, help="prompt tokens of the long workload")
+    ap.add_argument("--device-weights", action="store_true",
+                    help="draw the random weights on the GPU instead of writing and reading a model folder")
     ap.add_argument("--requests", type=int, default=64, help="requests of the serve workload")
     ap.add_argument("--max-new", type=int, default=256, help="new tokens per request of the serve workload")
     ap.add_argument("--attention", metavar="SEQS,NEW,PREFIX[,SHAPE]", default=None,
@@ -256,7 +364,18 @@ def main() -> int:
         return 0
     tmp = None
     model_dir = a.model
-    if model_dir is None:
+    preloaded = None
+    if a.device_weights:
+        if a.workload == "serve":
+            print("bench.py: --device-weights serves the decode and long workloads")
+            return 2
+        t0 = time.time()
+        log(f"drawing random weights of the {shape_name}, {CONFIG['num_hidden_layers']} layers, on the GPU ...")
+        preloaded = device_model(CONFIG, a.dtype)
+        torch.cuda.synchronize()
+        log(f"... {time.time() - t0:.0f}s, {preloaded.num_weight_bytes() / 1e9:.1f} GB of matrices")
+        model_dir = ""
+    elif model_dir is None:
         tmp = tempfile.mkdtemp(prefix="pico_bench_")
         model_dir = tmp
         t0 = time.time()
@@ -281,14 +400,42 @@ def main() -> int:
                            "preemptions": r["preemptions"]}}), flush=True)
             return 0
         if a.prefill_only:
-            print(json.dumps({"prefill": prefill_point(model_dir, None, a.dtype)}), flush=True)
+            print(json.dumps({"prefill": prefill_point(model_dir, preloaded, a.dtype)}), flush=True)
             return 0
-        main_res, model = decode_point(model_dir, None, a.dtype, a.batch, a.steps, a.warmup)
+        if a.workload == "long":
+            if a.prompt + 8 > CONTEXT:
+                print(f"bench.py: --prompt {a.prompt} does not fit --context {CONTEXT}")
+                return 2
+            lp, model = long_prompt_point(model_dir, preloaded, a.dtype, a.prompt)
+            log(f"prompt of {a.prompt} tokens in {lp['portions']} portions: {lp['ms']:.1f} ms, {lp['tok_s']:.0f} tok/s")
+            pts = {}
+            for b in (1, 8):
+                r, model = decode_point(model_dir, model, a.dtype, b, a.steps, a.warmup)
+                log(f"decode batch {b} at context {CONTEXT}: {r['tok_s']:.0f} tok/s, {r['ms_per_step']:.3f} ms/step, {r['gbps'] / 1e3:.2f} TB/s")
+                pts[f"decode_b{b}"] = {"tok_s": round(r["tok_s"], 1), "ms_per_step": round(r["ms_per_step"], 4),
+                                       "ms_per_step_median": round(r["ms_median"], 4), "gbytes_per_step": round(r["bytes"] / 1e9, 2),
+                                       "hbm_frac": round(r["gbps"] * 1e9 / HBM_PEAK, 4), "pages_in_use": r["pages_in_use"]}
+            print(json.dumps({
+                "metric": f"decode tok/s @ batch 8 at context {CONTEXT} after a {a.prompt}-token prompt in portions of {PREFILL_TOKENS}, {shape_name.split()[0]} bf16",
+                "value": pts["decode_b8"]["tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                "ms_per_step": pts["decode_b8"]["ms_per_step"], "higher_is_better": True,
+                "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+                "data": "synthetic: random weights N(0, 0.02)" + (" drawn on the GPU" if a.device_weights else "") + ", uniform random token ids",
+                "config": {"model": shape_name, "layers": full["num_hidden_layers"], "layers_run": CONFIG["num_hidden_layers"],
+                           "hidden": CONFIG["hidden_size"], "q_heads": CONFIG["num_attention_heads"],
+                           "kv_heads": CONFIG["num_key_value_heads"], "intermediate": CONFIG["intermediate_size"],
+                           "vocab": CONFIG["vocab_size"], "seq_len": CONTEXT, "prompt": a.prompt, "portion": PREFILL_TOKENS,
+                           "page_size": 16, "weight_gbytes": round(model.num_weight_bytes() / 1e9, 1)},
+                "long_prompt": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in lp.items()},
+                "points": pts}), flush=True)
+            return 0
+        main_res, model = decode_point(model_dir, preloaded, a.dtype, a.batch, a.steps, a.warmup)
         log(f"decode batch {a.batch}: {main_res['tok_s']:.0f} tok/s, {main_res['ms_per_step']:.3f} ms/step")
         out = {
             "metric": f"decode tok/s @ batch {a.batch}, {shape_name.split()[0]} bf16 (plus batch 1/64 and prefill @ 2048 tok)",
             "value": round(main_res["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
-            "warmup": a.warmup, "ms_per_step": round(main_res["ms_per_step"], 4), "higher_is_better": True,
+            "warmup": a.warmup, "ms_per_step": round(main_res["ms_per_step"], 4),
+            "ms_per_step_median": round(main_res["ms_median"], 4), "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
             "config": {"model": shape_name, "global_batch": a.batch, "seq_len": CONTEXT,
@@ -301,8 +448,14 @@ def main() -> int:
                        "page_size": 16, "prompt_len": int(main_res["prompt_len"]),
                        "context_in_timed_steps": round(main_res["context"], 1)},
             "roofline": {"bound": "hbm", "achieved": round(main_res["gbps"], 1), "peak": HBM_PEAK / 1e9,
-                         "unit": "GB/s", "frac": round(main_res["gbps"] * 1e9 / HBM_PEAK, 4)},
+                         "unit": "GB/s", "frac": round(main_res["gbps"] * 1e9 / HBM_PEAK, 4),
+                         "gbytes_per_step": round(main_res["bytes"] / 1e9, 3)},
+            "pages_in_use": main_res["pages_in_use"], "pages": main_res["pages"],
         }
+        if a.dtype == "bfloat16":
+            stream = measured_peaks()[0]
+            out["roofline"]["measured_peak"] = round(stream / 1e9, 1)
+            out["roofline"]["frac_of_measured"] = round(main_res["gbps"] * 1e9 / stream, 4)
         if not a.no_points:
             out["prefill"] = {k: (round(v, 4) if isinstance(v, float) else v)
                               for k, v in prefill_point(model_dir, model, a.dtype).items()}

@@ -31,6 +31,8 @@ CORE_SOURCES = ("errors.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip"
 
 ATTN_SOURCES = ("errors.hip", "attention_mfma.hip")
 
+PEAK_SOURCES = ("errors.hip", "peaks.hip")
+
 _loaded: Dict[str, ctypes.CDLL] = {}
 
 
@@ -139,9 +141,14 @@ def attention_library(head_dim: int) -> ctypes.CDLL:
     return load_library(f"pico_attn_d{head_dim}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={head_dim}",))
 
 
+def peaks() -> ctypes.CDLL:
+    """The two measuring kernels of the benchmark (a read stream, a matrix-core loop)."""
+    return load_library("pico_peaks", PEAK_SOURCES)
+
+
 def build_all(head_dims: Iterable[int] = (16, 32, 48, 64, 80, 96, 128, 160, 192, 224, 256), force: bool = True) -> List[str]:
     """Compile everything (used by the build check); returns the paths."""
-    out = [build_library("pico_core", CORE_SOURCES, force=force)]
+    out = [build_library("pico_core", CORE_SOURCES, force=force), build_library("pico_peaks", PEAK_SOURCES, force=force)]
     if os.path.isfile(os.path.join(CSRC, "attention_mfma.hip")):
         for d in head_dims:
             out.append(build_library(f"pico_attn_d{d}", ATTN_SOURCES, (f"-DPICO_HEAD_DIM={d}",), force=force))
