@@ -67,6 +67,19 @@ class ModelRunner:
         # state slots that new requests took start from zero; outside any graph
         self.storage.reset_state(self.manager.take_fresh_slots())
         decode_only = all(len(s.tokens) == 1 and list(s.want) == [0] for s in seqs)
+        back = None
+        if not decode_only:
+            # Single-token sequences first: the attention then serves them through the decode kernel, whoever
+            # ordered the batch (the scheduler does so itself; a replayed trace may not).  The logits go back
+            # into the caller's order below; what a row holds does not depend on where it stood.
+            order = sorted(range(len(seqs)), key=lambda i: len(seqs[i].tokens) != 1)
+            if order != list(range(len(seqs))):
+                first_row, at = {}, 0
+                for i in order:
+                    first_row[i] = at
+                    at += len(seqs[i].want)
+                back = [first_row[i] + j for i in range(len(seqs)) for j in range(len(seqs[i].want))]
+                seqs = [seqs[i] for i in order]
         if self.use_graph and decode_only and len(seqs) <= self.max_graph_batch:
             logits = self._step_graph(seqs, device_tokens)
         else:
@@ -79,6 +92,8 @@ class ModelRunner:
             if device_tokens is not None:
                 ctx.token_ids[:len(seqs)].copy_(device_tokens[:len(seqs)])
             logits = self.model.forward(ctx, self.storage)
+            if back is not None and logits.shape[0]:
+                logits = logits.index_select(0, torch.tensor(back, dtype=torch.long, device=logits.device))
         self.steps += 1
         self.tokens += sum(len(s.tokens) for s in seqs)
         return logits
