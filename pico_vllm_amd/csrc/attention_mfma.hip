@@ -17,6 +17,10 @@
 // Formulas as in pico_vllm/kernels/attention.py:136-213: scores (q.k) * scale, key visible iff its
 // position <= the query's, online softmax in float32, probabilities rounded to bfloat16 for the
 // P.V product, float32 accumulators.
+// A window (not in the reference: its model has none) hides keys at positions <= the query's minus the window; every
+// kernel takes it as `reach` = the window, or NO_WINDOW where there is none, so that one comparison serves both,
+// starts its key loop at the first tile that a query of the workgroup still sees and masks the lower edge in the
+// tiles that hold one.
 //
 // Matrix-core layout of the 32-query kernels (v_mfma_f32_32x32x16_bf16, D = A B, A 32x16, B 16x32): lane l supplies
 // A[l % 32][8 (l / 32) + 0..7] and B[8 (l / 32) + 0..7][l % 32]; it receives, in register r,
@@ -36,6 +40,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+constexpr int NO_WINDOW = 1 << 30;       // a reach no position gets to
 constexpr int D = PICO_HEAD_DIM;
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
 constexpr int DP = (D + 31) / 32 * 32;   // head size padded to whole 32-wide output tiles
@@ -98,13 +103,15 @@ struct TileRegs {
   // half h feeds into product m of sub-tile sub (keys 16 m + 4 h + 0..3 and 16 m + 8 + 4 h + 0..3 of the
   // sub-tile) are contiguous, so the P.V loop reads one 16-byte unit per product.  A chunk from
   // memory (8 consecutive keys) splits into two 8-byte halves that go to the units of h = 0 and 1.
-  __device__ __forceinline__ void commit(Tiles& t, int tile_start, int kv_end) const {
+  // kv_lo: keys before it are seen by no query of the workgroup (a window has passed them; their pages may
+  // belong to someone else by now): their values become zero like those beyond kv_end
+  __device__ __forceinline__ void commit(Tiles& t, int tile_start, int kv_end, int kv_lo = 0) const {
 #pragma unroll
     for (int i = 0; i < NK; i++) {
       const int c = threadIdx.x + i * NT;
       if (c < BN * KCH) *reinterpret_cast<u32x4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
     }
-    const bool tail = tile_start + BN > kv_end;              // the same for the whole workgroup
+    const bool tail = tile_start + BN > kv_end || tile_start < kv_lo;      // the same for the whole workgroup
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int c = threadIdx.x + i * NT;
@@ -116,7 +123,7 @@ struct TileRegs {
         uint32_t w[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
         for (int e = 0; e < 8; e++)
-          if (pos + e >= kv_end) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+          if (pos + e >= kv_end || pos + e < kv_lo) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
         x = make_uint4(w[0], w[1], w[2], w[3]);
       }
       // chunk kc covers keys 8 kc .. 8 kc + 7 of the tile: sub-tile kc / 4, product (kc % 4) / 2,
@@ -150,9 +157,9 @@ __device__ __forceinline__ void init_state(WaveState& st) {
 
 // One 32-key sub-tile (keys sub * 32 .. + 31 of the LDS tile) against the wave's 32 query columns.
 // q[step] is the B operand of step `step`; key_pos0 the absolute position of the sub-tile's first
-// key; q_pos the absolute position of this lane's query column (keys beyond it are masked).
+// key; q_pos the absolute position of this lane's query column (keys beyond it are masked, and keys before `lo`).
 __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf16x8* q, WaveState& st, float scale,
-                                               int key_pos0, int q_pos, bool need_mask) {
+                                               int key_pos0, int q_pos, bool need_mask, int lo = 0) {
   const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   f32x16 s;
 #pragma unroll
@@ -169,7 +176,7 @@ __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf
     float v = s[r] * scale;
     if (need_mask) {
       const int kpos = key_pos0 + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (kpos > q_pos) v = -INFINITY;
+      if (kpos > q_pos || kpos < lo) v = -INFINITY;
     }
     s[r] = v;
     mx = fmaxf(mx, v);
@@ -220,7 +227,7 @@ __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf
 //     Output and sum share the reference, so o / l is unchanged by the lag.
 template <int NS>
 __device__ __forceinline__ void attend_tile(const Tiles& t, int nsub, const bf16x8* q, WaveState& st, float c,
-                                            int key_pos0, int q_pos, bool need_mask) {
+                                            int key_pos0, int q_pos, bool need_mask, int reach = NO_WINDOW) {
   const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   f32x16 s[NS];
 #pragma unroll
@@ -242,7 +249,10 @@ __device__ __forceinline__ void attend_tile(const Tiles& t, int nsub, const bf16
     if (sub < nsub) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        if (need_mask && key_pos0 + 32 * sub + 8 * (r >> 2) + 4 * h + (r & 3) > q_pos) s[sub][r] = -INFINITY;
+        if (need_mask) {
+          const int kpos = key_pos0 + 32 * sub + 8 * (r >> 2) + 4 * h + (r & 3);
+          if (kpos > q_pos || kpos <= q_pos - reach) s[sub][r] = -INFINITY;
+        }
         mx = fmaxf(mx, s[sub][r]);
       }
     }
@@ -315,7 +325,7 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void prefill_kernel(
                                                       const int* __restrict__ cu_seqlens,
                                                       const int* __restrict__ context_lens, int num_seqs,
                                                       bf16_t* __restrict__ out, int nq, int nkv, int P,
-                                                      int num_pages, float scale) {
+                                                      int num_pages, float scale, int reach) {
   __shared__ Tiles tiles;
   // which (sequence, query tile) is this workgroup?  heavy (late) tiles of a sequence come first
   int b = 0, tile = (int)blockIdx.x, ntiles = 0;
@@ -348,16 +358,20 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void prefill_kernel(
   init_state(st);
   zero_pad_rows(tiles, 256);
   TileRegs<256> regs;
-  regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, 0, kv_end);
-  for (int tile_start = 0; tile_start < kv_end; tile_start += BN) {
+  // the first key tile that the workgroup's first query still sees (a multiple of 8, as the fetch wants)
+  const int kv_lo = max(0, prefix + tile * BM - reach + 1), kv_begin = kv_lo / BN * BN;
+  regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, kv_begin, kv_end);
+  for (int tile_start = kv_begin; tile_start < kv_end; tile_start += BN) {
     __syncthreads();                                          // everyone is done with the previous tile
-    regs.commit(tiles, tile_start, kv_end);
+    regs.commit(tiles, tile_start, kv_end, kv_lo);
     __syncthreads();
     if (tile_start + BN < kv_end) regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, tile_start + BN, kv_end);
     if (!wave_active || tile_start > wave_last_pos) continue;
+    if (tile_start + BN - 1 <= wave_first_pos - reach) continue;         // every key lies before every query's window
     // sub-tiles wholly beyond the causal frontier of this wave are left out
     const int nsub = min(BN / 32, (wave_last_pos - tile_start) / 32 + 1);
-    attend_tile<BN / 32>(tiles, nsub, qf, st, c, tile_start, q_pos, tile_start + 32 * nsub - 1 > wave_first_pos);
+    attend_tile<BN / 32>(tiles, nsub, qf, st, c, tile_start, q_pos,
+                         tile_start + 32 * nsub - 1 > wave_first_pos || tile_start <= wave_last_pos - reach, reach);
   }
   if (!q_ok) return;
   const float inv_l = 1.0f / st.l;
@@ -502,23 +516,25 @@ struct PfFetch {
       v[i] = *reinterpret_cast<const u32x4*>(vb + (off0 + ((uint32_t)((PF_NT / VCH) * i) << (pshift + 1))));
   }
 
-  __device__ __forceinline__ void commit(PfTiles<KT>& t, int tile_start, int kv_end) const {
+  // kv_lo: keys before it are seen by no query of the workgroup (a window has passed them)
+  __device__ __forceinline__ void commit(PfTiles<KT>& t, int tile_start, int kv_end, int kv_lo = 0) const {
 #pragma unroll
     for (int i = 0; i < N; i++) {
       const int c = threadIdx.x + PF_NT * i;
       *reinterpret_cast<u32x4*>(&t.k[(c / KCH) * KROW + (c % KCH) * 8]) = k[i];
     }
-    const bool tail = tile_start + PF_TK > kv_end;           // the same for the whole workgroup
+    const bool tail = tile_start + PF_TK > kv_end || tile_start < kv_lo;    // the same for the whole workgroup
     const int kc = threadIdx.x % VCH;
 #pragma unroll
     for (int i = 0; i < N; i++) {
       u32x4 x = v[i];
-      if (tail) {   // values of keys at or beyond kv_end hold whatever the page held before
+      if (tail) {   // values of keys at or beyond kv_end, or before kv_lo, hold whatever the page held before
         const int left = kv_end - (tile_start + kc * 8);       // keys of this chunk that exist
-        x[0] &= pair_mask(left);
-        x[1] &= pair_mask(left - 2);
-        x[2] &= pair_mask(left - 4);
-        x[3] &= pair_mask(left - 6);
+        const int skip = kv_lo - (tile_start + kc * 8);        // keys of this chunk before the first that is seen
+        x[0] &= pair_mask(left) & ~pair_mask(skip);
+        x[1] &= pair_mask(left - 2) & ~pair_mask(skip - 2);
+        x[2] &= pair_mask(left - 4) & ~pair_mask(skip - 4);
+        x[3] &= pair_mask(left - 6) & ~pair_mask(skip - 6);
       }
       *reinterpret_cast<u32x4*>(&t.vt[(threadIdx.x / VCH + (PF_NT / VCH) * i) * PF_VROW + kc * 8]) = x;
     }
@@ -539,7 +555,8 @@ struct PfState {
 // both at this lane quarter's 16 bytes; key_pos0: position of the team's first key.
 template <int NPAIR, bool MASK, int PF_VROW, int NQB>
 __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow, const bf16x8 (&q)[NQB][PF_KS],
-                                          PfState (&st)[NQB], float c, int key_pos0, const int (&q_pos)[NQB]) {
+                                          PfState (&st)[NQB], float c, int key_pos0, const int (&q_pos)[NQB],
+                                          int reach = NO_WINDOW) {
   const int kq = (threadIdx.x & 63) >> 4;
   f32x4p s[NQB][2 * NPAIR];
 #pragma unroll
@@ -561,7 +578,10 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
     for (int j = 0; j < 2 * NPAIR; j++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        if (MASK && key_pos0 + 32 * (j / 2) + 8 * kq + 4 * (j % 2) + r > q_pos[b]) s[b][j][r] = -INFINITY;
+        if (MASK) {
+          const int kpos = key_pos0 + 32 * (j / 2) + 8 * kq + 4 * (j % 2) + r;
+          if (kpos > q_pos[b] || kpos <= q_pos[b] - reach) s[b][j][r] = -INFINITY;
+        }
         mx = fmaxf(mx, s[b][j][r]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -616,7 +636,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
-    float scale) {
+    float scale, int reach) {
   static_assert(NQB == 1 || KT == 1, "two query blocks a wave: one team");
   constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
   constexpr int BMQ = PF_BM * NQB;            // queries per workgroup
@@ -679,15 +699,23 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   // whose chunks per key do not divide the workgroup's threads, or pages larger than that distance, go the long way
   constexpr int K_APART = PfFetch<KT>::PF_NT / PfFetch<KT>::KCH;            // keys between a thread's chunks
   const bool apart_ok = PfFetch<KT>::PF_NT % PfFetch<KT>::KCH == 0 && ((K_APART >> pshift) << pshift) == K_APART;
-  const int n_full = (apart_ok && pshift <= 4 && page_bytes < (1u << 24) && num_pages < (1 << 24)) ? kv_end / PF_TK : 0;
+  // (and no window: the first tile of a window holds keys whose values must read as zero)
+  const int n_full = (apart_ok && reach == NO_WINDOW && pshift <= 4 && page_bytes < (1u << 24) && num_pages < (1 << 24)) ? kv_end / PF_TK : 0;
+  // the first key that the workgroup's first query still sees, and its tile
+  const int kv_lo = max(0, prefix + tile * BMQ - reach + 1);
+  const int first_tile = kv_lo / PF_TK;
+  const int kv_begin = first_tile * PF_TK;
   regs.init(g, nkv, pshift);
-  regs.load_pages(bt, pshift, num_pages, 0, kv_end);
-  regs.fetch(k_cache, v_cache, g, nkv, pshift, 0, kv_end);
-  regs.load_pages(bt, pshift, num_pages, PF_TK, kv_end);
+  regs.load_pages(bt, pshift, num_pages, kv_begin, kv_end);
+  regs.fetch(k_cache, v_cache, g, nkv, pshift, kv_begin, kv_end);
+  regs.load_pages(bt, pshift, num_pages, kv_begin + PF_TK, kv_end);
   auto attend = [&](int tile_start) {
     const int key0 = tile_start + 64 * team;                    // this team's keys
     if (!wave_active || key0 > wave_last_pos) return;
-    if (key0 + 63 <= wave_first_pos) {
+    if (key0 + 63 <= wave_first_pos - reach) return;            // every key lies before every query's window
+    if (key0 <= wave_last_pos - reach) {                        // a window's lower edge runs through these keys
+      pf_attend<2, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos, reach);
+    } else if (key0 + 63 <= wave_first_pos) {
       pf_attend<2, false, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
     } else if (key0 + 32 <= wave_last_pos) {
       pf_attend<2, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
@@ -695,7 +723,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
       pf_attend<1, true, PF_VROW, NQB>(krow, vrow, qf, st, c, key0, q_pos);
     }
   };
-  int ti = 0;
+  int ti = first_tile;
   for (; ti + 2 < n_full; ti++) {            // this tile, the next and the one after it are whole
     __syncthreads();                                            // everyone is done with the previous tile
     regs.commit_full(tiles);
@@ -706,7 +734,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   }
   for (int tile_start = ti * PF_TK; tile_start < kv_end; tile_start += PF_TK) {
     __syncthreads();
-    regs.commit(tiles, tile_start, kv_end);
+    regs.commit(tiles, tile_start, kv_end, kv_lo);
     __syncthreads();
     // the next tile's keys and values (clamped to the last key if there is no next tile) and the
     // page numbers of the tile after it
@@ -782,15 +810,17 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(c
                                                      const int* __restrict__ block_table, int max_pages,
                                                      const int* __restrict__ context_lens,
                                                      float* __restrict__ part, int nsplit, int nq, int nkv, int P,
-                                                     int num_pages, float scale) {
+                                                     int num_pages, float scale, int reach) {
   __shared__ Tiles tiles;
   const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
   const int G = nq / nkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int ctx = context_lens[b];
+  // the query sits at position ctx - 1 and sees keys lo .. ctx - 1; the splits share them from the tile that holds lo on
+  const int lo = max(0, ctx - reach), lo_tile = lo / BN * BN;
   // this split's keys: a whole number of LDS tiles
-  const int per = ((ctx + nsplit - 1) / nsplit + BN - 1) / BN * BN;
-  const int k_begin = split * per, k_end = min(ctx, k_begin + per);
+  const int per = ((ctx - lo_tile + nsplit - 1) / nsplit + BN - 1) / BN * BN;
+  const int k_begin = lo_tile + split * per, k_end = min(ctx, k_begin + per);
   const int* bt = block_table + (size_t)b * max_pages;
   const bool col_ok = col < G;
   const int head = g * G + (col_ok ? col : 0);
@@ -805,14 +835,15 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(c
   if (k_begin < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, k_begin, k_end);
   for (int tile_start = k_begin; tile_start < k_end; tile_start += BN) {
     __syncthreads();
-    regs.commit(tiles, tile_start, k_end);
+    regs.commit(tiles, tile_start, k_end, lo);
     __syncthreads();
     if (tile_start + BN < k_end) regs.fetch(k_cache, v_cache, bt, g, nkv, pshift, num_pages, tile_start + BN, k_end);
     for (int sub = wave; sub < BN / 32 && wave < 2; sub += 2) {   // waves 2 and 3 only help to move the tiles
       const int key0 = tile_start + sub * 32;
       if (key0 >= k_end) break;
-      // every query sits at position ctx - 1: only keys at or beyond k_end need the mask
-      attend_subtile(tiles, sub, qf, st, scale, key0, k_end - 1, key0 + 32 > k_end);
+      if (key0 + 32 <= lo) continue;                 // wholly before the window
+      // every query sits at position ctx - 1: only keys at or beyond k_end, or before lo, need the mask
+      attend_subtile(tiles, sub, qf, st, scale, key0, k_end - 1, key0 + 32 > k_end || key0 < lo, lo);
     }
   }
   // merge the two waves through LDS (reusing the tile memory), then write the split's partial result
@@ -871,15 +902,17 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
                                                           const int* __restrict__ block_table, int max_pages,
                                                           const int* __restrict__ context_lens,
                                                           float* __restrict__ part, int nsplit, int nq, int nkv, int P,
-                                                          int num_pages, float scale) {
+                                                          int num_pages, float scale, int reach) {
   __shared__ float xo[3][D][16];     // outputs of waves 1..3 for the final merge
   __shared__ float xml[3][2][16];
   const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
   const int G = nq / nkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
   const int ctx = context_lens[b];
-  const int per = ((ctx + nsplit - 1) / nsplit + 31) / 32 * 32;
-  const int k_begin = split * per, k_end = min(ctx, k_begin + per);
+  // the query sits at position ctx - 1 and sees keys lo .. ctx - 1; the splits share them from the block that holds lo on
+  const int lo = max(0, ctx - reach), lo_block = lo & ~31;
+  const int per = ((ctx - lo_block + nsplit - 1) / nsplit + 31) / 32 * 32;
+  const int k_begin = lo_block + split * per, k_end = min(ctx, k_begin + per);
   const int* bt = block_table + (size_t)b * max_pages;
   const bool col_ok = col < G;
   const int head = g * G + (col_ok ? col : 0);
@@ -941,19 +974,19 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
       __builtin_amdgcn_sched_barrier(0);
       load_k(next);
       __builtin_amdgcn_sched_barrier(0);
-      const bool tail = key0 + 32 > k_end;                     // the same for the whole wave
+      const bool tail = key0 + 32 > k_end || key0 < lo;        // the same for the whole wave
       float sv[8];
       float mx = -INFINITY;
 #pragma unroll
       for (int r = 0; r < 8; r++) {
         float v = (r < 4 ? s0[r & 3] : s1[r & 3]) * scale;
-        if (tail && key0 + 8 * kq + r >= k_end) v = -INFINITY;
+        if (tail && (key0 + 8 * kq + r >= k_end || key0 + 8 * kq + r < lo)) v = -INFINITY;
         sv[r] = v;
         mx = fmaxf(mx, v);
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);                        // finite: the block holds at least one key < k_end
+      const float m_new = fmaxf(m, mx);                        // finite: the block holds at least one key in lo .. k_end - 1
       const float alpha = __expf(m - m_new);
       float sum = 0.f;
 #pragma unroll
@@ -967,11 +1000,14 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
       m = m_new;
       const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack2_bf16(sv[0], sv[1]), pack2_bf16(sv[2], sv[3]),
                                                                pack2_bf16(sv[4], sv[5]), pack2_bf16(sv[6], sv[7])));
-      if (tail) {   // values of keys beyond the split hold whatever the page held before: make them zero
-        const int left = k_end - (key0 + 8 * kq);               // keys of this lane's eight that exist
+      if (tail) {   // values of keys beyond the split or before the window hold whatever the page held before: make them zero
+        const int left = k_end - (key0 + 8 * kq);               // this lane's eight keys exist below `left` ...
+        const int skip = lo - (key0 + 8 * kq);                  // ... and from `skip` on
         uint32_t keep[4];
 #pragma unroll
-        for (int w = 0; w < 4; w++) keep[w] = left >= 2 * w + 2 ? 0xffffffffu : left == 2 * w + 1 ? 0x0000ffffu : 0u;
+        for (int w = 0; w < 4; w++)
+          keep[w] = ((left >= 2 * w + 2 ? 0xffffffffu : left == 2 * w + 1 ? 0x0000ffffu : 0u) &
+                     (skip <= 2 * w ? 0xffffffffu : skip == 2 * w + 1 ? 0xffff0000u : 0u));
 #pragma unroll
         for (int tt = 0; tt < DT16; tt++) {
           vr[tt].x &= keep[0];
@@ -1117,8 +1153,10 @@ extern "C" int pico_attn_head_dim() { return D; }
 extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int* block_table, int max_pages, const int* cu_seqlens,
                                  const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
-                                 int d, int P, int num_pages, float scale, int teams, hipStream_t stream) {
+                                 int d, int P, int num_pages, float scale, int teams, int window, hipStream_t stream) {
   if (check_common("pico_attn_prefill", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
+  PICO_REQUIRE(window >= 0 && window < NO_WINDOW, "pico_attn_prefill: bad window %d", window);
+  const int reach = window > 0 ? window : NO_WINDOW;
   PICO_REQUIRE(num_seqs > 0 && num_tokens >= num_seqs, "pico_attn_prefill: bad batch (%d sequences, %d tokens)", num_seqs, num_tokens);
   PICO_REQUIRE(nq <= 65535, "pico_attn_prefill: too many heads");
   PICO_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "pico_attn_prefill: misaligned tensors");
@@ -1132,19 +1170,19 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
       grid.y = num_tokens / (2 * PF_BM) + num_seqs;
       prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 256, 0, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
-          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
     } else if (teams == 1 || PF_KT_MAX == 1)
       prefill16_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                                    (const bf16_t*)v_cache, block_table, max_pages, cu_seqlens,
-                                                   context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+                                                   context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
     else if (teams == 3 && PF_KT_MAX == 2)
       prefill16_kernel<PF_KT_MAX == 2 ? 3 : 1><<<grid, 768, 0, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
-          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
     else
       prefill16_kernel<PF_KT_MAX><<<grid, 256 * PF_KT_MAX, 0, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
-          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale);
+          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
     PICO_LAUNCH_CHECK();
     return 0;
   }
@@ -1153,7 +1191,7 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
   dim3 grid(max_tiles, nq);
   prefill_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                           block_table, max_pages, cu_seqlens, context_lens, num_seqs, (bf16_t*)out,
-                                          nq, nkv, P, num_pages, scale);
+                                          nq, nkv, P, num_pages, scale, reach);
   PICO_LAUNCH_CHECK();
   return 0;
 }
@@ -1162,8 +1200,10 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
 extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                 const int* block_table, int max_pages, const int* context_lens, int num_seqs,
                                 void* out, float* part, int nsplit, int nq, int nkv, int d, int P, int num_pages,
-                                float scale, hipStream_t stream) {
+                                float scale, int window, hipStream_t stream) {
   if (check_common("pico_attn_decode", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
+  PICO_REQUIRE(window >= 0 && window < NO_WINDOW, "pico_attn_decode: bad window %d", window);
+  const int reach = window > 0 ? window : NO_WINDOW;
   PICO_REQUIRE(nq / nkv <= 32, "pico_attn_decode: %d query heads per kv head are more than 32", nq / nkv);
   PICO_REQUIRE(num_seqs > 0 && nsplit >= 1 && nsplit <= MERGE_MAX_SPLITS && nkv <= 65535, "pico_attn_decode: bad sizes (1 to %d splits)", MERGE_MAX_SPLITS);
   PICO_REQUIRE(((uintptr_t)q % 16 == 0), "pico_attn_decode: misaligned queries");
@@ -1174,12 +1214,12 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
   if (direct)
     decode16_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                              (const bf16_t*)v_cache, block_table, max_pages, context_lens, part,
-                                             nsplit, nq, nkv, P, num_pages, scale);
+                                             nsplit, nq, nkv, P, num_pages, scale, reach);
 #endif
   if (!direct)
     decode_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                            block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
-                                           scale);
+                                           scale, reach);
   PICO_LAUNCH_CHECK();
   dim3 mgrid(num_seqs, nq);
   decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq);

@@ -66,8 +66,13 @@ class Scheduler:
         if longest > self.max_seq_len:
             raise ValueError(f"request {req.request_id}: prompt + max_new_tokens = {longest} exceeds "
                              f"max_seq_len = {self.max_seq_len}")
-        pages = -(-longest // self.manager.page_size)
+        P = self.manager.page_size
         for g in self.manager.groups:
+            pages = -(-longest // P)
+            if g.window > 0:
+                # a group with a window holds the window and the step's own tokens, whatever the length: pages that
+                # the window has passed went back before the step
+                pages = min(pages, -(-(g.window + self.max_num_batched_tokens) // P) + 1)
             if pages > g.pool.num_pages:
                 raise ValueError(f"request {req.request_id} needs {pages} pages at its longest; the pool has "
                                  f"{g.pool.num_pages}, so it could never finish")

@@ -23,13 +23,13 @@ def compute_units(device: int = 0) -> int:
 
 
 def supported(nq: int, nkv: int, head_dim: int, window: int) -> bool:
-    """Head sizes in steps of 16 up to 256, no window; anything else goes to the plain kernel."""
-    return head_dim % 16 == 0 and 16 <= head_dim <= 256 and window == 0 and nq % nkv == 0
+    """Head sizes in steps of 16 up to 256, with or without a window; anything else goes to the plain kernel."""
+    return head_dim % 16 == 0 and 16 <= head_dim <= 256 and 0 <= window < (1 << 30) and nq % nkv == 0
 
 
 class FastAttention:
-    def __init__(self, nq: int, nkv: int, head_dim: int):
-        self.nq, self.nkv, self.d = nq, nkv, head_dim
+    def __init__(self, nq: int, nkv: int, head_dim: int, window: int = 0):
+        self.nq, self.nkv, self.d, self.window = nq, nkv, head_dim, window
         self.lib = library.attention_library(head_dim)
         if self.lib.pico_attn_head_dim() != head_dim:
             raise KernelError("attention library was built for another head size")
@@ -45,9 +45,10 @@ class FastAttention:
         while padded < num_seqs:
             padded *= 2
         by_fill = max(1, 2 * self.cus // max(1, padded * self.nkv))
-        by_len = max(1, -(-max_context // 64))
+        keys = min(max_context, self.window + 31) if self.window else max_context      # what a query reads at most
+        by_len = max(1, -(-keys // 64))
         if by_len > 64:
-            by_len = max(64, -(-max_context // 128))
+            by_len = max(64, -(-keys // 128))
         return max(1, min(by_fill, by_len, 256))
 
     def prefill_teams(self, new_lens, context_lens) -> int:
@@ -61,8 +62,11 @@ class FastAttention:
         prompts, 622 against 825 us for four portions of 2,048 tokens after 2,048 with 40 heads), but coarser
         tiles, so only for much work in portions that fill them."""
         longest, total, tokens, padded = 1, 0, 0, 0
+        window = getattr(self, "window", 0)
         for n, c in zip(new_lens, context_lens):
             n, c = int(n), int(c)
+            if window:
+                c = min(c, window + n)                    # the keys that the portion's queries still see
             tiles = -(-n // 64)
             longest = max(longest, -(-c // 64))
             total += tiles * max(1, (2 * c - n) // 128)      # mean key tiles of the portion's query tiles
@@ -87,7 +91,7 @@ class FastAttention:
         _check(self.lib, self.lib.pico_attn_prefill(
             _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens), _ptr(context_lens), num_seqs, T, _ptr(out), nq, nkv, d, P, pages, c_float(scale),
-            teams, _stream()))
+            teams, self.window, _stream()))
         return out
 
     def decode(self, q: torch.Tensor, k_cache, v_cache, block_table, context_lens, num_seqs: int, scale: float,
@@ -107,7 +111,7 @@ class FastAttention:
         _check(self.lib, self.lib.pico_attn_decode(
             _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(context_lens), num_seqs, _ptr(out), _ptr(part), nsplit, nq, nkv, d, P, pages, c_float(scale),
-            _stream()))
+            self.window, _stream()))
         return out
 
     def _check_q(self, q, k_cache):
@@ -162,4 +166,4 @@ def choose(nq: int, nkv: int, head_dim: int, window: int) -> Optional[FastAttent
     take (the plain kernel then serves them)."""
     if not supported(nq, nkv, head_dim, window):
         return None
-    return FastAttention(nq, nkv, head_dim)
+    return FastAttention(nq, nkv, head_dim, window)

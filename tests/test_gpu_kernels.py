@@ -325,7 +325,8 @@ def test_sampling_top_p(K):
 
 
 # ---- matrix-core attention (bfloat16) ----------------------------------------------------------
-def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0, as_step=False):
+def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0, as_step=False,
+               window=0):
     from pico_vllm_amd.ops.attention_fast import FastAttention
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(seed)
@@ -344,7 +345,7 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
     T = sum(new_lens)
     wide = torch.zeros(T, (nq + 2 * nkv) * d, dtype=dtype, device=DEV)
     wide[:, :nq * d] = torch.cat(qs, 0).reshape(T, nq * d).to(DEV, dtype)
-    fa = FastAttention(nq, nkv, d)
+    fa = FastAttention(nq, nkv, d, window)
     scale = 1.0 / math.sqrt(d)
     if as_step:          # the way the attention part calls it: the kernels are chosen from the shape of the batch
         from types import SimpleNamespace
@@ -355,9 +356,54 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
         out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
     else:
         out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale, teams=teams)
-    want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n))
+    want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n), window=window)
                       for qb, kb, vb, n, p in zip(qs, ks, vs, new_lens, prefix_lens)], 0)
     return out.reshape(-1, nq, d), want
+
+
+@pytest.mark.parametrize("window", [1, 20, 64, 100, 129, 1000])
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(12, 2, 128, 16), (6, 3, 32, 8), (4, 1, 64, 16), (5, 5, 48, 16), (4, 1, 16, 16), (4, 2, 256, 32),
+                                        (4, 1, 96, 16)])
+def test_fast_attention_with_a_window(K, nq, nkv, d, Pg, window):
+    # only the last `window` keys count: prompt portions (the window's edge inside a key tile, at a tile's end, beyond the
+    # prefix), decode tokens with every split, a mixed step; keys before the window are made large so that one that is
+    # let in shows (their pages are what a cache manager gives back)
+    def boost(qs, ks, vs):
+        for q in qs:
+            q *= 2.0
+    new_lens, prefix_lens = [70, 1, 200, 2, 1, 130], [0, 300, 131, 63, 17, 500]
+    for teams in (1, 2, 3, 4):
+        out, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=window, boost=boost, teams=teams, window=window)
+        close(out, want, torch.bfloat16)
+    for nsplit in (1, 3, 8):
+        out, want = _fast_case([1, 1, 1, 1], [300, 17, 0, 1000], nq, nkv, d, Pg, seed=window + 1, boost=boost, decode=True,
+                               nsplit=nsplit, window=window)
+        close(out, want, torch.bfloat16)
+    out, want = _fast_case([1, 1, 40, 9], [300, 64, 100, 0], nq, nkv, d, Pg, seed=window + 2, boost=boost, as_step=True, window=window)
+    close(out, want, torch.bfloat16)
+
+
+def test_a_window_reads_nothing_before_it(K):
+    # pages before the window hold not-a-number: a kernel that let one of their keys or values into a sum would show it
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    nq, nkv, d, Pg, window = 4, 2, 64, 16, 40
+    g = torch.Generator().manual_seed(3)
+    N = 400
+    k = torch.randn(N, nkv, d, generator=g).bfloat16().float()
+    v = torch.randn(N, nkv, d, generator=g).bfloat16().float()
+    dead = N - window                                     # the one query, at position N - 1, sees keys dead .. N - 1
+    k[:dead], v[:dead] = float("nan"), float("nan")
+    kc, vc, bt = paged_cache([k], [v], Pg, N // Pg + 2, torch.bfloat16, 1, garbage=False)
+    q = torch.randn(1, nq, d, generator=g).bfloat16()
+    fa = FastAttention(nq, nkv, d, window)
+    ctxl = torch.tensor([N], dtype=torch.int32, device=DEV)
+    want = P.causal_attention(q.float(), k[dead:], v[dead:], window=window)
+    for nsplit in (1, 4):
+        out = fa.decode(q.reshape(1, -1).to(DEV), kc, vc, bt, ctxl, 1, d ** -0.5, nsplit)
+        close(out.reshape(1, nq, d), want, torch.bfloat16)
+    cu = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+    out = fa.prefill(q.reshape(1, -1).to(DEV), kc, vc, bt, cu, ctxl, 1, d ** -0.5)
+    close(out.reshape(1, nq, d), want, torch.bfloat16)
 
 
 @pytest.mark.parametrize("case", range(len(REFERENCE_CASES)))
@@ -507,8 +553,8 @@ def test_fast_attention_finds_a_far_key_among_twenty_thousand(K, far):
 
 def test_fast_kernels_refuse_what_they_cannot_do(K):
     from pico_vllm_amd.ops.attention_fast import choose, supported
-    assert choose(4, 2, 24, 0) is None and choose(4, 2, 512, 0) is None and choose(4, 2, 64, 16) is None
-    assert supported(12, 2, 128, 0)
+    assert choose(4, 2, 24, 0) is None and choose(4, 2, 512, 0) is None and choose(4, 2, 64, -1) is None
+    assert supported(12, 2, 128, 0) and supported(12, 2, 128, 4096)
 
 
 # ---- weight-streaming GEMM --------------------------------------------------------------------

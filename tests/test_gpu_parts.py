@@ -100,16 +100,17 @@ def test_attention_and_mlp_and_block_parts(name, dtype):
     close_to_plain(resid2 + whole(pending), wantb, P.block(x, plain.w, 0, cfg, pos, rnd=P.to_bf16), dtype)
 
 
+@pytest.mark.parametrize("d", [16, 64])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attention_part_with_a_window(dtype):
+def test_attention_part_with_a_window(dtype, d):
     """The same mixer class with window = 24: its cache group gives pages back, and the result is
-    the plain windowed attention."""
+    the plain windowed attention (head size 16: the 32-query matrix-core kernels in bfloat16, 64: the 16-query ones)."""
     from pico_vllm_amd.cache.manager import CacheManager
     from pico_vllm_amd.cache.storage import CacheStorage
     from pico_vllm_amd.engine.batch import BatchBuffers, SeqStep, build_context
     from pico_vllm_amd.parts.registry import build_part
     from pico_vllm_amd.parts.spec import PartSpec
-    H, nq, nkv, d, W, Pg = 96, 6, 2, 16, 24, 8
+    H, nq, nkv, W, Pg = 96, 6, 2, 24, 8
     spec = PartSpec("gqa_attention", dict(hidden_size=H, num_heads=nq, num_kv_heads=nkv, head_dim=d, qkv_bias=True,
                                           window=W, position=PartSpec("rotary_half", {"rotary_dim": d, "theta": 1e4})))
     mixer = build_part("mixer", spec, act_dtype=dtype)

@@ -176,3 +176,17 @@ def test_a_preempted_request_can_finish_while_it_waits():
     assert b.status is RequestStatus.FINISHED and list(s.waiting) == [] and s.running == [a]
     m.check()
 
+
+
+def test_a_windowed_group_is_sized_by_its_window_not_by_the_length():
+    # layers that read only the last 40 keys hold 40 + a step's tokens, whatever the length of the request: a pool
+    # of 8 pages (128 tokens) serves a request of 400 tokens, which a group without a window would refuse
+    win = {0: CacheSpec("paged_kv", num_kv_heads=1, head_dim=16, window=40)}
+    m = CacheManager(win, 16, 8, 2)
+    s = Scheduler(m, 2, 32, 512)
+    s.add_request(req(0, 300, 100))
+    order = drive(s, None)
+    assert order == [0] and m.groups[0].pool.num_free == 8 and m.groups[0].pool.peak_used <= 6
+    full, s2 = make(num_pages=8, budget=32, max_seqs=2)
+    with pytest.raises(ValueError, match="could never finish"):
+        s2.add_request(req(1, 300, 100))
