@@ -7,8 +7,12 @@
 // The draw is the inverse CDF in vocabulary order at the uniform number u[row] that the
 // host supplies (the reference calls torch.multinomial; only the distribution is shared).
 // The kept set of top-p is found without sorting: with e_i = exp((x_i - max) / T) and
-// f(t) = sum of e_i > t, the kept tokens are those with e_i >= t*, t* being the smallest
-// float with f(t*) < top_p * sum(e); t* comes from bisection over the float's bit pattern.
+// f(t) = sum of e_i > t, the kept tokens are those with e_i > t*, t* being the smallest
+// float with f(t*) < top_p * sum(e), and of the tokens with e_i == t* exactly (the token that
+// crosses, and any tied with it) the first ceil((top_p * sum - f(t*)) / t*) in vocabulary order:
+// a sort keeps a prefix of tied tokens, not all of them (sampler.py:25-32; which of them is the
+// sort's choice there, the lowest indices here, as a stable sort would).  t* comes from
+// bisection over the float's bit pattern.
 // All sums run in a fixed order, so a row's result depends on its inputs only.
 #include "common.h"
 
@@ -43,6 +47,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   __shared__ int chosen_chunk;
   __shared__ double chosen_before;
   __shared__ double chosen_target;
+  __shared__ int ties_before[SAMPLE_THREADS];   // tokens with e == thr in the chunks before a thread's own
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* x = logits + (size_t)row * ld;
   const float temp = temperature[row];
@@ -82,7 +87,12 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   }
   const float inv_t = 1.0f / temp;
   const float tp = top_p[row];
-  float thr = 0.f;  // keep e >= thr
+  float thr = 0.f;  // keep e > thr, and the first `ties_kept` tokens with e == thr
+  int ties_kept = 0x7fffffff;
+  // thread i owns a contiguous chunk of the vocabulary
+  const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int b = min(tid * chunk, V), e_ = min(b + chunk, V);
+  int my_ties_before = 0;
   if (tp < 1.0f) {
     const float total = masked_sum(x, V, mx, inv_t, -1.f, false, scratch);
     const float target = tp * total;
@@ -93,14 +103,29 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
       if (f < target) hi = mid; else lo = mid;
     }
     thr = __uint_as_float(hi);
+    // the mass above the threshold is below the target; tied tokens are taken, in vocabulary order, while
+    // the mass before them still is
+    const float above = masked_sum(x, V, mx, inv_t, thr, false, scratch);
+    ties_kept = max(1, (int)ceilf((target - above) / thr));
+    int mine = 0;
+    for (int i = b; i < e_; i++) mine += expf((x[i] - mx) * inv_t) == thr;
+    ties_before[tid] = mine;
+    __syncthreads();
+    if (tid == 0) {
+      int run = 0;
+      for (int i = 0; i < SAMPLE_THREADS; i++) { const int n = ties_before[i]; ties_before[i] = run; run += n; }
+    }
+    __syncthreads();
+    my_ties_before = ties_before[tid];
   }
-  // inverse CDF over the kept tokens in vocabulary order; thread i owns a contiguous chunk
-  const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int b = min(tid * chunk, V), e_ = min(b + chunk, V);
+  // inverse CDF over the kept tokens in vocabulary order
   double s = 0.0;
-  for (int i = b; i < e_; i++) {
-    const float e = expf((x[i] - mx) * inv_t);
-    if (e >= thr) s += (double)e;
+  {
+    int tie = my_ties_before;
+    for (int i = b; i < e_; i++) {
+      const float e = expf((x[i] - mx) * inv_t);
+      if (e > thr || (e == thr && tie++ < ties_kept)) s += (double)e;
+    }
   }
   part[tid] = s;
   __syncthreads();
@@ -125,10 +150,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   if (tid == chosen_chunk) {
     const double target = chosen_target;
     double run = chosen_before;
-    int pick = -1, last_kept = mi;
+    int pick = -1, last_kept = mi, tie = my_ties_before;
     for (int i = b; i < e_; i++) {
       const float e = expf((x[i] - mx) * inv_t);
-      if (e >= thr) {
+      if (e > thr || (e == thr && tie++ < ties_kept)) {
         last_kept = i;
         run += (double)e;
         if (run > target) { pick = i; break; }

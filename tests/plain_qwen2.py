@@ -264,9 +264,12 @@ def temperature_probs(logits: torch.Tensor, temperature: float) -> torch.Tensor:
 def top_p_probs(logits: torch.Tensor, temperature: float, top_p: float) -> torch.Tensor:
     """Sort descending, drop entries whose preceding cumulative mass is
     >= top_p (so the first token that crosses is kept), renormalise
-    (sampler.py:25-32).  Returned in vocabulary order."""
+    (sampler.py:25-32).  Returned in vocabulary order.  Of tokens with equal
+    probability a prefix in sorted order survives; which of them come first is
+    the sort's choice in the reference (torch.sort is not stable there), the
+    lowest indices here (a stable sort)."""
     probs = temperature_probs(logits, temperature)
-    sp, si = torch.sort(probs, descending=True)
+    sp, si = torch.sort(probs, descending=True, stable=True)
     cum = torch.cumsum(sp, dim=-1)
     sp = sp.masked_fill(cum - sp >= top_p, 0.0)
     sp = sp / sp.sum()

@@ -298,6 +298,22 @@ def test_sampling_temperature_follows_the_inverse_cdf(K, V):
     assert agree >= R - 3
 
 
+def test_sampling_top_p_keeps_a_prefix_of_tied_tokens(K):
+    # tokens of equal probability at the threshold: the sorted rule keeps as many of them as it takes to reach
+    # top_p, not all (pico_vllm/sampler.py:25-32); which ones is the sort's choice, here the lowest indices
+    cases = [(torch.tensor([0.2, 0.4, 0.2, 0.2]), 0.5, {1, 0}), (torch.tensor([0.2, 0.4, 0.2, 0.2]), 0.7, {1, 0, 2}),
+             (torch.tensor([0.2, 0.4, 0.2, 0.2]), 0.95, {0, 1, 2, 3}), (torch.full((100,), 0.01), 0.305, set(range(31))),
+             (torch.tensor([0.25, 0.25, 0.25, 0.25]), 0.1, {0})]
+    for probs, top_p, kept in cases:
+        logits = probs.log()[None, :].contiguous()
+        assert set(torch.nonzero(P.top_p_probs(logits[0], 1.0, top_p)).flatten().tolist()) == kept
+        seen = set()
+        for u in torch.linspace(0.001, 0.999, 97):
+            tok = K.sample(logits.to(DEV), torch.ones(1, device=DEV), torch.tensor([top_p], device=DEV), u.reshape(1).to(DEV))
+            seen.add(int(tok[0]))
+        assert seen == kept, (probs.tolist()[:5], top_p, sorted(seen))
+
+
 def test_sampling_top_p(K):
     probs = torch.tensor([[0.05, 0.5, 0.15, 0.3]])
     logits = torch.log(probs)
