@@ -25,6 +25,7 @@ class PagedKVLayer:
     v: torch.Tensor
     group: int
     page_size: int
+    read_only: bool = False    # True for a run that reads another run's cache: it attends over it and stores nothing
 
 
 @dataclass
@@ -54,8 +55,12 @@ class CacheStorage:
             else:
                 self._layers[layer] = None
 
-    def layer(self, index: int):
-        return self._layers.get(index)
+    def layer(self, index: int, read_only: bool = False):
+        """The cache of run entry ``index``; ``read_only`` for a run that was given another run's cache."""
+        entry = self._layers.get(index)
+        if read_only and isinstance(entry, PagedKVLayer):
+            return PagedKVLayer(entry.k, entry.v, entry.group, entry.page_size, read_only=True)
+        return entry
 
     def save_state(self):
         """Copies of every per-request state tensor (for ``restore_state``)."""

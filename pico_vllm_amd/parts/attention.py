@@ -1,6 +1,7 @@
 """Grouped-query attention over the paged cache."""
 from __future__ import annotations
 
+import dataclasses
 import math
 from typing import Dict, List, Optional
 
@@ -22,7 +23,9 @@ class GQAAttention(Mixer):
     :148-152, rows [q; k; v] :42-43 of weights.py, o_proj without bias :147).
     Keys and values of the new tokens are written first and attention then
     reads old and new alike from the cache (model.py:216-221), which is what
-    makes a prompt cut into portions equal the whole prompt.  The checkpoint
+    makes a prompt cut into portions equal the whole prompt.  A run that was
+    given another run's cache (``cache.read_only``) stores nothing and attends
+    over what the owner stored in the same step.  The checkpoint
     holds q_proj, k_proj and v_proj separately; they are concatenated at load.
     ``window`` > 0 restricts every query to the last ``window`` keys."""
 
@@ -77,6 +80,12 @@ class GQAAttention(Mixer):
         bt = ctx.block_tables[cache.group]
         if isinstance(x, DeferredNorm) and not getattr(self.position, "takes_deferred_norm", False):
             x = x.run()
+        if getattr(cache, "read_only", False):
+            # another run's keys and values: this run encodes its queries and attends over them; every token's slot
+            # reads as "none", which the stores of all position encodings honour
+            if "no_slots" not in ctx.shared:
+                ctx.shared["no_slots"] = torch.full_like(ctx.slot_mapping[cache.group], -1)
+            ctx = dataclasses.replace(ctx, slot_mapping=[ctx.shared["no_slots"]] * len(ctx.slot_mapping))
         # [T, >= nq d]: the encoded queries first; keys and values are in the cache after this
         qkv = self.position.project_rotate_store(x, self.qkv, ctx, cache, bt, nq, nkv, d)
         if self.fast is not None and cache.k.dtype == torch.bfloat16:

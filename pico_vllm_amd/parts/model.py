@@ -128,7 +128,9 @@ class DecoderModel:
         resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens], scale=self.spec.embed_scale)
         pending = None
         for i, e in enumerate(self.spec.run_order):
-            resid, pending = self.layers[e.layer].forward(resid, pending, ctx, storage.layer(self.spec.cache_id(i)))
+            # a run that names another run's cache reads it and stores nothing of its own
+            resid, pending = self.layers[e.layer].forward(resid, pending, ctx,
+                                                          storage.layer(self.spec.cache_id(i), read_only=e.cache_of is not None))
         if ctx.want_rows.numel() == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
         h = self.final_norm.add_norm(resid, pending, rows=ctx.want_rows)

@@ -573,3 +573,59 @@ def test_a_description_with_an_embedding_multiplier_a_head_bias_and_a_soft_cap(d
             r.advance(seq)
             i += n
         close_to_plain(torch.cat(got), exact, rounded, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_run_may_read_another_runs_cache(dtype):
+    """Run order [layer 0, layer 1 with the cache of run 0]: layer 1 projects and encodes its own queries, attends over
+    the keys and values that layer 0 stored, and stores nothing (the cache of run 0 is the model's only one).  In
+    portions and token by token the result is the plain computation of that model."""
+    import dataclasses
+    from pico_vllm_amd.config.registry import load_model_description
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import DecoderModel
+    from pico_vllm_amd.parts.spec import RunEntry
+    from pico_vllm_amd.weights.loader import load_checkpoint
+    d = model_dir("A")
+    _, cfg, spec = load_model_description(d)
+    spec = dataclasses.replace(spec, run_order=[RunEntry(0), RunEntry(1, cache_of=0)])
+    model = DecoderModel(spec, dtype, torch.device(DEV))
+    model.load(load_checkpoint(d, model.param_specs(), dtype))
+    assert sorted(model.cache_specs()) == [0]
+    r = ModelRunner(model, 16, 8, 2, 128, 128)
+    plain = P.PlainModel(d)
+    w, c = plain.w, plain.cfg
+    toks = torch.randint(0, 255, (45,), generator=torch.Generator().manual_seed(4)).tolist()
+    pos = torch.arange(len(toks))
+
+    def want(rnd):
+        nq, nkv, hd = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+        x = w["model.embed_tokens.weight"][toks].float()
+        kv = None
+        for i in (0, 1):
+            p = f"model.layers.{i}"
+            h = rnd(P.rms_norm(x, w[f"{p}.input_layernorm.weight"], c.rms_norm_eps))
+            W = torch.cat([w[f"{p}.self_attn.{n}_proj.weight"] for n in "qkv"])
+            b = torch.cat([w[f"{p}.self_attn.{n}_proj.bias"] for n in "qkv"])
+            q, k, v = P.split_qkv(rnd(h @ W.T + b), nq, nkv, hd)
+            cos, sin = P.rope_tables(pos, hd, c.rope_theta)
+            q, k = rnd(P.apply_rope(q, cos, sin)), rnd(P.apply_rope(k, cos, sin))
+            if i == 0:
+                kv = (k, v)                      # what run 0 stores is what run 1 reads
+            o = rnd(P.causal_attention(q, kv[0], kv[1], rnd_p=None if rnd is P._same else rnd))
+            x = x + rnd(o.reshape(len(toks), nq * hd) @ w[f"{p}.self_attn.o_proj.weight"].T)
+            x = x + P.mlp_layer(rnd(P.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], c.rms_norm_eps)), w, p, rnd)
+        return rnd(P.rms_norm(x, w["model.norm.weight"], c.rms_norm_eps)) @ w["model.embed_tokens.weight"].T
+    exact, rounded = want(P._same), want(P.to_bf16)
+    ordinary = plain.logits(toks)
+    assert float((exact - ordinary).abs().max()) > 0.05 * float(ordinary.std())       # it is another model than the ordinary one
+    r.manager.add_request("r")
+    got, i = [], 0
+    for n in (20, 3, 1, 1, 20):
+        assert r.manager.grow("r", i + n)
+        seq = [SeqStep("r", toks[i:i + n], list(range(n)))]
+        got.append(r.step(seq))
+        r.advance(seq)
+        i += n
+    close_to_plain(torch.cat(got), exact, rounded, dtype)
