@@ -23,7 +23,15 @@ def register_part(category: str, kind: str, cls=None):
     return _put if cls is None else _put(cls)
 
 
+def _register_own_parts() -> None:
+    """The parts of this package register themselves when their modules load; whoever asks the registry first
+    makes sure they have."""
+    from . import attention, block, mlp, norm, rotary  # noqa: F401
+
+
 def part_class(category: str, kind: str):
+    if kind not in _REGISTRY.get(category, {}):
+        _register_own_parts()
     try:
         return _REGISTRY[category][kind]
     except KeyError:

@@ -629,3 +629,84 @@ def test_a_run_may_read_another_runs_cache(dtype):
         r.advance(seq)
         i += n
     close_to_plain(torch.cat(got), exact, rounded, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layers_with_and_without_a_window_in_one_model(dtype):
+    """Layer 0 reads the last 24 keys only, layers 1 and 2 all of them: two groups of layers with pages of their own, the
+    windowed group giving pages back while the request runs.  A request of 120 tokens in portions and token by token,
+    and a second one beside it, in pools so small that the windowed group's pages are used again; against the plain
+    computation of that model."""
+    import dataclasses
+    import tempfile
+    from pico_vllm_amd.config.model_config import Qwen2Config
+    from pico_vllm_amd.config.qwen2 import qwen2_spec
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.spec import LayerSpec, PartSpec
+    from pico_vllm_amd.weights.random_init import write_random_model
+    from tiny_configs import TINY_B, strong
+    W = 24
+
+    def spec_with_window(cfg):
+        spec = qwen2_spec(cfg)
+        l0 = spec.layers[0]
+        name, attn = l0.slots["mixer"]
+        windowed = PartSpec(attn.kind, dict(attn.params, window=W))
+        return dataclasses.replace(spec, layers=[LayerSpec(l0.prefix, l0.block, {**l0.slots, "mixer": (name, windowed)})] + list(spec.layers[1:]))
+    register_architecture("ToyWindowFirstLM", Qwen2Config.from_dict, spec_with_window)
+    cfg = dict(TINY_B, architectures=["ToyWindowFirstLM"])
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=8, std_overrides=strong(cfg))
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        r = ModelRunner(model, 8, 20, 2, 64, 160)          # 20 pages of 8 a group: 160 tokens, two requests of 120 + 30 need the give-back
+        m = r.manager
+        assert len(m.groups) == 2 and sorted(g.window for g in m.groups) == [0, W]
+        plain = P.PlainModel(d)
+        w, c = plain.w, plain.cfg
+
+        def want(toks, rnd):
+            nq, nkv, hd = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+            pos = torch.arange(len(toks))
+            x = w["model.embed_tokens.weight"][toks].float()
+            for i in range(c.num_hidden_layers):
+                p = f"model.layers.{i}"
+                h = rnd(P.rms_norm(x, w[f"{p}.input_layernorm.weight"], c.rms_norm_eps))
+                Wm = torch.cat([w[f"{p}.self_attn.{n}_proj.weight"] for n in "qkv"])
+                b = torch.cat([w[f"{p}.self_attn.{n}_proj.bias"] for n in "qkv"])
+                q, k, v = P.split_qkv(rnd(h @ Wm.T + b), nq, nkv, hd)
+                cos, sin = P.rope_tables(pos, hd, c.rope_theta)
+                q, k = rnd(P.apply_rope(q, cos, sin)), rnd(P.apply_rope(k, cos, sin))
+                o = rnd(P.causal_attention(q, k, v, window=W if i == 0 else 0, rnd_p=None if rnd is P._same else rnd))
+                x = x + rnd(o.reshape(len(toks), nq * hd) @ w[f"{p}.self_attn.o_proj.weight"].T)
+                x = x + P.mlp_layer(rnd(P.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], c.rms_norm_eps)), w, p, rnd)
+            return rnd(P.rms_norm(x, w["model.norm.weight"], c.rms_norm_eps)) @ w["lm_head.weight"].T
+        g = torch.Generator().manual_seed(9)
+        a, b = torch.randint(0, 383, (120,), generator=g).tolist(), torch.randint(0, 383, (30,), generator=g).tolist()
+        assert float((want(a, P._same) - plain.logits(a)).abs().max()) > 0.05 * float(plain.logits(a).std())   # the window matters
+        m.add_request("a")
+        m.add_request("b")
+        got = {"a": [], "b": []}
+        fed = {"a": 0, "b": 0}
+        plan = [(40, 0), (13, 7), (1, 1), (1, 1), (30, 2), (1, 19), (34, 0)]
+        for na, nb in plan:
+            seqs = []
+            for rid, n, toks in (("a", na, a), ("b", nb, b)):
+                if n:
+                    assert m.grow(rid, fed[rid] + n)
+                    seqs.append(SeqStep(rid, toks[fed[rid]:fed[rid] + n], list(range(n))))
+            out = r.step(seqs)
+            r.advance(seqs)
+            o = 0
+            for s in seqs:
+                got[s.req].append(out[o:o + len(s.tokens)])
+                o += len(s.tokens)
+                fed[s.req] += len(s.tokens)
+            m.check()
+        assert fed == {"a": 120, "b": 30}
+        windowed = [gr for gr in m.groups if gr.window][0]
+        assert windowed.pool.peak_used < 20 and windowed.pool.num_used < [gr for gr in m.groups if not gr.window][0].pool.num_used
+        for rid, toks in (("a", a), ("b", b)):
+            close_to_plain(torch.cat(got[rid]), want(toks, P._same), want(toks, P.to_bf16), dtype)
