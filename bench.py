@@ -201,6 +201,37 @@ def prefill_point(model_dir, model, dtype, reps=7):
     return out
 
 
+def sweep_point(model_dir, model, dtype, batch, bin_width=256):
+    """Decode from a prompt of 16 tokens up to the context length, an event behind every step: the median time of a
+    step for every `bin_width` positions of context (the reference sweeps sequence lengths 16 to 4096 this way,
+    pico_vllm/profiling/profile_pagedkvcacheTritoncompile.py:43-113, for its successive engines)."""
+    import torch
+    eng = make_engine(model_dir, dtype, batch, model)
+    V = CONFIG["vocab_size"]
+    g = torch.Generator().manual_seed(11)
+    new = CONTEXT - 16
+    for _ in range(batch):
+        eng.submit(torch.randint(0, V, (16,), generator=g).tolist(), max_new_tokens=new, temperature=0.0, ignore_eos=True)
+    eng.step()                                        # the prompts
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True)]
+    marks[0].record()
+    while not eng.is_done():
+        eng.step()
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        marks.append(e)
+    torch.cuda.synchronize()
+    ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(len(marks) - 1)]
+    rows = []
+    for lo in range(0, len(ms), bin_width):
+        part = sorted(ms[lo:lo + bin_width])
+        if len(part) >= bin_width // 2:
+            med = part[len(part) // 2]
+            rows.append({"context": 16 + lo + len(part) // 2, "ms_per_step": round(med, 4), "tok_s": round(batch / med * 1e3, 1)})
+    return rows
+
+
 def long_prompt_point(model_dir, model, dtype, prompt_len):
     """One prompt of ``prompt_len`` tokens through the scheduler, cut into portions of PREFILL_TOKENS; the time
     until its first token is sampled."""
@@ -323,9 +354,10 @@ def main() -> int:
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
     ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "sweep"],
                     help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once; "
-                         "long: one prompt of --prompt tokens in portions, then decode at batch 1 and 8 at the context length")
+                         "long: one prompt of --prompt tokens in portions, then decode at batch 1 and 8 at the context length; "
+                         "sweep: decode from context 16 to the context length, the time of a step by context")
     ap.add_argument("--prompt", type=int, default=16384, help="prompt tokens of the long workload")
     ap.add_argument("--device-weights", action="store_true",
                     help="draw the random weights on the GPU instead of writing and reading a model folder")
@@ -401,6 +433,12 @@ def main() -> int:
             return 0
         if a.prefill_only:
             print(json.dumps({"prefill": prefill_point(model_dir, preloaded, a.dtype)}), flush=True)
+            return 0
+        if a.workload == "sweep":
+            rows = sweep_point(model_dir, preloaded, a.dtype, a.batch)
+            print(json.dumps({"metric": f"decode ms/step by context, batch {a.batch}, {shape_name.split()[0]} {a.dtype}",
+                              "unit": "ms", "n_gpus": 1, "batch": a.batch, "layers_run": CONFIG["num_hidden_layers"],
+                              "layers": full["num_hidden_layers"], "rows": rows}), flush=True)
             return 0
         if a.workload == "long":
             if a.prompt + 8 > CONTEXT:

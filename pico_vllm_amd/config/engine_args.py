@@ -29,6 +29,7 @@ class EngineArgs:
     manual_seed: int = 42
     pipeline_decode: bool = True         # keep one decode step in flight while the host prepares the next
     tune_library_gemm: bool = False      # let the library time its solutions for whole prompt portions (stalls the first such step)
+    profile_phases: bool = False         # time the phases of every step (host clock and device events) and mark them for a profiler
     device: str = "cuda:0"
 
     def validate(self) -> None:

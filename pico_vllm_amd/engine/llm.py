@@ -19,6 +19,7 @@ from ..parts.model import DecoderModel, load_model
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import SeqStep
+from .phases import PhaseTimers
 from .request import Request, RequestStatus
 from .scheduler import Scheduler
 from .step import ModelRunner
@@ -67,6 +68,7 @@ class LLMEngine:
         self._next_id = 0
         self.requests: Dict[int, Request] = {}
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+        self.timers = PhaseTimers(args.profile_phases)
         self._inflight: Optional[_Inflight] = None      # a launched step whose tokens have not been read
 
     # ---- the reference's trio -------------------------------------------
@@ -100,7 +102,8 @@ class LLMEngine:
         plan = None
         if prev is not None:
             if self._foreseeable(prev):
-                plan = self.scheduler.schedule()
+                with self.timers.phase("schedule"):
+                    plan = self.scheduler.schedule()
                 if not plan.preempted and [s.request for s in plan.seqs] == [s.request for s in prev.sampling] \
                         and all(s.num_tokens == 1 for s in plan.seqs):
                     nxt = self._launch(plan, from_device=True)
@@ -112,7 +115,8 @@ class LLMEngine:
             if plan is not None:
                 plan.seqs = [s for s in plan.seqs if s.request.status is RequestStatus.RUNNING]
         if plan is None:
-            plan = self.scheduler.schedule()
+            with self.timers.phase("schedule"):
+                plan = self.scheduler.schedule()
         self.stats["preemptions"] += len(plan.preempted)
         if not plan.seqs:
             if self.scheduler.has_unfinished():
@@ -149,12 +153,14 @@ class LLMEngine:
             r = s.request
             toks = [0] if from_device else r.all_ids[r.num_computed:r.num_computed + s.num_tokens]
             seqs.append(SeqStep(r.request_id, toks, [s.num_tokens - 1] if s.samples else []))
-        logits = self.runner.step(seqs, self.sampler.device_tokens if from_device else None)
+        with self.timers.phase("model", device=True):
+            logits = self.runner.step(seqs, self.sampler.device_tokens if from_device else None)
         sampling = [s for s in plan.seqs if s.samples]
-        ticket = self.sampler.launch(
-            logits,
-            [s.request.params.temperature for s in sampling], [s.request.params.top_p for s in sampling],
-            [s.request.seed for s in sampling], [s.request.num_generated for s in sampling])
+        with self.timers.phase("sample", device=True):
+            ticket = self.sampler.launch(
+                logits,
+                [s.request.params.temperature for s in sampling], [s.request.params.top_p for s in sampling],
+                [s.request.seed for s in sampling], [s.request.num_generated for s in sampling])
         for s in plan.seqs:
             self.stats["decode_tokens" if s.num_tokens == 1 and s.request.num_generated else "prefill_tokens"] += s.num_tokens
             self.scheduler.on_step_done(s)
@@ -166,7 +172,9 @@ class LLMEngine:
     def _resolve(self, step: "_Inflight") -> List[RequestOutput]:
         """Read the tokens of a launched step and finish what they finish."""
         done: List[RequestOutput] = []
-        for s, tok in zip(step.sampling, self.sampler.read(step.ticket)):
+        with self.timers.phase("read"):
+            tokens = self.sampler.read(step.ticket)
+        for s, tok in zip(step.sampling, tokens):
             r = s.request
             if r.status is RequestStatus.FINISHED:      # ended by the token before this one: computed too many
                 continue
@@ -185,6 +193,19 @@ class LLMEngine:
                 self.scheduler.finish(r, reason)
                 done.append(self._output(r))
         return done
+
+    # ---- counters -------------------------------------------------------
+    def report(self) -> Dict[str, object]:
+        """Counters of the engine: steps, prompt and decoded tokens, preemptions, pages in use and at the peak per
+        group of layers, and, with ``profile_phases``, the time of every phase."""
+        m = self.runner.manager
+        out: Dict[str, object] = dict(self.stats)
+        out["pages"] = [{"window": g.window, "layers": len(g.layers), "total": g.pool.num_pages, "in_use": g.pool.num_used,
+                         "peak": g.pool.peak_used, "reused": g.pool.reuse_count} for g in m.groups]
+        out["graphs"] = sorted(self.runner._graphs)
+        if self.timers.enabled:
+            out["phases"] = self.timers.report()
+        return out
 
     # ---- helpers --------------------------------------------------------
     def _encode(self, prompt) -> List[int]:

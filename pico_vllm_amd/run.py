@@ -44,6 +44,8 @@ def main(argv=None) -> int:
                     "(tiny-a, tiny-b, 1.5b, 7b, 32b) instead of --model; with --write-random: that size")
     ap.add_argument("--no-pipeline-decode", dest="pipeline_decode", action="store_false", default=True,
                     help="read every step's tokens before the next step starts")
+    ap.add_argument("--profile-phases", action="store_true",
+                    help="time the phases of every step, mark them for rocprofv3 --marker-trace, and print the report to stderr")
     args = ap.parse_args(argv)
 
     if args.write_random:
@@ -95,12 +97,14 @@ def _generate(ap, args) -> int:
                     num_gpu_blocks=args.num_gpu_blocks, max_seq_len=args.max_seq_len,
                     max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
                     use_cuda_graph=args.use_cuda_graph, max_batch_size=args.max_batch_size,
-                    manual_seed=args.manual_seed, pipeline_decode=args.pipeline_decode)
+                    manual_seed=args.manual_seed, pipeline_decode=args.pipeline_decode, profile_phases=args.profile_phases)
     llm = LLM(tokenizer=tokenizer, engine_args=ea)
     sp = SamplingParams(args.max_new_tokens, args.temperature, args.top_p, args.seed, args.ignore_eos)
     for o in llm.generate(prompts, sp):
         shown = o.text if o.text is not None else " ".join(map(str, o.token_ids))
         print(f"[{o.request_id}] ({o.finish_reason}) {shown}")
+    if args.profile_phases:
+        print(json.dumps(llm.engine.report(), indent=1), file=sys.stderr)
     return 0
 
 

@@ -265,3 +265,21 @@ def test_a_finished_request_leaves_the_engine():
     eng = llm("A", "float32")
     eng.generate(prompts_for("A", [5, 9, 3]), SamplingParams(max_new_tokens=4, ignore_eos=True))
     assert eng.engine.requests == {} and not eng.engine.runner.manager.requests
+
+
+def test_phase_timers_behind_their_flag_change_nothing():
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("A", [5, 30, 11], seed=6)
+    sp = SamplingParams(max_new_tokens=12, temperature=0.0, ignore_eos=True)
+    plain_run = llm("A", "bfloat16", use_cuda_graph=True, max_batch_size=4)
+    timed = llm("A", "bfloat16", use_cuda_graph=True, max_batch_size=4, profile_phases=True)
+    a, b = plain_run.generate(prompts, sp), timed.generate(prompts, sp)
+    assert [o.token_ids for o in a] == [o.token_ids for o in b]
+    assert "phases" not in plain_run.engine.report()
+    rep = timed.engine.report()
+    steps = rep["steps"]
+    assert steps >= 12 and rep["decode_tokens"] > 0 and rep["prefill_tokens"] == 46
+    assert rep["phases"]["model"]["calls"] == steps == rep["phases"]["sample"]["calls"]
+    assert rep["phases"]["model"]["device_ms"] > 0 and rep["phases"]["model"]["host_ms_per_call"] > 0
+    assert rep["phases"]["schedule"]["calls"] >= steps and rep["phases"]["read"]["calls"] == steps
+    assert rep["pages"][0]["in_use"] == 0 and rep["pages"][0]["peak"] > 0 and rep["graphs"]
