@@ -265,7 +265,7 @@ def prefill_flops_long(cfg, T):
     return prefill_flops(cfg, T)
 
 
-def serve_point(model_dir, dtype, requests, max_new):
+def serve_point(model_dir, dtype, requests, max_new, model=None):
     """The mixed workload: `requests` requests with prompt lengths uniform in 128..4096 (seeded) and
     `max_new` new tokens each, all submitted at once; the scheduler admits, cuts prompts into portions of at most
     2,048 tokens beside the decoding requests, decodes, finishes and frees."""
@@ -281,7 +281,7 @@ def serve_point(model_dir, dtype, requests, max_new):
     pages = sum(-(-(n + max_new) // block) for n in lens) + 8
     eng = LLMEngine(EngineArgs(model=model_dir, dtype=dtype, block_size=block, num_gpu_blocks=pages, max_seq_len=CONTEXT,
                                max_num_seqs=requests, max_num_batched_tokens=PREFILL_TOKENS, use_cuda_graph=True,
-                               max_batch_size=64, tune_library_gemm=True))
+                               max_batch_size=64, tune_library_gemm=True), model=model)
     V = CONFIG["vocab_size"]
     # a short run first: kernels built and tuned, graphs captured for the batch sizes of the run's tail
     for n in (PREFILL_TOKENS, 300):
@@ -398,9 +398,6 @@ def main() -> int:
     model_dir = a.model
     preloaded = None
     if a.device_weights:
-        if a.workload == "serve":
-            print("bench.py: --device-weights serves the decode and long workloads")
-            return 2
         t0 = time.time()
         log(f"drawing random weights of the {shape_name}, {CONFIG['num_hidden_layers']} layers, on the GPU ...")
         preloaded = device_model(CONFIG, a.dtype)
@@ -416,7 +413,7 @@ def main() -> int:
         log(f"... {time.time() - t0:.0f}s")
     try:
         if a.workload == "serve":
-            r = serve_point(model_dir, a.dtype, a.requests, a.max_new)
+            r = serve_point(model_dir, a.dtype, a.requests, a.max_new, preloaded)
             total = r["prompt_tokens"] + r["new_tokens"]
             print(json.dumps({
                 "metric": f"tokens/s (prompt + new) serving {a.requests} requests at once, {shape_name.split()[0]} bf16",
