@@ -171,6 +171,7 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
 def prefill_point(model_dir, model, dtype, reps=7):
     import torch
     from pico_vllm_amd.engine.batch import SeqStep
+    peak = measured_peaks()[1] if dtype == "bfloat16" else None       # before the timed steps: a profile ends with them
     eng = make_engine(model_dir, dtype, 1, model)
     V = CONFIG["vocab_size"]
     ids = torch.randint(0, V, (PREFILL_TOKENS,), generator=torch.Generator().manual_seed(7)).tolist()
@@ -194,8 +195,7 @@ def prefill_point(model_dir, model, dtype, reps=7):
     flops = prefill_flops(CONFIG, PREFILL_TOKENS)
     out = {"value": PREFILL_TOKENS / dt, "tokens": PREFILL_TOKENS, "ms": dt * 1e3, "ms_min": times[0] * 1e3,
            "tflops": flops / dt / 1e12, "frac": flops / dt / MFMA_PEAK[dtype]}
-    if dtype == "bfloat16":
-        peak = measured_peaks()[1]
+    if peak is not None:
         out["measured_peak_tflops"] = peak / 1e12
         out["frac_of_measured"] = flops / dt / peak
     return out
