@@ -47,22 +47,36 @@ class BatchBuffers:
 
 
 def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers, act_dtype: torch.dtype,
-                  vocab_size: int, pad_to: Optional[int] = None) -> StepContext:
+                  vocab_size: int, pad_to: Optional[int] = None, pad_tokens_to: Optional[int] = None) -> StepContext:
     """Pack ``seqs`` into ``buf`` and describe the device views.
 
     ``pad_to``: pad a pure-decode batch with empty rows up to that many
     sequences (for replaying a graph captured at that size); a padded row has a
     block table of -1 and a context of 0, so nothing is written for it, its state slot is
     the spare one behind the requests' slots, and its output is ignored.
+    ``pad_tokens_to``: bring the step to that many tokens (for replaying a graph of a prompt step
+    recorded at that size) with one more sequence of filler tokens behind the given ones: positions
+    from 0, a context of its own length, a block table of -1, slots of -1, the spare state slot,
+    nothing wanted; it may be empty.
     """
     B = len(seqs)
     if B == 0:
         raise BatchError("a step needs at least one sequence")
-    rows = max(B, pad_to or 0)
+    if pad_to and pad_tokens_to:
+        raise BatchError("a step is padded with rows or with tokens, not with both")
     lens = [len(s.tokens) for s in seqs]
     if min(lens) < 1:
         raise BatchError("every sequence of a step brings at least one token")
-    T = sum(lens) + (rows - B)
+    filler = 0
+    if pad_tokens_to is not None:
+        filler = pad_tokens_to - sum(lens)
+        if filler < 0:
+            raise BatchError(f"the step has {sum(lens)} tokens, more than the {pad_tokens_to} it is to be padded to")
+        rows = B + 1
+        T = pad_tokens_to
+    else:
+        rows = max(B, pad_to or 0)
+        T = sum(lens) + (rows - B)
     R = sum(len(s.want) for s in seqs) + (rows - B if pad_to else 0)
     P = manager.page_size
     if T > buf.max_tokens or rows > buf.max_seqs or R > buf.max_want:
@@ -124,14 +138,22 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         h_slot[b] = manager.slot(s.req)
         max_ctx = max(max_ctx, cached + n)
         need_pages = max(need_pages, -(-(cached + n) // P))
-    for b in range(B, rows):                       # padding rows of a captured decode batch
-        h_tok[t] = 0; h_pos[t] = 0; h_seq[t] = b
-        h_want[r] = t; r += 1
-        t += 1
-        h_cu[b + 1] = t
-        h_ctx[b] = 0
-        h_slot[b] = manager.slots.num_slots       # the spare slot that no request ever holds
-    width = buf.max_pages if pad_to else need_pages
+    if pad_tokens_to is not None:                  # the sequence of filler tokens of a recorded prompt step
+        h_tok[t:T] = 0
+        h_pos[t:T] = np.arange(filler)
+        h_seq[t:T] = B
+        h_cu[B + 1] = T
+        h_ctx[B] = filler
+        h_slot[B] = manager.slots.num_slots
+    else:
+        for b in range(B, rows):                   # padding rows of a captured decode batch
+            h_tok[t] = 0; h_pos[t] = 0; h_seq[t] = b
+            h_want[r] = t; r += 1
+            t += 1
+            h_cu[b + 1] = t
+            h_ctx[b] = 0
+            h_slot[b] = manager.slots.num_slots   # the spare slot that no request ever holds
+    width = buf.max_pages if (pad_to or pad_tokens_to is not None) else need_pages
     if width > buf.max_pages:
         raise BatchError(f"a sequence needs {width} pages, the buffers hold {buf.max_pages} per sequence")
     tables = h[bt_off:bt_off + G * rows * width].reshape(G, rows, width)
@@ -163,7 +185,7 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         block_tables=[d[bt_off + g * rows * width:bt_off + (g + 1) * rows * width].view(rows, width) for g in range(G)],
         slot_mapping=[d[(3 + g) * buf.max_tokens:(3 + g) * buf.max_tokens + T] for g in range(G)],
         act_dtype=act_dtype,
-        max_new_tokens=max(lens), max_context=max_ctx, all_decode=max(lens) == 1,
+        max_new_tokens=max(lens), max_context=max_ctx, all_decode=max(lens) == 1 and pad_tokens_to is None,
         host={"cu_seqlens": h_cu.copy(), "context_lens": h_ctx.copy()},
     )
     return ctx

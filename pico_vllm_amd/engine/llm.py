@@ -57,7 +57,8 @@ class LLMEngine:
             num_pages = args.max_num_seqs * (-(-args.max_seq_len // args.block_size))
         self.runner = ModelRunner(self.model, args.block_size, num_pages, args.max_num_seqs,
                                   args.max_num_batched_tokens, args.max_seq_len,
-                                  use_graph=args.use_cuda_graph, max_graph_batch=args.max_batch_size)
+                                  use_graph=args.use_cuda_graph, max_graph_batch=args.max_batch_size,
+                                  graph_prompts=args.graph_prompts)
         self.scheduler = Scheduler(self.runner.manager, args.max_num_seqs, args.max_num_batched_tokens,
                                    args.max_seq_len)
         self.sampler = Sampler(self.model.device, args.max_num_seqs)
@@ -203,6 +204,7 @@ class LLMEngine:
         out["pages"] = [{"window": g.window, "layers": len(g.layers), "total": g.pool.num_pages, "in_use": g.pool.num_used,
                          "peak": g.pool.peak_used, "reused": g.pool.reuse_count} for g in m.groups]
         out["graphs"] = sorted(self.runner._graphs)
+        out["prompt_graphs"] = sorted(size for size, _ in self.runner._prompt_graphs)
         if self.timers.enabled:
             out["phases"] = self.timers.report()
         return out

@@ -8,7 +8,11 @@ together (:403-410) through two different model entry points.
 
 A pure-decode step whose batch fits ``max_batch_size`` replays a HIP graph
 captured for its size (the reference captures one CUDA graph at a fixed batch
-of 8, engine.py:98-137).
+of 8, engine.py:98-137).  A step that is one prompt portion alone replays a
+graph too, recorded at the next of a few sizes and padded to it with filler
+tokens in a sequence of their own: such a step is a few hundred launches and
+library calls that cost the host more than they cost the GPU (4.1 ms against
+1.6 ms for 300 tokens of the 1.5B shape).
 """
 from __future__ import annotations
 
@@ -29,9 +33,21 @@ def _bucket(n: int) -> int:
     return b
 
 
+def prompt_sizes(most: int) -> List[int]:
+    """The sizes at which prompt steps are recorded: 16, 32, 64, then steps of 64 to 512, of 128 to 1,024 and of
+    256 beyond, up to ``most``: at most a quarter of a recorded step is filler, beyond 64 tokens an eighth."""
+    out = [16, 32]
+    n = 64
+    while n <= most:
+        out.append(n)
+        n += 64 if n < 512 else 128 if n < 1024 else 256
+    return [s for s in out if s <= most]
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_size: int, num_pages: int, max_seqs: int,
-                 max_tokens_per_step: int, max_seq_len: int, use_graph: bool = False, max_graph_batch: int = 8):
+                 max_tokens_per_step: int, max_seq_len: int, use_graph: bool = False, max_graph_batch: int = 8,
+                 graph_prompts: bool = True):
         self.model = model
         self.device = model.device
         specs = model.cache_specs()
@@ -40,13 +56,17 @@ class ModelRunner:
         self.max_pages = -(-max_seq_len // page_size)
         self.max_seq_len = max_seq_len
         # a decode batch is padded to the power of two its graph was captured at: rows for that too
-        rows = max(max_seqs, _bucket(min(max_seqs, max_graph_batch))) if use_graph else max_seqs
+        # (and a recorded prompt step has a second sequence, of filler)
+        rows = max(max_seqs, _bucket(min(max_seqs, max_graph_batch)), 2) if use_graph else max_seqs
         self.buffers = BatchBuffers(self.device, max(max_tokens_per_step, rows), rows, self.max_pages,
                                     max(1, len(self.manager.groups)))
         # a part that decides on the host per step (``Part.graph_safe`` False) keeps the whole model out of graphs
         self.use_graph = use_graph and model.is_graph_safe()
+        self.graph_prompts = self.use_graph and graph_prompts and model.is_graph_safe(prompts=True)
+        self.prompt_sizes = prompt_sizes(min(max_tokens_per_step, self.max_pages * page_size))
         self.max_graph_batch = max_graph_batch
         self._graphs: Dict[int, tuple] = {}
+        self._prompt_graphs: Dict[tuple, tuple] = {}       # (recorded size, wanted rows) -> (graph, logits)
         self.steps = 0
         self.tokens = 0
 
@@ -80,8 +100,11 @@ class ModelRunner:
                     at += len(seqs[i].want)
                 back = [first_row[i] + j for i in range(len(seqs)) for j in range(len(seqs[i].want))]
                 seqs = [seqs[i] for i in order]
+        size = self._prompt_size(seqs) if self.graph_prompts and not decode_only else 0
         if self.use_graph and decode_only and len(seqs) <= self.max_graph_batch:
             logits = self._step_graph(seqs, device_tokens)
+        elif size:
+            logits = self._step_prompt_graph(seqs[0], size)
         else:
             ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size)
             if decode_only:
@@ -115,13 +138,40 @@ class ModelRunner:
         graph.replay()
         return out[:B]
 
+    # ---- graph replay of a prompt portion alone ---------------------------
+    def _prompt_size(self, seqs: List[SeqStep]) -> int:
+        """The recorded size that serves this step, or 0: one sequence of two tokens or more, at most one wanted
+        row, and room in the block table for the filler's positions."""
+        if len(seqs) != 1 or len(seqs[0].tokens) < 2 or len(seqs[0].want) > 1:
+            return 0
+        n = len(seqs[0].tokens)
+        for size in self.prompt_sizes:
+            if size >= n:
+                fits = self.manager.num_computed(seqs[0].req) + size <= self.max_pages * self.manager.page_size
+                return size if fits else 0
+        return 0
+
+    def _step_prompt_graph(self, seq: SeqStep, size: int) -> torch.Tensor:
+        key = (size, len(seq.want))
+        if key not in self._prompt_graphs:
+            ctx = build_context([seq], self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
+                                pad_tokens_to=size)
+            self._prompt_graphs[key] = self._record(ctx)
+        graph, out = self._prompt_graphs[key]
+        build_context([seq], self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size, pad_tokens_to=size)
+        graph.replay()
+        return out
+
     def _capture(self, size: int, seqs: List[SeqStep]) -> None:
-        """Warm up on the real batch, then record the graph.  The warm-up runs write this step's keys and
-        values, which the replay that follows writes again with the same values; per-request state, which
-        a run changes from what it was, is put back afterwards so that only the replay counts."""
         ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
                             pad_to=size)
         ctx.max_context = self.max_seq_len          # kernel choices must hold for every later replay
+        self._graphs[size] = self._record(ctx)
+
+    def _record(self, ctx) -> tuple:
+        """Warm up on the real batch, then record the graph.  The warm-up runs write this step's keys and
+        values, which the replay that follows writes again with the same values; per-request state, which
+        a run changes from what it was, is put back afterwards so that only the replay counts."""
         saved = self.storage.save_state()
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream())
@@ -134,7 +184,7 @@ class ModelRunner:
         with torch.cuda.graph(graph):
             out = self.model.forward(ctx, self.storage)
         self.storage.restore_state(saved)
-        self._graphs[size] = (graph, out)
+        return graph, out
 
     # ---- sizes for reports ----------------------------------------------
     def decode_bytes(self, context_lens: List[int]) -> int:

@@ -30,6 +30,7 @@ class GQAAttention(Mixer):
     ``window`` > 0 restricts every query to the last ``window`` keys."""
 
     takes_deferred_norm = True
+    graph_safe_prompts = True       # the shape of the prefill workgroups is a hint taken from the recorded step
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, position: PartSpec, window: int = 0,

@@ -56,12 +56,20 @@ class Part:
     ``graph_safe``: whether the part's work in a decode step is fixed once the step's shape is (device work only,
     nothing decided from values on the host, no synchronisation), so that the step may be recorded into a HIP graph
     and replayed.  A part that reads ``ctx.host`` or copies values to the host per step sets it to False; a model
-    with such a part anywhere never runs from a graph, whatever the engine's options say."""
-    graph_safe = True
+    with such a part anywhere never runs from a graph, whatever the engine's options say.
 
-    def is_graph_safe(self) -> bool:
+    ``graph_safe_prompts``: the same for a step that is one prompt portion, which is recorded padded: behind the
+    portion's sequence stands a second one of filler tokens (slot -1, a block table of -1, outputs ignored) that
+    brings the step to a recorded size.  A part that says True does device work only in such a step, may take what
+    it decides on the host from the step that was recorded (``ctx.host`` is that step's), and keeps nothing of the
+    filler.  The default is False: prompt steps of a model with such a part run unrecorded."""
+    graph_safe = True
+    graph_safe_prompts = False
+
+    def is_graph_safe(self, prompts: bool = False) -> bool:
         """This part and the parts it is built from."""
-        return self.graph_safe and all(p.is_graph_safe() for p in vars(self).values() if isinstance(p, Part))
+        own = self.graph_safe_prompts if prompts else self.graph_safe
+        return own and all(p.is_graph_safe(prompts) for p in vars(self).values() if isinstance(p, Part))
 
     def param_specs(self) -> List[ParamSpec]:
         return []
@@ -149,8 +157,9 @@ class Block(Part):
     def __init__(self, parts: Dict[str, Part]):
         self.parts = parts
 
-    def is_graph_safe(self) -> bool:
-        return self.graph_safe and all(p.is_graph_safe() for p in self.parts.values())
+    def is_graph_safe(self, prompts: bool = False) -> bool:
+        own = self.graph_safe_prompts if prompts else self.graph_safe
+        return own and all(p.is_graph_safe(prompts) for p in self.parts.values())
 
     @property
     def mixer(self) -> Mixer:

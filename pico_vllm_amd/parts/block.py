@@ -13,6 +13,7 @@ class PreNormBlock(Block):
     its last delta on as ``pending`` and the next block's (or the model's
     final) norm adds it.  The sums are float32."""
     slot_categories = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ff": "feed_forward"}
+    graph_safe_prompts = True
 
     @staticmethod
     def _normed(norm, consumer, resid, delta):

@@ -19,6 +19,7 @@ class SwiGLUMLP(FeedForward):
     at load so one GEMM makes both."""
 
     takes_deferred_norm = True      # Linear.swiglu runs or fuses it
+    graph_safe_prompts = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, act_dtype: torch.dtype = torch.bfloat16):
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size

@@ -103,9 +103,10 @@ class DecoderModel:
         self.head = Linear(tensors[spec.head_name].to(dev) if spec.head_name else self.embed,
                            tensors[spec.head_bias_name].to(dev) if spec.head_bias_name else None)
 
-    def is_graph_safe(self) -> bool:
-        """Whether a decode step of this model may be recorded into a HIP graph: every part says so."""
-        return all(blk.is_graph_safe() for blk in self.layers) and self.final_norm.is_graph_safe()
+    def is_graph_safe(self, prompts: bool = False) -> bool:
+        """Whether a decode step (``prompts``: a padded prompt step) of this model may be recorded into a HIP
+        graph: every part says so."""
+        return all(blk.is_graph_safe(prompts) for blk in self.layers) and self.final_norm.is_graph_safe(prompts)
 
     def num_weight_bytes(self) -> int:
         """Bytes a decode step streams: every matrix once (the embedding table only as the

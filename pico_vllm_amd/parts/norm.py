@@ -14,6 +14,7 @@ from .spec import ParamSpec
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
     """y = x / sqrt(mean(x^2) + eps) * weight, in float32 (pico_vllm/RMSNorm.py:22-31)."""
+    graph_safe_prompts = True
 
     def __init__(self, size: int, eps: float, act_dtype: torch.dtype = torch.bfloat16):
         self.size, self.eps, self.act_dtype = size, eps, act_dtype

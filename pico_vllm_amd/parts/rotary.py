@@ -15,6 +15,8 @@ class RotaryHalf(PositionEncoding):
     and are computed inside the kernel from the position, so there is no table
     whose length bounds the sequence (the reference keeps a [131072, d] table)."""
 
+    graph_safe_prompts = True
+
     def __init__(self, rotary_dim: int, theta: float, act_dtype: torch.dtype = torch.bfloat16):
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim must be even, got {rotary_dim}")
@@ -60,6 +62,7 @@ class RotaryHalf(PositionEncoding):
 @register_part("position", "none")
 class NoPosition(PositionEncoding):
     """No position encoding: keys and values are stored as they are."""
+    graph_safe_prompts = True
 
     def __init__(self, act_dtype: torch.dtype = torch.bfloat16):
         pass

@@ -203,3 +203,69 @@ def test_graph_replay_and_the_step_in_flight_at_head_size_128():
             for k, t in enumerate(gen):
                 row = logits[len(p) + k - 1]
                 assert float(row[t]) >= float(row.max()) - 0.05 * float(row.std()), (batch, len(p), k, t, int(row.argmax()))
+
+
+def test_prompt_steps_replayed_from_graphs_at_sizes_that_take_the_library_products():
+    """A prompt portion that is a step of its own replays a graph recorded at the next of a few sizes, padded with
+    filler tokens in a sequence of their own.  At the 1.5B layer sizes such a step holds library matrix products;
+    whatever those record into a graph must give the same on every replay: every replay (prompts of other lengths
+    and contents at the same recorded size, portions after a prefix, decode steps and synchronisations between them)
+    is compared bit for bit with the same padded step run unrecorded, and with the plain implementation."""
+    import plain_qwen2 as P
+    from tiny_configs import CONFIGS, model_dir
+    from pico_vllm_amd.engine.batch import SeqStep, build_context
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import load_model
+    name = "L1.5B"
+    V = CONFIGS[name]["vocab_size"]
+    model = load_model(model_dir(name), "bfloat16", "cuda:0")
+    rec = ModelRunner(model, 16, 256, 4, 1024, 2048, use_graph=True, max_graph_batch=4)
+    raw = ModelRunner(model, 16, 256, 4, 1024, 2048, use_graph=False)
+    assert rec.graph_prompts and 320 in rec.prompt_sizes and 1024 in rec.prompt_sizes
+    plain = P.PlainModel(model_dir(name))
+    rng = random.Random(9)
+
+    def both(rid, toks, want):
+        """The step on both runners; the unrecorded one is padded by hand to the size the recorded one takes."""
+        outs = []
+        for r in (rec, raw):
+            m = r.manager
+            if rid not in m.requests:
+                assert m.add_request(rid)
+            assert m.grow(rid, m.num_computed(rid) + len(toks))
+            seq = SeqStep(rid, toks, want)
+            if r is rec:
+                size = r._prompt_size([seq])
+                outs.append(r.step([seq]).clone())
+            elif size:
+                ctx = build_context([seq], m, r.buffers, model.dtype, V, pad_tokens_to=size)
+                outs.append(model.forward(ctx, r.storage).clone())
+            else:
+                outs.append(r.step([seq]).clone())
+            r.advance([seq])
+        torch.cuda.synchronize()
+        return outs[0], outs[1], size
+
+    sizes_seen = []
+    for i, (n_first, n_second) in enumerate([(300, 290), (310, 17), (257, 200), (300, 0), (1000, 24), (318, 5)]):
+        rid = f"p{i}"
+        toks = [rng.randrange(V) for _ in range(n_first + n_second + 3)]
+        a, b, size = both(rid, toks[:n_first], [n_first - 1])
+        sizes_seen.append(size)
+        assert size >= n_first and torch.equal(a, b), (i, "first portion", size)
+        ref = plain.logits(toks[:n_first])[-1]
+        assert float((a[0].cpu() - ref).abs().max()) < 0.1 * float(ref.std())
+        if n_second:
+            a, b, size2 = both(rid, toks[n_first:n_first + n_second], [n_second - 1])     # a portion after a prefix
+            assert torch.equal(a, b), (i, "second portion", size2)
+            ref = plain.logits(toks[:n_first + n_second])[-1]
+            assert float((a[0].cpu() - ref).abs().max()) < 0.1 * float(ref.std())
+        for t in toks[n_first + n_second:]:                                              # decode steps in between
+            a, b, _ = both(rid, [t], [0])
+            assert torch.equal(a, b)
+        for r in (rec, raw):
+            r.manager.free_request(rid)
+    assert sizes_seen.count(320) >= 3 and 1024 in sizes_seen          # a recorded size was replayed after other work
+    assert len(rec._prompt_graphs) >= 4 and not raw._prompt_graphs
+    del rec, raw, model
+    torch.cuda.empty_cache()
