@@ -67,6 +67,9 @@ class ModelRunner:
         self.max_graph_batch = max_graph_batch
         self._graphs: Dict[int, tuple] = {}
         self._prompt_graphs: Dict[tuple, tuple] = {}       # (recorded size, wanted rows) -> (graph, logits)
+        # all graphs take their intermediate tensors from one pool (they never run at the same time), so that a
+        # dozen recorded sizes hold the memory of the largest, not of all
+        self._graph_pool = torch.cuda.graph_pool_handle() if self.use_graph else None
         self.steps = 0
         self.tokens = 0
 
@@ -181,7 +184,7 @@ class ModelRunner:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, pool=self._graph_pool):
             out = self.model.forward(ctx, self.storage)
         self.storage.restore_state(saved)
         return graph, out
