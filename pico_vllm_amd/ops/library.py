@@ -146,7 +146,7 @@ def peaks() -> ctypes.CDLL:
     return load_library("pico_peaks", PEAK_SOURCES)
 
 
-def build_all(head_dims: Iterable[int] = (16, 32, 48, 64, 80, 96, 128, 160, 192, 224, 256), force: bool = True) -> List[str]:
+def build_all(head_dims: Iterable[int] = tuple(range(16, 257, 16)), force: bool = True) -> List[str]:
     """Compile everything (used by the build check); returns the paths."""
     out = [build_library("pico_core", CORE_SOURCES, force=force), build_library("pico_peaks", PEAK_SOURCES, force=force)]
     if os.path.isfile(os.path.join(CSRC, "attention_mfma.hip")):

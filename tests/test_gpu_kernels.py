@@ -450,17 +450,21 @@ def test_fast_prefill_with_every_shape_of_workgroup(K, nq, nkv, d, Pg, teams):
 
 
 @pytest.mark.parametrize("Pg", [8, 16, 32])
-@pytest.mark.parametrize("d", [32, 64, 96, 128, 160, 192, 224, 256])
+@pytest.mark.parametrize("d", list(range(16, 257, 16)))
 def test_fast_prefill_whole_key_tiles_at_every_head_size_and_page_size(K, d, Pg):
     # contexts of three and more whole key tiles: where a thread's chunks of K are a whole number of pages
     # apart the kernel prepares its addresses once per tile, elsewhere it must not; queries are scaled up so
     # that a few keys carry each row's weight and a wrong key or row part shows
     def boost(qs, ks, vs):
         for q in qs:
-            q *= 3.0
+            q *= 4.0            # a power of two: the scaled queries are bfloat16 numbers still
     out, want = _fast_case([200, 70, 3], [0, 330, 400], 2, 1, d, Pg, seed=17 + d + Pg, boost=boost)
     assert float(want.abs().mean()) > 0.3
     close(out, want, torch.bfloat16)
+    # and the decode kernels of that head size, whole and split
+    for nsplit in (1, 5):
+        out, want = _fast_case([1, 1], [330, 65], 2, 1, d, Pg, seed=d + Pg, boost=boost, decode=True, nsplit=nsplit)
+        close(out, want, torch.bfloat16)
 
 
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(12, 2, 128, 16), (6, 3, 32, 8), (5, 5, 48, 16), (4, 1, 16, 16)])
