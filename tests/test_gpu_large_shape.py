@@ -269,3 +269,20 @@ def test_prompt_steps_replayed_from_graphs_at_sizes_that_take_the_library_produc
     assert len(rec._prompt_graphs) >= 4 and not raw._prompt_graphs
     del rec, raw, model
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_all_28_layers_of_the_1_5b_shape_against_the_plain_implementation(dtype):
+    """The benchmark's own configuration, every layer and the whole vocabulary of 151,936, with random weights: a prompt
+    of 48 tokens whole and with its last 8 tokens one by one against the plain implementation in float64, with the
+    bounds of the replay tests (28 layers of rounding on top of one another)."""
+    import test_gpu_replay as R
+    reqs = R.make_requests("F1.5B", [48], seed=23)
+    print(f"[real sizes] F1.5B {dtype}", flush=True)
+    for label, trace in (("whole", R.whole(reqs)), ("tail", R.tail_one_by_one(reqs, tail=8))):
+        got, _ = R.replay("F1.5B", dtype, trace)
+        R.compare("F1.5B", dtype, reqs, got, f"28 layers {label}")
+    torch.cuda.empty_cache()
+    if dtype == "bfloat16":
+        for key in [k for k in R._plain_cache if k == "F1.5B" or (isinstance(k, tuple) and k[0] == "F1.5B")]:
+            del R._plain_cache[key]          # 18 GB of float32 and float64 weights

@@ -75,7 +75,9 @@ def _real(hidden, heads, kv_heads, inter, layers, vocab, tied):
 # Layers of the sizes of real models (the vocabulary cut down so that the plain implementation stays quick): two
 # layers of Qwen2.5-1.5B, one each of 7B (groups of 7 heads) and 32B (groups of 5, a width beyond 4,096)
 REAL = {"L1.5B": _real(1536, 12, 2, 8960, 2, 20011, True), "L7B": _real(3584, 28, 4, 18944, 1, 4099, False),
-        "L32B": _real(5120, 40, 8, 27648, 1, 3001, False)}
+        "L32B": _real(5120, 40, 8, 27648, 1, 3001, False),
+        # the whole Qwen2.5-1.5B shape: all 28 layers and the whole vocabulary
+        "F1.5B": _real(1536, 12, 2, 8960, 28, 151936, True)}
 for _name, _cfg in REAL.items():
     CONFIGS[_name], PAGE_SIZE[_name] = _cfg, 16
 
