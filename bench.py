@@ -239,9 +239,9 @@ def long_prompt_point(model_dir, model, dtype, prompt_len):
     eng = make_engine(model_dir, dtype, 1, model)
     V = CONFIG["vocab_size"]
     g = torch.Generator().manual_seed(3)
-    warm = eng.submit(torch.randint(0, V, (PREFILL_TOKENS + 40,), generator=g).tolist(), max_new_tokens=2, ignore_eos=True)
+    warm = eng.submit(torch.randint(0, V, (prompt_len,), generator=g).tolist(), max_new_tokens=2, ignore_eos=True)
     while not eng.is_done():
-        eng.step()                                   # kernels built, library products chosen
+        eng.step()                                   # kernels built, library products chosen, steps recorded
     torch.cuda.synchronize()
     rid = eng.submit(torch.randint(0, V, (prompt_len,), generator=g).tolist(), max_new_tokens=2, temperature=0.0, ignore_eos=True)
     req = eng.requests[rid]

@@ -66,7 +66,7 @@ class ModelRunner:
         self.prompt_sizes = prompt_sizes(min(max_tokens_per_step, self.max_pages * page_size))
         self.max_graph_batch = max_graph_batch
         self._graphs: Dict[int, tuple] = {}
-        self._prompt_graphs: Dict[tuple, tuple] = {}       # (recorded size, wanted rows) -> (graph, logits)
+        self._prompt_graphs: Dict[tuple, tuple] = {}       # (recorded size, wanted rows, the parts' choices) -> (graph, logits)
         # all graphs take their intermediate tensors from one pool (they never run at the same time), so that a
         # dozen recorded sizes hold the memory of the largest, not of all
         self._graph_pool = torch.cuda.graph_pool_handle() if self.use_graph else None
@@ -155,13 +155,14 @@ class ModelRunner:
         return 0
 
     def _step_prompt_graph(self, seq: SeqStep, size: int) -> torch.Tensor:
-        key = (size, len(seq.want))
+        ctx = build_context([seq], self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
+                            pad_tokens_to=size)
+        # what parts choose on the host for this step (a kernel's shape for a short or a long context) is part of
+        # the key: a replay runs what the step would run unrecorded
+        key = (size, len(seq.want), self.model.graph_variant(ctx))
         if key not in self._prompt_graphs:
-            ctx = build_context([seq], self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
-                                pad_tokens_to=size)
-            self._prompt_graphs[key] = self._record(ctx)
+            self._prompt_graphs[key] = self._record(ctx)        # leaves the step's arrays as they are
         graph, out = self._prompt_graphs[key]
-        build_context([seq], self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size, pad_tokens_to=size)
         graph.replay()
         return out
 

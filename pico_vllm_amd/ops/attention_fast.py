@@ -129,15 +129,12 @@ class FastAttention:
             if t is not None and (t.dtype != torch.int32 or t.numel() < n or not t.is_contiguous()):
                 raise KernelError("sequence metadata must be contiguous int32")
 
-    def __call__(self, qkv, cache, block_table, ctx, scale):
-        B = ctx.num_seqs
-        grouped = self.nq // self.nkv <= 32
-        if ctx.all_decode and grouped:
-            return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, B, scale,
-                               self.num_splits(B, ctx.max_context))
-        # what the host decides from the shape of the batch is the same for every layer of the step
-        plan = ("fast_attention", self.nq, self.nkv, self.d)
-        if plan not in ctx.shared:
+    def plan(self, ctx) -> tuple:
+        """(teams, lead) of a step with prompt portions: the shape of the prefill workgroups and how many single
+        tokens stand first.  Decided on the host from the shape of the batch, once for every layer of the step."""
+        key = ("fast_attention", self.nq, self.nkv, self.d, self.window)
+        if key not in ctx.shared:
+            B = ctx.num_seqs
             teams, lead = 0, 0
             if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
                 cu = ctx.host["cu_seqlens"]
@@ -145,8 +142,16 @@ class FastAttention:
                 while lead < B and lens[lead] == 1:
                     lead += 1
                 teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
-            ctx.shared[plan] = (teams, lead)
-        teams, lead = ctx.shared[plan]
+            ctx.shared[key] = (int(teams), int(lead))
+        return ctx.shared[key]
+
+    def __call__(self, qkv, cache, block_table, ctx, scale):
+        B = ctx.num_seqs
+        grouped = self.nq // self.nkv <= 32
+        if ctx.all_decode and grouped:
+            return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, B, scale,
+                               self.num_splits(B, ctx.max_context))
+        teams, lead = self.plan(ctx)
         if lead == 0 or not grouped:
             return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, scale, teams=teams)
         # A mixed step: the scheduler puts the decoding requests first.  Their tokens (one row each, rows

@@ -30,7 +30,7 @@ class GQAAttention(Mixer):
     ``window`` > 0 restricts every query to the last ``window`` keys."""
 
     takes_deferred_norm = True
-    graph_safe_prompts = True       # the shape of the prefill workgroups is a hint taken from the recorded step
+    graph_safe_prompts = True       # what the host chooses (the shape of the prefill workgroups) is the graph's variant
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, position: PartSpec, window: int = 0,
@@ -75,6 +75,10 @@ class GQAAttention(Mixer):
         if self.act_dtype == torch.bfloat16:
             from ..ops import attention_fast
             self.fast = attention_fast.choose(self.nq, self.nkv, self.d, self.window)
+
+    def graph_variant(self, ctx: StepContext) -> tuple:
+        own = (("gqa_attention",) + self.fast.plan(ctx),) if self.fast is not None and not ctx.all_decode else ()
+        return own + super().graph_variant(ctx)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         nq, nkv, d = self.nq, self.nkv, self.d

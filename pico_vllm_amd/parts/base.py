@@ -62,14 +62,28 @@ class Part:
     portion's sequence stands a second one of filler tokens (slot -1, a block table of -1, outputs ignored) that
     brings the step to a recorded size.  A part that says True does device work only in such a step, may take what
     it decides on the host from the step that was recorded (``ctx.host`` is that step's), and keeps nothing of the
-    filler.  The default is False: prompt steps of a model with such a part run unrecorded."""
+    filler.  The default is False: prompt steps of a model with such a part run unrecorded.
+
+    ``graph_variant(ctx)``: what such a part decides on the host for a prompt step (a kernel's shape, say), as
+    something hashable.  Steps whose variants differ are recorded apart, so that a replayed step runs what the
+    same step unrecorded would."""
     graph_safe = True
     graph_safe_prompts = False
+
+    def graph_variant(self, ctx: "StepContext") -> tuple:
+        """This part's and its parts' host-side choices for the step (empty: none)."""
+        out = ()
+        for p in self._sub_parts():
+            out += p.graph_variant(ctx)
+        return out
+
+    def _sub_parts(self) -> List["Part"]:
+        return [p for p in vars(self).values() if isinstance(p, Part)]
 
     def is_graph_safe(self, prompts: bool = False) -> bool:
         """This part and the parts it is built from."""
         own = self.graph_safe_prompts if prompts else self.graph_safe
-        return own and all(p.is_graph_safe(prompts) for p in vars(self).values() if isinstance(p, Part))
+        return own and all(p.is_graph_safe(prompts) for p in self._sub_parts())
 
     def param_specs(self) -> List[ParamSpec]:
         return []
@@ -157,9 +171,8 @@ class Block(Part):
     def __init__(self, parts: Dict[str, Part]):
         self.parts = parts
 
-    def is_graph_safe(self, prompts: bool = False) -> bool:
-        own = self.graph_safe_prompts if prompts else self.graph_safe
-        return own and all(p.is_graph_safe(prompts) for p in self.parts.values())
+    def _sub_parts(self) -> List[Part]:
+        return list(self.parts.values())
 
     @property
     def mixer(self) -> Mixer:

@@ -108,6 +108,16 @@ class DecoderModel:
         graph: every part says so."""
         return all(blk.is_graph_safe(prompts) for blk in self.layers) and self.final_norm.is_graph_safe(prompts)
 
+    def graph_variant(self, ctx) -> tuple:
+        """The host-side choices of all parts for this step, each distinct one once (layers of one kind choose
+        alike): part of the key under which a prompt step is recorded."""
+        seen = []
+        for blk in self.layers:
+            v = blk.graph_variant(ctx)
+            if v and v not in seen:
+                seen.append(v)
+        return tuple(seen)
+
     def num_weight_bytes(self) -> int:
         """Bytes a decode step streams: every matrix once (the embedding table only as the
         output matrix when tied)."""

@@ -219,8 +219,8 @@ def test_prompt_steps_replayed_from_graphs_at_sizes_that_take_the_library_produc
     name = "L1.5B"
     V = CONFIGS[name]["vocab_size"]
     model = load_model(model_dir(name), "bfloat16", "cuda:0")
-    rec = ModelRunner(model, 16, 256, 4, 1024, 2048, use_graph=True, max_graph_batch=4)
-    raw = ModelRunner(model, 16, 256, 4, 1024, 2048, use_graph=False)
+    rec = ModelRunner(model, 16, 448, 4, 2048, 6144, use_graph=True, max_graph_batch=4)
+    raw = ModelRunner(model, 16, 448, 4, 2048, 6144, use_graph=False)
     assert rec.graph_prompts and 320 in rec.prompt_sizes and 1024 in rec.prompt_sizes
     plain = P.PlainModel(model_dir(name))
     rng = random.Random(9)
@@ -267,6 +267,14 @@ def test_prompt_steps_replayed_from_graphs_at_sizes_that_take_the_library_produc
             r.manager.free_request(rid)
     assert sizes_seen.count(320) >= 3 and 1024 in sizes_seen          # a recorded size was replayed after other work
     assert len(rec._prompt_graphs) >= 4 and not raw._prompt_graphs
+    # What the attention chooses on the host (the shape of its prefill workgroups) differs between a first portion and
+    # one behind thousands of tokens: the two are recorded apart, and each replay is the unrecorded step bit for bit.
+    toks = [rng.randrange(V) for _ in range(6000)]
+    for at, n in ((0, 2048), (2048, 2048), (4096, 1900)):
+        a, b, size = both("long", toks[at:at + n], [n - 1])
+        assert size == 2048 and torch.equal(a, b), (at, n)
+    variants = {key[2] for key in rec._prompt_graphs if key[0] == 2048}
+    assert len(variants) >= 2, variants
     del rec, raw, model
     torch.cuda.empty_cache()
 
