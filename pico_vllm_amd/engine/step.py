@@ -143,15 +143,15 @@ class ModelRunner:
 
     # ---- graph replay of a prompt portion alone ---------------------------
     def _prompt_size(self, seqs: List[SeqStep]) -> int:
-        """The recorded size that serves this step, or 0: one sequence of two tokens or more, at most one wanted
-        row, and room in the block table for the filler's positions."""
+        """The recorded size that serves this step, or 0: one sequence of two tokens or more and at most one
+        wanted row.  (The filler is a sequence of its own with positions from 0, so it needs no room behind the
+        request's tokens.)"""
         if len(seqs) != 1 or len(seqs[0].tokens) < 2 or len(seqs[0].want) > 1:
             return 0
         n = len(seqs[0].tokens)
         for size in self.prompt_sizes:
             if size >= n:
-                fits = self.manager.num_computed(seqs[0].req) + size <= self.max_pages * self.manager.page_size
-                return size if fits else 0
+                return size
         return 0
 
     def _step_prompt_graph(self, seq: SeqStep, size: int) -> torch.Tensor:
