@@ -226,6 +226,33 @@ def forward(tokens: Sequence[int], w: Dict[str, torch.Tensor], cfg: PlainConfig,
     return x @ f32(out_w).T
 
 
+def permute_inner_dimensions(w: Dict[str, torch.Tensor], cfg: PlainConfig, generator: torch.Generator) -> Dict[str, torch.Tensor]:
+    """The same model with its hidden and intermediate dimensions in another (random) order: every matrix and norm
+    weight is permuted consistently, so the function from tokens to logits is unchanged (model.py:361-374 adds and
+    norms along the hidden dimension, model.py:309-318 contracts over the intermediate one; neither cares about the
+    order), but every sum over those dimensions runs in another order.  In float32 each such model is an independent
+    draw of what float32 rounding does to the logits.  Head dimensions keep their order (rotation pairs j with
+    j + d/2, model.py:116-123)."""
+    ph = torch.randperm(cfg.hidden_size, generator=generator)
+    pi = torch.randperm(cfg.intermediate_size, generator=generator)
+    out = {}
+    for name, t in w.items():
+        if name.endswith("embed_tokens.weight") or name.endswith("lm_head.weight"):
+            t = t[:, ph]
+        elif name.endswith("layernorm.weight") or name == "model.norm.weight":
+            t = t[ph]
+        elif name.endswith(("q_proj.weight", "k_proj.weight", "v_proj.weight")):
+            t = t[:, ph]
+        elif name.endswith("o_proj.weight"):
+            t = t[ph, :]
+        elif name.endswith(("gate_proj.weight", "up_proj.weight")):
+            t = t[pi][:, ph]
+        elif name.endswith("down_proj.weight"):
+            t = t[ph][:, pi]
+        out[name] = t.contiguous()
+    return out
+
+
 class PlainModel:
     """A model folder read once; ``logits(tokens)`` runs the whole sequence."""
 

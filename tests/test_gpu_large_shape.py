@@ -283,7 +283,7 @@ def test_prompt_steps_replayed_from_graphs_at_sizes_that_take_the_library_produc
 def test_all_28_layers_of_the_1_5b_shape_against_the_plain_implementation(dtype):
     """The benchmark's own configuration, every layer and the whole vocabulary of 151,936, with random weights: a prompt
     of 48 tokens whole and with its last 8 tokens one by one against the plain implementation in float64, with the
-    bounds of the replay tests (28 layers of rounding on top of one another)."""
+    yardsticks of the replay tests (in float32: eight permuted float32 runs of the plain implementation)."""
     import test_gpu_replay as R
     reqs = R.make_requests("F1.5B", [48], seed=23)
     print(f"[real sizes] F1.5B {dtype}", flush=True)

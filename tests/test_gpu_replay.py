@@ -1,6 +1,7 @@
 """Trace replay against the plain implementation: the same requests whole, with the last 32
 tokens one by one, in portions of changing size, and mixed with other requests in a pool so small
 that pages are used again; in 32-bit and in bfloat16."""
+import functools
 import json
 import os
 import random
@@ -17,18 +18,48 @@ from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-# float32: the engine and the plain implementation differ in summation order only; errors are
-# measured against the spread (standard deviation) of the request's logits.
+# float32: the engine and the plain implementation differ in summation order only, and what a summation order does
+# to a logit depends on the position: at most positions about 1e-6 of the logits' spread, at an ill-conditioned one (a
+# residual stream that nearly cancels in front of a norm) ten times that, for every float32 arithmetic alike.  The
+# yardstick is therefore taken per position: the plain implementation in float32, run F32_DRAWS times with its hidden
+# and intermediate dimensions permuted (plain_qwen2.permute_inner_dimensions: the same function, other orders of
+# summation), against itself in float64.  Each run is an independent draw of float32 rounding at every position; the
+# engine's error is one more.  Where the error of a position is essentially one direction (the worst case for tails),
+# the engine's rms error over the position's logits, divided by the rms of the K draws there, is Student's |t| with K
+# degrees of freedom, and its largest error over the largest of the K draws' is |a| / max |b_k| of K + 1 normal
+# numbers: F32_FALSE_ALARM is the probability per position that a float32 arithmetic as noisy as the CPU library's would
+# exceed the bounds below.  (The engine's sums are trees of radix 16: it measures 0.6 of the draws' rms at the
+# median position, 2.1 at the worst of 70,000 positions of 340 drawn configurations.)  No fixed fraction of the spread
+# is asserted: the plain float32 run itself exceeds any that typical positions would make meaningful.
 # bfloat16: the yardstick is the plain implementation itself with every activation between the
 # parts rounded to bfloat16 (plain_qwen2.to_bf16): how far that moves the logits of this request
 # is the rounding noise of this model at this length.  The engine must stay within a small
 # multiple of it; a fault larger than the rounding noise fails, whatever the model's sensitivity.
-F32_REL_MAX, F32_REL_MEAN = 2e-5, 4e-6        # for models of up to three layers; the rounding of L layers adds up like sqrt(L)
-# The yardstick that adapts to the model, as for bfloat16: the plain implementation itself in float32 (torch on the
-# CPU, its own summation orders) against the same in float64 shows what float32 arithmetic costs THIS request of THIS
-# model.  The engine's sums are trees of radix 16 (2 half-units in the last place rms for any K, against 4 to 5 for
-# the CPU library's), so it stays below the plain float32 run's own error; a fault does not.
-F32_VS_PLAIN32_RMS, F32_VS_PLAIN32_MAX = 1.25, 2.0
+F32_FALSE_ALARM = 1e-5
+F32_GLOBAL_RMS = 1.25         # the engine's rms error over a whole request against the draws' (measured: 0.65 median, 1.05 worst)
+
+
+def f32_draws(name) -> int:
+    """How many permuted float32 runs make the yardstick: 32 for the tiny models, fewer where one run takes seconds."""
+    c = CONFIGS[name]
+    params = c["num_hidden_layers"] * c["hidden_size"] * (3 * c["intermediate_size"] + 4 * c["hidden_size"]) + c["vocab_size"] * c["hidden_size"]
+    return 32 if params <= 20e6 else 16 if params <= 1e9 else 8
+
+
+@functools.lru_cache(maxsize=None)
+def f32_bounds(K: int):
+    """(bound on a position's rms error in units of the K draws' rms there, bound on its largest error in units of the
+    K draws' largest there) at F32_FALSE_ALARM."""
+    from scipy import integrate, optimize, stats
+    t_rms = float(stats.t.isf(F32_FALSE_ALARM / 2, K))
+
+    def exceed(T):       # P(|a| > T max_k |b_k|), a and the K b_k standard normal
+        f = lambda m: K * (2 * stats.norm.cdf(m) - 1) ** (K - 1) * 2 * stats.norm.pdf(m) * 2 * stats.norm.sf(T * m)
+        return integrate.quad(f, 0, 12, limit=200)[0]
+    t_max = float(optimize.brentq(lambda T: exceed(T) - F32_FALSE_ALARM, 0.5, 500))
+    return t_rms, t_max
+
+
 BF16_RMS_FACTOR, BF16_MAX_FACTOR = 1.5, 2.0
 # The engine stores bfloat16 where the rounded plain computation rounds (activations between parts,
 # probabilities before P.V), so it follows THAT computation at least as closely as the exact one:
@@ -183,18 +214,33 @@ def bf16_noise(name, tokens):
 _noise32_cache = {}
 
 
-def f32_noise(name, tokens):
-    """(rms, max) of the logit error of the plain implementation run in float32 against float64."""
-    key = (name, tuple(tokens))
-    if key not in _noise32_cache:
-        ref = plain_logits(name, tokens)
-        err = np.abs(_plain_cache[name].logits(tokens).numpy().astype(np.float64) - ref)
-        _noise32_cache[key] = (float(np.sqrt((err ** 2).mean())), float(err.max()))
-    return _noise32_cache[key]
+def f32_noise(name, reqs):
+    """For every request: (rms [positions], largest [positions]) of the logit errors of ``f32_draws(name)`` permuted
+    plain float32 runs against the plain float64 run, over the draws and the vocabulary."""
+    missing = [toks for toks in reqs.values() if (name, tuple(toks)) not in _noise32_cache]
+    if missing:
+        plain_logits(name, missing[0])                                   # the models are read
+        m32 = _plain_cache[name]
+        K = f32_draws(name)
+        gen = torch.Generator().manual_seed(1234)
+        sq = {tuple(t): 0.0 for t in missing}
+        mx = {tuple(t): 0.0 for t in missing}
+        for _ in range(K):                                               # one permuted model at a time: it may be large
+            w = P.permute_inner_dimensions(m32.w, m32.cfg, gen)
+            for toks in missing:
+                with torch.no_grad():
+                    e = P.forward(toks, w, m32.cfg).numpy().astype(np.float64) - plain_logits(name, toks)
+                sq[tuple(toks)] = sq[tuple(toks)] + (e ** 2).mean(axis=1)
+                mx[tuple(toks)] = np.maximum(mx[tuple(toks)], np.abs(e).max(axis=1))
+            del w
+        for toks in missing:
+            _noise32_cache[name, tuple(toks)] = (np.sqrt(sq[tuple(toks)] / K), mx[tuple(toks)])
+    return {rid: _noise32_cache[name, tuple(toks)] for rid, toks in reqs.items()}
 
 
 def compare(name, dtype, reqs, got, label):
     worst = 0.0
+    noise32 = f32_noise(name, reqs) if dtype == "float32" else None
     for rid, toks in reqs.items():
         ref = plain_logits(name, toks)
         spread = float(ref.std())
@@ -204,17 +250,19 @@ def compare(name, dtype, reqs, got, label):
         if dtype == "float32":
             rel = err.max(axis=1) / spread
             worst = max(worst, float(rel.max()))
-            n_rms, n_max = f32_noise(name, toks)
-            rms = float(np.sqrt((err.astype(np.float64) ** 2).mean()))
-            print(f"[replay] {label} {name} f32 {rid}: rms {rms / n_rms:.2f}x max {err.max() / n_max:.2f}x of the plain float32 "
-                  f"run's own error (max {n_max / spread:.2e} of the spread); worst {rel.max():.2e} of the spread")
-            depth = max(1.0, (CONFIGS[name]["num_hidden_layers"] / 3.0) ** 0.5)
-            assert rel.max() <= F32_REL_MAX * depth, (f"{label} {name} {dtype}: request {rid} first wrong position "
-                                                      f"{int(np.argmax(rel > F32_REL_MAX * depth))}, worst {rel.max():.3e} at {int(rel.argmax())}")
-            assert err.mean() / spread <= F32_REL_MEAN * depth, f"{label} {name}: mean error {err.mean() / spread:.3e}"
-            assert rms <= F32_VS_PLAIN32_RMS * n_rms and err.max() <= F32_VS_PLAIN32_MAX * n_max, \
-                (f"{label} {name} float32: request {rid}: {rms / n_rms:.2f}x (rms) {err.max() / n_max:.2f}x (max) the error of "
-                 f"the plain implementation in float32")
+            n_rms, n_max = noise32[rid]
+            t_rms, t_max = f32_bounds(f32_draws(name))
+            pos_rms = np.sqrt((err.astype(np.float64) ** 2).mean(axis=1))
+            a, b = pos_rms / n_rms, err.max(axis=1) / n_max
+            g = float(np.sqrt((pos_rms ** 2).mean() / (n_rms ** 2).mean()))
+            print(f"[replay] {label} {name} f32 {rid}: of the permuted float32 runs' own error: rms over the request {g:.2f}x, "
+                  f"a position's rms {np.median(a):.2f}x (median) {a.max():.2f}x (worst, bound {t_rms:.2f}), a position's largest "
+                  f"{b.max():.2f}x (bound {t_max:.2f}); worst {rel.max():.2e} of the spread, where the runs reach {n_max[int(rel.argmax())] / spread:.2e}")
+            assert a.max() <= t_rms, (f"{label} {name} float32: request {rid} position {int(a.argmax())}: rms error {a.max():.2f}x "
+                                      f"that of the permuted float32 runs there (first position above {t_rms:.2f}: {int(np.argmax(a > t_rms))})")
+            assert b.max() <= t_max, (f"{label} {name} float32: request {rid} position {int(b.argmax())}: largest error {b.max():.2f}x "
+                                      f"the largest of the permuted float32 runs there (bound {t_max:.2f})")
+            assert g <= F32_GLOBAL_RMS, f"{label} {name} float32: request {rid}: rms error {g:.2f}x that of the permuted float32 runs"
         else:
             noise_rms, noise_max, rounded = bf16_noise(name, toks)
             rms = float(np.sqrt((err ** 2).mean()))
@@ -338,8 +386,10 @@ def test_long_decoding_and_first_tokens():
         compare("A", dtype, reqs, got, "long decode")
         first = np.stack([got[("r0", p)] for p in range(4)])
         ref = plain_logits("A", toks)[:4]
-        bound = F32_REL_MAX * ref.std() if dtype == "float32" else BF16_MAX_FACTOR * bf16_noise("A", toks)[1]
-        assert np.abs(first - ref).max() <= bound
+        if dtype == "float32":
+            assert (np.abs(first - ref).max(axis=1) <= f32_bounds(f32_draws("A"))[1] * f32_noise("A", reqs)["r0"][1][:4]).all()
+        else:
+            assert np.abs(first - ref).max() <= BF16_MAX_FACTOR * bf16_noise("A", toks)[1]
 
 
 def test_the_program_itself_in_a_subprocess():

@@ -208,6 +208,25 @@ def test_model_is_causal_and_shift_invariant(name):
     assert not torch.allclose(m.logits(ids2)[-1], full[-1], atol=1e-4)            # the far token does matter
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_a_model_with_its_inner_dimensions_permuted_is_the_same_function(name):
+    # the yardstick of the float32 replay tests: in float64 the permuted model gives the same logits to the last
+    # places, in float32 it rounds differently (an independent draw of float32 rounding)
+    d = model_dir(name)
+    m64, m32 = P.PlainModel(d, torch.float64), _plain(name)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, m64.cfg.vocab_size, (20,), generator=g).tolist()
+    ref = m64.logits(ids)
+    w64 = P.permute_inner_dimensions(m64.w, m64.cfg, g)
+    assert any(not torch.equal(w64[k], m64.w[k]) for k in w64)
+    with torch.no_grad():
+        assert float((P.forward(ids, w64, m64.cfg) - ref).abs().max()) < 1e-11 * float(ref.std())
+        a = m32.logits(ids).double()
+        b = P.forward(ids, P.permute_inner_dimensions(m32.w, m32.cfg, g), m32.cfg).double()
+    assert not torch.equal(a, b)                                         # other roundings
+    assert float((b - ref).abs().max()) < 1e-4 * float(ref.std())        # of the same, small, size
+
+
 def test_qkv_bias_is_used():
     m = _plain("A")
     w = {k: (torch.zeros_like(v) if k.endswith("_proj.bias") else v) for k, v in m.w.items()}
