@@ -170,6 +170,19 @@ def to_bf16(x: torch.Tensor) -> torch.Tensor:
     return x.to(torch.bfloat16).float()
 
 
+def dithered_bf16(generator: torch.Generator):
+    """A rounding to bfloat16 whose error is drawn anew at every call (subtractive dither): x + d is rounded, d uniform
+    within one unit in the last place of x, and d is taken off again.  The error is that of a bfloat16 rounding, uniform
+    within half a unit in the last place, but independent of x and of every other call: runs of the plain
+    implementation with it are independent draws of what bfloat16 storage of activations does to the logits."""
+    def rnd(x: torch.Tensor) -> torch.Tensor:
+        _, e = torch.frexp(x)                                        # |x| in [2^(e-1), 2^e)
+        ulp = torch.ldexp(torch.ones_like(x), e - 8)                 # bfloat16 keeps 8 significant bits
+        d = (torch.rand(x.shape, generator=generator, dtype=x.dtype) - 0.5) * ulp
+        return (x + d).to(torch.bfloat16).to(x.dtype) - d
+    return rnd
+
+
 def attention_layer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
                     cfg: PlainConfig, positions: torch.Tensor, rnd=_same) -> torch.Tensor:
     """qkv = h W^T + b with bias on q, k, v only (model.py:148-152); RoPE on

@@ -18,55 +18,52 @@ from tiny_configs import CONFIGS, PAGE_SIZE, model_dir
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-# float32: the engine and the plain implementation differ in summation order only, and what a summation order does
-# to a logit depends on the position: at most positions about 1e-6 of the logits' spread, at an ill-conditioned one (a
-# residual stream that nearly cancels in front of a norm) ten times that, for every float32 arithmetic alike.  The
-# yardstick is therefore taken per position: the plain implementation in float32, run F32_DRAWS times with its hidden
-# and intermediate dimensions permuted (plain_qwen2.permute_inner_dimensions: the same function, other orders of
-# summation), against itself in float64.  Each run is an independent draw of float32 rounding at every position; the
-# engine's error is one more.  Where the error of a position is essentially one direction (the worst case for tails),
-# the engine's rms error over the position's logits, divided by the rms of the K draws there, is Student's |t| with K
-# degrees of freedom, and its largest error over the largest of the K draws' is |a| / max |b_k| of K + 1 normal
-# numbers: F32_FALSE_ALARM is the probability per position that a float32 arithmetic as noisy as the CPU library's would
-# exceed the bounds below.  (The engine's sums are trees of radix 16: it measures 0.6 of the draws' rms at the
-# median position, 2.1 at the worst of 70,000 positions of 340 drawn configurations.)  No fixed fraction of the spread
-# is asserted: the plain float32 run itself exceeds any that typical positions would make meaningful.
-# bfloat16: the yardstick is the plain implementation itself with every activation between the
-# parts rounded to bfloat16 (plain_qwen2.to_bf16): how far that moves the logits of this request
-# is the rounding noise of this model at this length.  The engine must stay within a small
-# multiple of it; a fault larger than the rounding noise fails, whatever the model's sensitivity.
-F32_FALSE_ALARM = 1e-5
-F32_GLOBAL_RMS = 1.25         # the engine's rms error over a whole request against the draws' (measured: 0.65 median, 1.05 worst)
+# What rounding does to a logit depends on the position: in float32 about 1e-6 of the logits' spread at most positions,
+# ten times that at an ill-conditioned one (a residual stream that nearly cancels in front of a norm), for every
+# arithmetic alike; in bfloat16 the same a few thousand times larger.  The yardstick is therefore taken per position, from
+# DRAWS independent runs of the plain implementation with the rounding in question, against the plain implementation in
+# float64:
+#   float32   the plain implementation in float32 with its hidden and intermediate dimensions permuted
+#             (plain_qwen2.permute_inner_dimensions: the same function, other orders of summation);
+#   bfloat16  the plain implementation with every activation between the parts, and the probabilities in front of P.V,
+#             rounded to bfloat16 with a subtractive dither (plain_qwen2.dithered_bf16: the error of each rounding is that
+#             of a bfloat16 rounding, uniform within half a unit in the last place, but drawn anew in every run).
+# Each run is a draw of that rounding's effect on every position; the engine's error is one more.  Where the error of a
+# position is essentially one direction (the worst case for tails), the engine's rms error over the position's logits
+# divided by the rms of the K draws there is Student's |t| with K degrees of freedom, and its largest error over the
+# largest of the K draws' is |a| / max |b_k| of K + 1 normal numbers: FALSE_ALARM is the probability per position that an
+# arithmetic exactly as noisy as the draws' would exceed the bounds (noise_bounds).  NOISIER says how much noisier than
+# the draws the engine may be: it bounds the engine's rms error at the median position of a request of 16 tokens or
+# more in units of the draws' (a statistic that no single position decides), and scales the two bounds per position.  float32: 1 (the CPU
+# library's sums are longer runs than the engine's trees of radix 16; the engine measures 0.6 at the median position).
+# bfloat16: 1.5 (the engine does not round exactly where the draws do: it rounds the unnormalised probabilities of an
+# online softmax, and fused kernels skip roundings; it measures 0.9).
+# No fixed fraction of the spread is asserted, and no ratio to one single draw: at an ill-conditioned position the ratio of
+# two draws has no useful bound (3.8 was seen in float32 among 340 configurations, where the plain float32 run itself was
+# 2.3e-5 of the spread off).
+FALSE_ALARM = 1e-5
+NOISIER = {"float32": 1.0, "bfloat16": 1.5}
 
 
-def f32_draws(name) -> int:
-    """How many permuted float32 runs make the yardstick: 32 for the tiny models, fewer where one run takes seconds."""
+def noise_draws(name) -> int:
+    """How many runs make the yardstick: 32 for the tiny models, fewer where one run takes seconds."""
     c = CONFIGS[name]
     params = c["num_hidden_layers"] * c["hidden_size"] * (3 * c["intermediate_size"] + 4 * c["hidden_size"]) + c["vocab_size"] * c["hidden_size"]
     return 32 if params <= 20e6 else 16 if params <= 1e9 else 8
 
 
 @functools.lru_cache(maxsize=None)
-def f32_bounds(K: int):
+def noise_bounds(K: int):
     """(bound on a position's rms error in units of the K draws' rms there, bound on its largest error in units of the
-    K draws' largest there) at F32_FALSE_ALARM."""
+    K draws' largest there) at FALSE_ALARM, for an arithmetic as noisy as the draws'."""
     from scipy import integrate, optimize, stats
-    t_rms = float(stats.t.isf(F32_FALSE_ALARM / 2, K))
+    t_rms = float(stats.t.isf(FALSE_ALARM / 2, K))
 
     def exceed(T):       # P(|a| > T max_k |b_k|), a and the K b_k standard normal
         f = lambda m: K * (2 * stats.norm.cdf(m) - 1) ** (K - 1) * 2 * stats.norm.pdf(m) * 2 * stats.norm.sf(T * m)
         return integrate.quad(f, 0, 12, limit=200)[0]
-    t_max = float(optimize.brentq(lambda T: exceed(T) - F32_FALSE_ALARM, 0.5, 500))
+    t_max = float(optimize.brentq(lambda T: exceed(T) - FALSE_ALARM, 0.5, 500))
     return t_rms, t_max
-
-
-BF16_RMS_FACTOR, BF16_MAX_FACTOR = 1.5, 2.0
-# The engine stores bfloat16 where the rounded plain computation rounds (activations between parts,
-# probabilities before P.V), so it follows THAT computation at least as closely as the exact one:
-# where both round the same value the errors cancel (measured 0.0x-0.4x with the plain attention
-# kernel); where the rounded values differ slightly (the matrix-core kernel rounds unnormalised
-# probabilities of an online softmax) the two rounding patterns are independent (measured 0.6x-0.7x).
-BF16_VS_ROUNDED_FACTOR = 1.0
 
 
 def make_requests(name, lengths, seed=0):
@@ -199,89 +196,63 @@ def replay(name, dtype, trace, max_tokens=None):
 _noise_cache = {}
 
 
-def bf16_noise(name, tokens):
-    """(rms, max) of the logit error that bfloat16 storage of activations causes in the plain
-    implementation for this request."""
-    key = (name, tuple(tokens))
-    if key not in _noise_cache:
-        plain_logits(name, tokens)
-        rounded = _plain_cache[name].logits(tokens, rnd=P.to_bf16).numpy()
-        err = np.abs(rounded - plain_logits(name, tokens))
-        _noise_cache[key] = (float(np.sqrt((err ** 2).mean())), float(err.max()), rounded)
-    return _noise_cache[key]
-
-
-_noise32_cache = {}
-
-
-def f32_noise(name, reqs):
-    """For every request: (rms [positions], largest [positions]) of the logit errors of ``f32_draws(name)`` permuted
-    plain float32 runs against the plain float64 run, over the draws and the vocabulary."""
-    missing = [toks for toks in reqs.values() if (name, tuple(toks)) not in _noise32_cache]
+def rounding_noise(name, dtype, reqs):
+    """For every request: (rms [positions], largest [positions]) of the logit errors of ``noise_draws(name)`` runs of
+    the plain implementation with the rounding of ``dtype`` (see the top of the file) against the plain float64 run,
+    over the draws and the vocabulary."""
+    missing = [toks for toks in reqs.values() if (name, dtype, tuple(toks)) not in _noise_cache]
     if missing:
         plain_logits(name, missing[0])                                   # the models are read
         m32 = _plain_cache[name]
-        K = f32_draws(name)
         gen = torch.Generator().manual_seed(1234)
         sq = {tuple(t): 0.0 for t in missing}
         mx = {tuple(t): 0.0 for t in missing}
-        for _ in range(K):                                               # one permuted model at a time: it may be large
-            w = P.permute_inner_dimensions(m32.w, m32.cfg, gen)
+        K = noise_draws(name)
+        for _ in range(K):
+            # float32: one permuted model at a time (it may be large); bfloat16: the model as it is, rounding drawn anew
+            w = P.permute_inner_dimensions(m32.w, m32.cfg, gen) if dtype == "float32" else m32.w
+            rnd = P._same if dtype == "float32" else P.dithered_bf16(gen)
             for toks in missing:
                 with torch.no_grad():
-                    e = P.forward(toks, w, m32.cfg).numpy().astype(np.float64) - plain_logits(name, toks)
+                    e = P.forward(toks, w, m32.cfg, rnd=rnd).numpy().astype(np.float64) - plain_logits(name, toks)
                 sq[tuple(toks)] = sq[tuple(toks)] + (e ** 2).mean(axis=1)
                 mx[tuple(toks)] = np.maximum(mx[tuple(toks)], np.abs(e).max(axis=1))
             del w
         for toks in missing:
-            _noise32_cache[name, tuple(toks)] = (np.sqrt(sq[tuple(toks)] / K), mx[tuple(toks)])
-    return {rid: _noise32_cache[name, tuple(toks)] for rid, toks in reqs.items()}
+            _noise_cache[name, dtype, tuple(toks)] = (np.sqrt(sq[tuple(toks)] / K), mx[tuple(toks)])
+    return {rid: _noise_cache[name, dtype, tuple(toks)] for rid, toks in reqs.items()}
 
 
 def compare(name, dtype, reqs, got, label):
+    noise = rounding_noise(name, dtype, reqs)
+    t_rms, t_max = noise_bounds(noise_draws(name))
+    f = NOISIER[dtype]
     worst = 0.0
-    noise32 = f32_noise(name, reqs) if dtype == "float32" else None
     for rid, toks in reqs.items():
         ref = plain_logits(name, toks)
         spread = float(ref.std())
         mine = np.stack([got[(rid, p)] for p in range(len(toks))])
         assert np.isfinite(mine).all()
-        err = np.abs(mine - ref)
-        if dtype == "float32":
-            rel = err.max(axis=1) / spread
-            worst = max(worst, float(rel.max()))
-            n_rms, n_max = noise32[rid]
-            t_rms, t_max = f32_bounds(f32_draws(name))
-            pos_rms = np.sqrt((err.astype(np.float64) ** 2).mean(axis=1))
-            a, b = pos_rms / n_rms, err.max(axis=1) / n_max
-            g = float(np.sqrt((pos_rms ** 2).mean() / (n_rms ** 2).mean()))
-            print(f"[replay] {label} {name} f32 {rid}: of the permuted float32 runs' own error: rms over the request {g:.2f}x, "
-                  f"a position's rms {np.median(a):.2f}x (median) {a.max():.2f}x (worst, bound {t_rms:.2f}), a position's largest "
-                  f"{b.max():.2f}x (bound {t_max:.2f}); worst {rel.max():.2e} of the spread, where the runs reach {n_max[int(rel.argmax())] / spread:.2e}")
-            assert a.max() <= t_rms, (f"{label} {name} float32: request {rid} position {int(a.argmax())}: rms error {a.max():.2f}x "
-                                      f"that of the permuted float32 runs there (first position above {t_rms:.2f}: {int(np.argmax(a > t_rms))})")
-            assert b.max() <= t_max, (f"{label} {name} float32: request {rid} position {int(b.argmax())}: largest error {b.max():.2f}x "
-                                      f"the largest of the permuted float32 runs there (bound {t_max:.2f})")
-            assert g <= F32_GLOBAL_RMS, f"{label} {name} float32: request {rid}: rms error {g:.2f}x that of the permuted float32 runs"
-        else:
-            noise_rms, noise_max, rounded = bf16_noise(name, toks)
-            rms = float(np.sqrt((err ** 2).mean()))
-            per_pos = np.sqrt((err ** 2).mean(axis=1))
-            worst = max(worst, rms / noise_rms)
-            print(f"[replay] {label} {name} bf16 {rid}: rms {rms / noise_rms:.2f}x max {err.max() / noise_max:.2f}x of the "
-                  f"rounding noise (rms {noise_rms / spread:.2e}, max {noise_max / spread:.2e} of the spread); "
-                  f"vs rounded plain: rms {np.sqrt(((mine - rounded) ** 2).mean()) / noise_rms:.2f}x")
-            assert np.sqrt(((mine - rounded) ** 2).mean()) <= BF16_VS_ROUNDED_FACTOR * noise_rms, \
-                f"{label} {name} bf16: request {rid} strays from the bfloat16-rounded plain computation"
-            assert rms <= BF16_RMS_FACTOR * noise_rms, \
-                f"{label} {name} bf16: request {rid}: rms error {rms / noise_rms:.2f}x the rounding noise"
-            assert err.max() <= BF16_MAX_FACTOR * noise_max, \
-                (f"{label} {name} bf16: request {rid}: max error {err.max() / noise_max:.2f}x the rounding noise, "
-                 f"first position above it {int(np.argmax(err.max(axis=1) > BF16_MAX_FACTOR * noise_max))}")
-            # no single position stands out: a fault at a page edge or at the start of a portion would
-            assert per_pos.max() <= 4.0 * BF16_RMS_FACTOR * noise_rms, \
-                f"{label} {name} bf16: request {rid}: position {int(per_pos.argmax())} is {per_pos.max() / noise_rms:.2f}x the noise"
-    print(f"[replay] {label} {name} {dtype}: worst {worst:.3e}")
+        err = np.abs(mine - ref).astype(np.float64)
+        n_rms, n_max = noise[rid]
+        pos_rms = np.sqrt((err ** 2).mean(axis=1))
+        a, b = pos_rms / n_rms, err.max(axis=1) / n_max
+        g = float(np.sqrt((pos_rms ** 2).mean() / (n_rms ** 2).mean()))
+        worst = max(worst, float(a.max()))
+        at = int(err.max(axis=1).argmax())
+        print(f"[replay] {label} {name} {dtype} {rid}: of the draws' own error: a position's rms {np.median(a):.2f}x (median, bound {f:.2f}) "
+              f"{a.max():.2f}x (worst, bound {f * t_rms:.2f}), a position's largest {b.max():.2f}x (bound {f * t_max:.2f}), rms over the "
+              f"request {g:.2f}x; worst {err.max() / spread:.2e} of the spread, where the draws reach {n_max[at] / spread:.2e}")
+        # no single position stands out: a fault at a page edge or at the start of a portion would
+        assert a.max() <= f * t_rms, (f"{label} {name} {dtype}: request {rid}: the rms error of position {int(a.argmax())} is {a.max():.2f}x that "
+                                      f"of the draws there (first position above {f * t_rms:.2f}: {int(np.argmax(a > f * t_rms))})")
+        assert b.max() <= f * t_max, (f"{label} {name} {dtype}: request {rid}: the largest error of position {int(b.argmax())} is {b.max():.2f}x "
+                                      f"the largest of the draws there (bound {f * t_max:.2f})")
+        # and the engine is no noisier than it may be where nothing is special (of fewer than 16 positions the median is
+        # hardly more than one position's draw, which the bounds above cover)
+        assert len(toks) < 16 or np.median(a) <= f, (f"{label} {name} {dtype}: request {rid}: the median position's rms error is "
+                                                     f"{np.median(a):.2f}x that of the draws (bound {f:.2f})")
+    print(f"[replay] {label} {name} {dtype}: worst position {worst:.2f}x the draws' rms there")
 
 
 LENGTHS = {"A": [70, 45, 100, 33, 64, 90], "B": [41, 97, 34, 80, 65, 50], "C": [50, 36, 81]}
@@ -386,10 +357,9 @@ def test_long_decoding_and_first_tokens():
         compare("A", dtype, reqs, got, "long decode")
         first = np.stack([got[("r0", p)] for p in range(4)])
         ref = plain_logits("A", toks)[:4]
-        if dtype == "float32":
-            assert (np.abs(first - ref).max(axis=1) <= f32_bounds(f32_draws("A"))[1] * f32_noise("A", reqs)["r0"][1][:4]).all()
-        else:
-            assert np.abs(first - ref).max() <= BF16_MAX_FACTOR * bf16_noise("A", toks)[1]
+        # (the first positions are among those that compare() has looked at one by one)
+        n_max = rounding_noise("A", dtype, reqs)["r0"][1][:4]
+        assert (np.abs(first - ref).max(axis=1) <= NOISIER[dtype] * noise_bounds(noise_draws("A"))[1] * n_max).all()
 
 
 def test_the_program_itself_in_a_subprocess():

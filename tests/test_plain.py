@@ -227,6 +227,19 @@ def test_a_model_with_its_inner_dimensions_permuted_is_the_same_function(name):
     assert float((b - ref).abs().max()) < 1e-4 * float(ref.std())        # of the same, small, size
 
 
+def test_dithered_rounding_errs_like_a_bfloat16_rounding_but_anew_every_time():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(200000, generator=g) * 3
+    rnd = P.dithered_bf16(g)
+    e0, e1, e2 = P.to_bf16(x) - x, rnd(x) - x, rnd(x) - x
+    ulp = torch.ldexp(torch.ones_like(x), torch.frexp(x)[1] - 8)
+    assert float((e1.abs() / ulp).max()) <= 0.5 + 1e-3                   # within half a unit in the last place (of x + d)
+    size = lambda e: float((e / x).pow(2).mean().sqrt())
+    assert abs(size(e1) / size(e0) - 1) < 0.02                           # the size of a rounding
+    corr = lambda a, b: float((a * b).mean() / (a.pow(2).mean() * b.pow(2).mean()).sqrt())
+    assert abs(corr(e1, e0)) < 0.02 and abs(corr(e1, e2)) < 0.02         # drawn anew
+
+
 def test_qkv_bias_is_used():
     m = _plain("A")
     w = {k: (torch.zeros_like(v) if k.endswith("_proj.bias") else v) for k, v in m.w.items()}
