@@ -303,7 +303,7 @@ def serve_point(model_dir, dtype, requests, max_new, model=None):
             "preemptions": eng.stats["preemptions"]}
 
 
-def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20):
+def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20, chunk_len=0):
     """The prefill attention kernel alone on ``nseq`` portions of ``new_len`` tokens after ``prefix`` cached ones,
     with the shape's heads; ``shape``: what FastAttention.prefill_teams would return, 0 = ask it."""
     import torch
@@ -322,9 +322,9 @@ def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20):
     cl = torch.full((nseq,), ctx, dtype=torch.int32, device=dev)
     fa = FastAttention(nq, nkv, d)
     shape = shape or fa.prefill_teams([new_len] * nseq, [ctx] * nseq)
-    run = lambda: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, teams=shape)
     out = torch.empty(nseq * new_len, nq * d, dtype=torch.bfloat16, device=dev)
-    run = lambda: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, out=out, teams=shape)
+    run = lambda: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, out=out, teams=shape, chunk_len=chunk_len,
+                             max_chunks=-(-ctx // chunk_len) if chunk_len else 0)
     for _ in range(5):
         run()
     torch.cuda.synchronize()
@@ -363,7 +363,7 @@ def main() -> int:
                     help="draw the random weights on the GPU instead of writing and reading a model folder")
     ap.add_argument("--requests", type=int, default=64, help="requests of the serve workload")
     ap.add_argument("--max-new", type=int, default=256, help="new tokens per request of the serve workload")
-    ap.add_argument("--attention", metavar="SEQS,NEW,PREFIX[,SHAPE]", default=None,
+    ap.add_argument("--attention", metavar="SEQS,NEW,PREFIX[,SHAPE[,CHUNK]]", default=None,
                     help="time only the prefill attention kernel on SEQS portions of NEW tokens after PREFIX cached ones")
     a = ap.parse_args()
     global CONFIG, CONTEXT
@@ -385,7 +385,8 @@ def main() -> int:
     from pico_vllm_amd.weights.random_init import write_random_model
     if a.attention:
         nums = [int(x) for x in a.attention.split(",")]
-        r = attention_point(CONFIG, nums[0], nums[1], nums[2], nums[3] if len(nums) > 3 else 0)
+        r = attention_point(CONFIG, nums[0], nums[1], nums[2], nums[3] if len(nums) > 3 else 0,
+                            chunk_len=nums[4] if len(nums) > 4 else 0)
         print(json.dumps({"metric": "prefill attention kernel", "unit": "us", "value": r["us"], "workgroup_shape": r["shape"],
                           "tflops": r["tflops"], "frac_of_bf16_peak": r["frac"], "sequences": nums[0], "new_tokens": nums[1],
                           "prefix": nums[2], "heads": CONFIG["num_attention_heads"], "kv_heads": CONFIG["num_key_value_heads"]}))

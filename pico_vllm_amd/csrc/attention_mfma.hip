@@ -412,6 +412,7 @@ constexpr int PF_BM = 64;                         // queries per workgroup
 constexpr int PF_KT_MAX = D <= 128 ? 2 : 1;       // 2: one, two or three teams of four waves; 1: one team
 constexpr int PF_KS = D / 32;                     // contraction steps of a 16-key block
 constexpr int PF_DT = D / 16;                     // 16-wide tiles of the output's head dimension
+constexpr int PF_PART_ROW = D + 4;                // floats of a chunk's partial result: D sums, the maximum, the sum of p, padding
 
 template <int KT>
 struct alignas(16) PfTiles {
@@ -636,7 +637,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
-    float scale, int reach) {
+    float scale, int reach, int chunk_len, int max_chunks, float* __restrict__ part) {
   static_assert(NQB == 1 || KT == 1, "two query blocks a wave: one team");
   constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
   constexpr int BMQ = PF_BM * NQB;            // queries per workgroup
@@ -652,6 +653,12 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   const int head = blockIdx.x, g = head / (nq / nkv);
   const int tok0 = cu_seqlens[b], new_len = cu_seqlens[b + 1] - tok0;
   const int ctx = context_lens[b], prefix = ctx - new_len;
+  const int tile_kv_end = min(ctx, prefix + min(new_len, (tile + 1) * BMQ));   // keys beyond the tile's last query are never needed
+  // chunk_len > 0: the keys of a tile are cut into chunks of that many (a multiple of the LDS tile; no window then),
+  // each a workgroup of its own (grid z); a tile of several chunks leaves partial results that pf_merge_kernel joins
+  const int n_chunks = chunk_len > 0 ? (tile_kv_end + chunk_len - 1) / chunk_len : 1;
+  const int chunk = chunk_len > 0 ? (int)blockIdx.z : 0;
+  if (chunk >= n_chunks) return;
   const int wave = (threadIdx.x >> 6) & 3, team = threadIdx.x >> 8;
   const int lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
   const int* bt = block_table + (size_t)b * max_pages;
@@ -676,7 +683,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   const int wave_first_pos = prefix + wave_q0;                              // lowest query position of the wave
   const int wave_last_pos = min(wave_first_pos + 16 * NQB - 1, ctx - 1);    // highest real one
   const bool wave_active = wave_q0 < new_len;
-  const int kv_end = min(ctx, prefix + min(new_len, (tile + 1) * BMQ));   // keys beyond the tile's last query are never needed
+  const int kv_end = chunk_len > 0 ? min(tile_kv_end, (chunk + 1) * chunk_len) : tile_kv_end;
 
   const float c = scale * 1.4426950408889634f;                 // scores go through 2^x
   const int pshift = 31 - __clz(P);                            // page sizes are powers of two
@@ -703,7 +710,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   const int n_full = (apart_ok && reach == NO_WINDOW && pshift <= 4 && page_bytes < (1u << 24) && num_pages < (1 << 24)) ? kv_end / PF_TK : 0;
   // the first key that the workgroup's first query still sees, and its tile
   const int kv_lo = max(0, prefix + tile * BMQ - reach + 1);
-  const int first_tile = kv_lo / PF_TK;
+  const int first_tile = chunk_len > 0 ? chunk * (chunk_len / PF_TK) : kv_lo / PF_TK;
   const int kv_begin = first_tile * PF_TK;
   regs.init(g, nkv, pshift);
   regs.load_pages(bt, pshift, num_pages, kv_begin, kv_end);
@@ -767,6 +774,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     const float m_use = (M == -INFINITY) ? 0.f : M;
     const float a0 = __builtin_amdgcn_exp2f((s0.m - m_use) * c);
     s0.l *= a0;
+    s0.m = M;                                                  // what the merged sums are relative to (a chunk's part says so)
 #pragma unroll
     for (int tt = 0; tt < PF_DT; tt++) s0.o[tt] *= a0;
 #pragma unroll
@@ -779,6 +787,25 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
 #pragma unroll
         for (int r = 0; r < 4; r++) s0.o[tt][r] += at * theirs[(4 * tt + r) * 64];
     }
+  }
+  if (n_chunks > 1) {
+    // this chunk's part of the tile: unnormalised sums, the reference maximum they are relative to, and the sum of
+    // the probabilities, per (token, head, chunk)
+#pragma unroll
+    for (int qb = 0; qb < NQB; qb++) {
+      if (!q_ok[qb]) continue;
+      float l = st[qb].l;
+      l += __shfl_xor(l, 16, 64);
+      l += __shfl_xor(l, 32, 64);
+      float* prow = part + (((size_t)(tok0 + q_idx[qb]) * nq + head) * max_chunks + chunk) * PF_PART_ROW + 4 * kq;
+#pragma unroll
+      for (int tt = 0; tt < PF_DT; tt++) *reinterpret_cast<f32x4p*>(prow + 16 * tt) = st[qb].o[tt];
+      if (kq == 0) {
+        prow[D] = st[qb].m;
+        prow[D + 1] = l;
+      }
+    }
+    return;
   }
 #pragma unroll
   for (int qb = 0; qb < NQB; qb++) {
@@ -796,6 +823,35 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
       *reinterpret_cast<uint2*>(orow + 16 * tt) = v;
     }
   }
+}
+
+// Joins the chunks of the tiles that prefill16_kernel cut (chunk_len > 0): out[token, head, :] =
+// sum_i 2^((m_i - M) c) o_i / sum_i 2^((m_i - M) c) l_i over the tile's chunks; tokens of a tile with one chunk have
+// their result already.  One workgroup per (token, head), one thread per head dimension.  bmq: queries per tile.
+__global__ __launch_bounds__(D) void pf_merge_kernel(const float* __restrict__ part, int max_chunks, int chunk_len,
+                                                     const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+                                                     int num_seqs, bf16_t* __restrict__ out, int nq, float scale, int bmq) {
+  const int t = blockIdx.x, head = blockIdx.y, dim = threadIdx.x;
+  int b = 0;
+  while (b + 1 < num_seqs && cu_seqlens[b + 1] <= t) b++;
+  const int tok0 = cu_seqlens[b], new_len = cu_seqlens[b + 1] - tok0;
+  if (t < tok0 || t - tok0 >= new_len) return;      // a token in front of the portions (a decode row of a mixed step), or none
+  const int ctx = context_lens[b], prefix = ctx - new_len, tile = (t - tok0) / bmq;
+  const int tile_kv_end = min(ctx, prefix + min(new_len, (tile + 1) * bmq));
+  const int n_chunks = (tile_kv_end + chunk_len - 1) / chunk_len;
+  if (n_chunks <= 1) return;
+  const float c = scale * 1.4426950408889634f;
+  const float* rows = part + ((size_t)t * nq + head) * max_chunks * PF_PART_ROW;
+  float M = -INFINITY;
+  for (int i = 0; i < n_chunks; i++) M = fmaxf(M, rows[i * PF_PART_ROW + D]);
+  float o = 0.f, l = 0.f;
+  for (int i = 0; i < n_chunks; i++) {
+    const float m = rows[i * PF_PART_ROW + D];
+    const float a = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m - M) * c);     // a chunk that this query sees no key of
+    o += a * rows[i * PF_PART_ROW + dim];
+    l += a * rows[i * PF_PART_ROW + D + 1];
+  }
+  out[((size_t)t * nq + head) * D + dim] = f32_to_bf16(o / l);
 }
 #endif
 
@@ -1148,45 +1204,61 @@ static int check_common(const char* who, int nq, int nkv, int d, int P, int max_
 
 extern "C" int pico_attn_head_dim() { return D; }
 
-// teams: 1 or 2 waves per SIMD share the key loop of a query tile (0: the default, 2 where the head
-// size allows it); a hint, any value gives the same result up to rounding
+// teams: the shape of the workgroups (1 to 3 teams of four waves that share the key loop of a 64-query tile; 4: one
+// team of 128 queries; 0: two teams where the head size allows it); a hint, any value gives the same result up to
+// rounding.  chunk_len > 0 (a multiple of 128, no window, not three teams, head sizes in steps of 32): the keys of every tile are cut
+// into chunks of that many, each a workgroup of its own, and a second launch joins the chunks of a tile; part is
+// their workspace, float32 [num_tokens, nq, max_chunks, D + 4], and max_chunks at least ceil(longest context / chunk_len).
 extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int* block_table, int max_pages, const int* cu_seqlens,
                                  const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
-                                 int d, int P, int num_pages, float scale, int teams, int window, hipStream_t stream) {
+                                 int d, int P, int num_pages, float scale, int teams, int window, int chunk_len,
+                                 int max_chunks, float* part, hipStream_t stream) {
   if (check_common("pico_attn_prefill", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
   PICO_REQUIRE(window >= 0 && window < NO_WINDOW, "pico_attn_prefill: bad window %d", window);
   const int reach = window > 0 ? window : NO_WINDOW;
   PICO_REQUIRE(num_seqs > 0 && num_tokens >= num_seqs, "pico_attn_prefill: bad batch (%d sequences, %d tokens)", num_seqs, num_tokens);
   PICO_REQUIRE(nq <= 65535, "pico_attn_prefill: too many heads");
   PICO_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "pico_attn_prefill: misaligned tensors");
+  PICO_REQUIRE(chunk_len >= 0, "pico_attn_prefill: bad chunk length %d", chunk_len);
 #if PICO_HEAD_DIM % 32 == 0
   // the 16-query kernel addresses the cache with 32-bit byte offsets
   if ((uint64_t)num_pages * nkv * P * D * sizeof(bf16_t) < (1ull << 32)) {
     const int max_tiles = num_tokens / PF_BM + num_seqs;  // >= sum over sequences of ceil(len / PF_BM)
     PICO_REQUIRE(max_tiles <= 65535, "pico_attn_prefill: %d tokens are too many for one launch", num_tokens);
     dim3 grid(nq, max_tiles);
+    if (chunk_len > 0) {
+      // (a chunk holds whole LDS tiles of every team shape but the one with three teams, whose tiles are 192 keys)
+      PICO_REQUIRE(window == 0 && teams != 3 && chunk_len % 128 == 0 && max_chunks >= 1 && max_chunks <= 64 &&
+                       part != nullptr && (uintptr_t)part % 16 == 0,
+                   "pico_attn_prefill: chunks of keys need no window, one or two teams, a length that is a multiple of 128 "
+                   "(got %d), 1 to 64 chunks (got %d) and an aligned workspace", chunk_len, max_chunks);
+      grid.z = max_chunks;
+    }
+    int bmq = PF_BM;
+#define PF_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, \
+                cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach, chunk_len, max_chunks, part
     if (teams == 4 && PF_KT_MAX == 2) {      // 128 queries a workgroup, two blocks of 16 a wave
       grid.y = num_tokens / (2 * PF_BM) + num_seqs;
-      prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 256, 0, stream>>>(
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
-          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
+      bmq = 2 * PF_BM;
+      prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 256, 0, stream>>>(PF_ARGS);
     } else if (teams == 1 || PF_KT_MAX == 1)
-      prefill16_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-                                                   (const bf16_t*)v_cache, block_table, max_pages, cu_seqlens,
-                                                   context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
+      prefill16_kernel<1><<<grid, 256, 0, stream>>>(PF_ARGS);
     else if (teams == 3 && PF_KT_MAX == 2)
-      prefill16_kernel<PF_KT_MAX == 2 ? 3 : 1><<<grid, 768, 0, stream>>>(
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
-          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
+      prefill16_kernel<PF_KT_MAX == 2 ? 3 : 1><<<grid, 768, 0, stream>>>(PF_ARGS);
     else
-      prefill16_kernel<PF_KT_MAX><<<grid, 256 * PF_KT_MAX, 0, stream>>>(
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
-          cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach);
+      prefill16_kernel<PF_KT_MAX><<<grid, 256 * PF_KT_MAX, 0, stream>>>(PF_ARGS);
+#undef PF_ARGS
     PICO_LAUNCH_CHECK();
+    if (chunk_len > 0 && max_chunks > 1) {
+      pf_merge_kernel<<<dim3(num_tokens, nq), D, 0, stream>>>(part, max_chunks, chunk_len, cu_seqlens, context_lens, num_seqs,
+                                                             (bf16_t*)out, nq, scale, bmq);
+      PICO_LAUNCH_CHECK();
+    }
     return 0;
   }
 #endif
+  PICO_REQUIRE(chunk_len == 0, "pico_attn_prefill: chunks of keys are for head sizes in steps of 32 and caches below 4 GiB");
   const int max_tiles = num_tokens / BM + num_seqs;       // >= sum over sequences of ceil(len / BM)
   dim3 grid(max_tiles, nq);
   prefill_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,

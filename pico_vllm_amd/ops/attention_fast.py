@@ -77,10 +77,52 @@ class FastAttention:
             return 3
         return 4 if total * self.nq >= cus * 64 and 4 * tokens >= 3 * padded else 1
 
+    def prefill_chunks(self, new_lens, context_lens):
+        """(shape, chunk_len, max_chunks) when the keys of the query tiles are better cut into chunks that run as
+        workgroups of their own and are joined by a second launch, or None.  That pays where whole tiles leave
+        compute units idle or a last round of workgroups nearly empty: portions behind a long prefix with few
+        heads or few query tiles (2,048 tokens of 12 heads after 14,336: 341 against 539 us; of 40 heads after
+        30,720: 1.70 against 2.20 ms; 512 tokens of 12 heads after 7,680: 69 against 133 us), and not where there
+        is work for every unit anyway (28 heads: no gain) or no prefix (the causal triangle's tiles are short).
+        The cost of a cut into S chunks is counted in passes of a workgroup over all keys: rounds of workgroups
+        over the chip's places, each 1/S long, plus what the partial results cost to write, read and join (with 8
+        chunks of 2,048 tokens of 12 heads the second launch reads 104 MB and takes 25 us)."""
+        if self.window or self.d % 32:
+            return None
+        tokens = int(sum(int(n) for n in new_lens))
+        keys = int(sum(int(c) for c in context_lens))
+        longest = max(int(c) for c in context_lens)
+        if keys - tokens < tokens or longest < 2048:               # the prefix is the smaller part of the work, or short
+            return None
+        padded = sum(-(-int(n) // 128) * 128 for n in new_lens)
+        shape = 4 if 4 * tokens >= 3 * padded else 1               # 128-query tiles where the portions fill them
+        per_tile, resident = (128, 2) if shape == 4 else (64, 3)
+        workgroups = sum(-(-int(n) // per_tile) for n in new_lens) * self.nq
+        places = self.cus * resident
+        # whole tiles: rounds of workgroups, the last one as good as full when the tiles' lengths differ (long ones
+        # start first and short ones fill the gaps), nearly empty when the prefix makes them all alike
+        rounds, alike = workgroups / places, (keys - tokens) / keys
+        whole = max(1.0, rounds + alike * (-(-workgroups // places) - rounds))
+        best, choice = 0.8 * whole, None
+        for want in (2, 4, 8, 16):
+            chunk_len = 512
+            while chunk_len * want < longest:
+                chunk_len *= 2                                     # powers of two: few different recorded steps
+            chunks = -(-longest // chunk_len)
+            if chunks < 2:
+                continue
+            cost = -(-workgroups * chunks // places) / chunks + 8.0 * chunks / (longest / 64)
+            if cost < best:
+                best, choice = cost, (shape, chunk_len, want)
+        return choice
+
     def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
-                scale: float, out: Optional[torch.Tensor] = None, teams: int = 0) -> torch.Tensor:
+                scale: float, out: Optional[torch.Tensor] = None, teams: int = 0, chunk_len: int = 0,
+                max_chunks: int = 0) -> torch.Tensor:
         """q [T, >= nq*d] bfloat16 (row stride free); any mixture of portions; returns [T, nq*d].
-        teams: 0 lets the kernel choose, else the result of ``prefill_teams``."""
+        teams: 0 lets the kernel choose, else the result of ``prefill_teams``.  chunk_len > 0: the keys of every
+        query tile are cut into chunks of that many, each a workgroup of its own (``max_chunks`` of them cover the
+        longest context), and a second launch joins them."""
         nq, nkv, d = self.nq, self.nkv, self.d
         T = q.shape[0]
         pages, P = _check_cache(k_cache, v_cache, nkv, d)
@@ -88,10 +130,17 @@ class FastAttention:
         self._check_meta(block_table, cu_seqlens, num_seqs + 1, context_lens, num_seqs)
         if out is None:
             out = torch.empty(T, nq * d, dtype=torch.bfloat16, device=q.device)
+        part = None
+        if chunk_len and k_cache.numel() * k_cache.element_size() >= (1 << 32):
+            chunk_len = max_chunks = 0          # the kernel that cuts keys into chunks addresses the cache with 32 bits
+        if chunk_len:
+            if self.window or d % 32 or max_chunks < 1:
+                raise KernelError("chunks of keys: no window, a head size in steps of 32 and at least one chunk")
+            part = torch.empty(T * nq * max_chunks * (d + 4), dtype=torch.float32, device=q.device)
         _check(self.lib, self.lib.pico_attn_prefill(
             _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens), _ptr(context_lens), num_seqs, T, _ptr(out), nq, nkv, d, P, pages, c_float(scale),
-            teams, self.window, _stream()))
+            teams, self.window, chunk_len, max_chunks, _ptr(part), _stream()))
         return out
 
     def decode(self, q: torch.Tensor, k_cache, v_cache, block_table, context_lens, num_seqs: int, scale: float,
@@ -130,19 +179,24 @@ class FastAttention:
                 raise KernelError("sequence metadata must be contiguous int32")
 
     def plan(self, ctx) -> tuple:
-        """(teams, lead) of a step with prompt portions: the shape of the prefill workgroups and how many single
-        tokens stand first.  Decided on the host from the shape of the batch, once for every layer of the step."""
+        """(teams, lead, chunk_len, max_chunks) of a step with prompt portions: the shape of the prefill workgroups,
+        how many single tokens stand first, and into what chunks the keys are cut (0, 0: whole).  Decided on the host
+        from the shape of the batch, once for every layer of the step."""
         key = ("fast_attention", self.nq, self.nkv, self.d, self.window)
         if key not in ctx.shared:
             B = ctx.num_seqs
-            teams, lead = 0, 0
+            teams, lead, chunk_len, max_chunks = 0, 0, 0, 0
             if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
                 cu = ctx.host["cu_seqlens"]
                 lens = cu[1:B + 1] - cu[:B]
                 while lead < B and lens[lead] == 1:
                     lead += 1
-                teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
-            ctx.shared[key] = (int(teams), int(lead))
+                if lead < B:
+                    teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
+                    cut = self.prefill_chunks(lens[lead:], ctx.host["context_lens"][lead:B])
+                    if cut is not None:
+                        teams, chunk_len, max_chunks = cut
+            ctx.shared[key] = (int(teams), int(lead), int(chunk_len), int(max_chunks))
         return ctx.shared[key]
 
     def __call__(self, qkv, cache, block_table, ctx, scale):
@@ -151,9 +205,10 @@ class FastAttention:
         if ctx.all_decode and grouped:
             return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, B, scale,
                                self.num_splits(B, ctx.max_context))
-        teams, lead = self.plan(ctx)
+        teams, lead, chunk_len, max_chunks = self.plan(ctx)
         if lead == 0 or not grouped:
-            return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, scale, teams=teams)
+            return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, scale, teams=teams,
+                                chunk_len=chunk_len, max_chunks=max_chunks)
         # A mixed step: the scheduler puts the decoding requests first.  Their tokens (one row each, rows
         # 0 .. lead - 1) go through the decode kernel, which reads keys and values once for all query heads of
         # a group; the prompt portions behind them through the prefill kernel, whose offsets are absolute.
@@ -162,7 +217,7 @@ class FastAttention:
                     self.num_splits(lead, ctx.max_context), out=out[:lead])
         if lead < B:
             self.prefill(qkv, cache.k, cache.v, block_table[lead:], ctx.cu_seqlens[lead:], ctx.context_lens[lead:],
-                         B - lead, scale, out=out, teams=teams)
+                         B - lead, scale, out=out, teams=teams, chunk_len=chunk_len, max_chunks=max_chunks)
         return out
 
 

@@ -342,7 +342,7 @@ def test_sampling_top_p(K):
 
 # ---- matrix-core attention (bfloat16) ----------------------------------------------------------
 def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0, as_step=False,
-               window=0):
+               window=0, chunk_len=0, max_chunks=0):
     from pico_vllm_amd.ops.attention_fast import FastAttention
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(seed)
@@ -371,7 +371,8 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
     elif decode:
         out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
     else:
-        out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale, teams=teams)
+        out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale, teams=teams, chunk_len=chunk_len,
+                         max_chunks=max_chunks or (-(-max(totals) // chunk_len) if chunk_len else 0))
     want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n), window=window)
                       for qb, kb, vb, n, p in zip(qs, ks, vs, new_lens, prefix_lens)], 0)
     return out.reshape(-1, nq, d), want
@@ -484,6 +485,55 @@ def test_fast_attention_of_a_step_with_much_work(K):
     fa.nq = 16
     assert fa.prefill_teams([256] * 8, [2304] * 8) == 4
     out, want = _fast_case([256] * 8, [2048] * 8, 16, 4, 32, 16, seed=13, as_step=True)
+    close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("teams", [0, 1, 2, 4])
+@pytest.mark.parametrize("nq,nkv,d,Pg,chunk_len", [(12, 2, 128, 16, 256), (6, 3, 32, 8, 128), (2, 2, 64, 8, 384), (4, 1, 96, 32, 128),
+                                                  (4, 2, 256, 16, 512), (2, 1, 160, 8, 256)])
+def test_fast_prefill_with_the_keys_cut_into_chunks(K, nq, nkv, d, Pg, chunk_len, teams):
+    # every chunk of a tile's keys is a workgroup of its own and a second launch joins them: tiles of one chunk and of
+    # many in one batch, a chunk's edge inside a tile's own positions (its first queries see no key of the last
+    # chunk), portions of one and two tokens, a context that ends one key into a chunk, more room for chunks than needed;
+    # queries are scaled up so that few keys carry a row's weight and a chunk that is lost or joined wrongly shows
+    def boost(qs, ks, vs):
+        for q in qs:
+            q *= 2.0
+    new_lens, prefix_lens = [300, 77, 1, 130, 2, 64], [1000, 0, 555, 2 * chunk_len - 129, chunk_len - 1, 3 * chunk_len]
+    out, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=chunk_len + d, boost=boost, teams=teams, chunk_len=chunk_len)
+    close(out, want, torch.bfloat16)
+    more, _ = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=chunk_len + d, boost=boost, teams=teams, chunk_len=chunk_len,
+                         max_chunks=-(-max(n + p for n, p in zip(new_lens, prefix_lens)) // chunk_len) + 3)
+    assert torch.equal(out, more)
+
+
+def test_fast_prefill_refuses_chunks_it_cannot_cut(K):
+    from pico_vllm_amd.ops.kernels import KernelError
+    for kw in (dict(teams=3, chunk_len=256), dict(teams=1, chunk_len=200), dict(teams=1, chunk_len=256, window=50),
+               dict(teams=1, chunk_len=256, max_chunks=65)):
+        with pytest.raises(KernelError):
+            _fast_case([70], [300], 4, 2, 64, 16, **kw)
+    with pytest.raises(KernelError):            # a head size that the 16-query kernel does not serve
+        _fast_case([70], [300], 4, 2, 48, 16, teams=1, chunk_len=256)
+
+
+def test_a_step_behind_a_long_prefix_cuts_its_keys_into_chunks(K):
+    # the host's choice (FastAttention.prefill_chunks) and the step that it serves
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    fa = FastAttention.__new__(FastAttention)
+    fa.nq, fa.nkv, fa.d, fa.window, fa.cus = 12, 2, 128, 0, 256
+    assert fa.prefill_chunks([2048], [2048]) is None                    # no prefix: short tiles
+    assert fa.prefill_chunks([2048] * 8, [4096] * 8) is None            # work for every compute unit
+    assert fa.prefill_chunks([2048], [16384]) == (4, 8192, 2)           # 192 workgroups of 256 key tiles each on 512 places
+    assert fa.prefill_chunks([2048], [32768]) == (4, 4096, 8)
+    assert fa.prefill_chunks([64], [8064]) == (1, 2048, 4)              # one tile per head
+    fa.nq = 28
+    assert fa.prefill_chunks([2048], [16384]) is None                   # 448 workgroups on 512 places
+    fa.window = 100
+    assert fa.prefill_chunks([64], [8064]) is None
+    fa.nq, fa.nkv, fa.d, fa.window = 4, 2, 64, 0
+    assert fa.prefill_chunks([64, 70], [8064, 7070]) == (1, 2048, 4)
+    out, want = _fast_case([1, 64, 70], [300, 8000, 7000], 4, 2, 64, 16, seed=21, as_step=True)      # behind a decode row
     close(out, want, torch.bfloat16)
 
 
