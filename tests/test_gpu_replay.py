@@ -45,11 +45,12 @@ FALSE_ALARM = 1e-5
 NOISIER = {"float32": 1.0, "bfloat16": 1.5}
 
 
-def noise_draws(name) -> int:
-    """How many runs make the yardstick: 32 for the tiny models, fewer where one run takes seconds."""
+def noise_draws(name, longest: int = 0) -> int:
+    """How many runs make the yardstick: 32 for the tiny models, fewer where one run takes seconds (a large model, or
+    a request of thousands of tokens)."""
     c = CONFIGS[name]
     params = c["num_hidden_layers"] * c["hidden_size"] * (3 * c["intermediate_size"] + 4 * c["hidden_size"]) + c["vocab_size"] * c["hidden_size"]
-    return 32 if params <= 20e6 else 16 if params <= 1e9 else 8
+    return 32 if params <= 20e6 and longest <= 2048 else 16 if params <= 1e9 else 8
 
 
 @functools.lru_cache(maxsize=None)
@@ -197,7 +198,7 @@ _noise_cache = {}
 
 
 def rounding_noise(name, dtype, reqs):
-    """For every request: (rms [positions], largest [positions]) of the logit errors of ``noise_draws(name)`` runs of
+    """For every request: (rms [positions], largest [positions], the number of runs) of the logit errors of ``noise_draws`` runs of
     the plain implementation with the rounding of ``dtype`` (see the top of the file) against the plain float64 run,
     over the draws and the vocabulary."""
     missing = [toks for toks in reqs.values() if (name, dtype, tuple(toks)) not in _noise_cache]
@@ -207,7 +208,7 @@ def rounding_noise(name, dtype, reqs):
         gen = torch.Generator().manual_seed(1234)
         sq = {tuple(t): 0.0 for t in missing}
         mx = {tuple(t): 0.0 for t in missing}
-        K = noise_draws(name)
+        K = noise_draws(name, max(len(t) for t in reqs.values()))
         for _ in range(K):
             # float32: one permuted model at a time (it may be large); bfloat16: the model as it is, rounding drawn anew
             w = P.permute_inner_dimensions(m32.w, m32.cfg, gen) if dtype == "float32" else m32.w
@@ -219,13 +220,12 @@ def rounding_noise(name, dtype, reqs):
                 mx[tuple(toks)] = np.maximum(mx[tuple(toks)], np.abs(e).max(axis=1))
             del w
         for toks in missing:
-            _noise_cache[name, dtype, tuple(toks)] = (np.sqrt(sq[tuple(toks)] / K), mx[tuple(toks)])
+            _noise_cache[name, dtype, tuple(toks)] = (np.sqrt(sq[tuple(toks)] / K), mx[tuple(toks)], K)
     return {rid: _noise_cache[name, dtype, tuple(toks)] for rid, toks in reqs.items()}
 
 
 def compare(name, dtype, reqs, got, label):
     noise = rounding_noise(name, dtype, reqs)
-    t_rms, t_max = noise_bounds(noise_draws(name))
     f = NOISIER[dtype]
     worst = 0.0
     for rid, toks in reqs.items():
@@ -234,7 +234,8 @@ def compare(name, dtype, reqs, got, label):
         mine = np.stack([got[(rid, p)] for p in range(len(toks))])
         assert np.isfinite(mine).all()
         err = np.abs(mine - ref).astype(np.float64)
-        n_rms, n_max = noise[rid]
+        n_rms, n_max, draws = noise[rid]
+        t_rms, t_max = noise_bounds(draws)
         pos_rms = np.sqrt((err ** 2).mean(axis=1))
         a, b = pos_rms / n_rms, err.max(axis=1) / n_max
         g = float(np.sqrt((pos_rms ** 2).mean() / (n_rms ** 2).mean()))
@@ -318,6 +319,28 @@ def test_prompts_of_several_whole_key_tiles_at_head_size_96(dtype):
     compare("E", dtype, reqs, got, "tail")
 
 
+def test_a_context_of_thousands_of_tokens_in_portions_of_2048(monkeypatch):
+    # 6,200 tokens: whole in one step, and in portions of 2,048, 2,048, 2,048 and 52 with the last tokens one by
+    # one.  Behind 4,096 tokens and more the bfloat16 attention cuts a portion's keys into chunks that run as workgroups
+    # of their own (ops/attention_fast.py, prefill_chunks); a chunk lost or joined wrongly would move a row by a
+    # quarter of its weight.
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    cuts = []
+    chosen = FastAttention.prefill_chunks
+    monkeypatch.setattr(FastAttention, "prefill_chunks", lambda self, n, c: cuts.append(chosen(self, n, c)) or cuts[-1])
+    reqs = make_requests("F", [6200], seed=31)
+    for dtype in ("bfloat16", "float32"):
+        got, _ = replay("F", dtype, whole(reqs))
+        compare("F", dtype, reqs, got, "long whole")
+        del cuts[:]
+        got, _ = replay("F", dtype, portions(reqs, sizes=(2048, 2048, 2048, 52, 1, 1, 1, 1)))
+        compare("F", dtype, reqs, got, "long portions")
+        if dtype == "bfloat16":
+            assert any(c is not None for c in cuts), cuts          # the portions behind a long prefix were cut
+    for key in [k for k in _plain_cache if k == "F" or (isinstance(k, tuple) and k[0] == "F")]:
+        del _plain_cache[key]
+
+
 def test_fifty_more_drawn_configurations_in_every_way_of_cutting():
     # a sweep over sizes nobody looked at, in both precisions, whole, with the tail token by token and mixed in a
     # small pool; it stops at the first configuration that fails and names it
@@ -358,8 +381,8 @@ def test_long_decoding_and_first_tokens():
         first = np.stack([got[("r0", p)] for p in range(4)])
         ref = plain_logits("A", toks)[:4]
         # (the first positions are among those that compare() has looked at one by one)
-        n_max = rounding_noise("A", dtype, reqs)["r0"][1][:4]
-        assert (np.abs(first - ref).max(axis=1) <= NOISIER[dtype] * noise_bounds(noise_draws("A"))[1] * n_max).all()
+        _, n_max, draws = rounding_noise("A", dtype, reqs)["r0"]
+        assert (np.abs(first - ref).max(axis=1) <= NOISIER[dtype] * noise_bounds(draws)[1] * n_max[:4]).all()
 
 
 def test_the_program_itself_in_a_subprocess():

@@ -31,8 +31,14 @@ TINY_E = {   # head size 96 (three chunks of 32; its 12 chunks of 16 bytes a key
     "num_key_value_heads": 2, "head_dim": 96, "intermediate_size": 232, "rms_norm_eps": 3e-6,
     "rope_theta": 100000.0, "tie_word_embeddings": True, "max_position_embeddings": 2048, "hidden_act": "silu",
 }
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+TINY_F = {   # for contexts of thousands of tokens: two heads of 64 on one kv head, positions up to 16,384
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 299, "hidden_size": 128, "num_hidden_layers": 2, "num_attention_heads": 2,
+    "num_key_value_heads": 1, "intermediate_size": 264, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
+    "tie_word_embeddings": False, "max_position_embeddings": 16384, "hidden_act": "silu",
+}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "F": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
 
 
 def drawn(seed: int):
