@@ -1,6 +1,6 @@
 """Each part alone against the plain function of the same part, a model whose run order names a
-layer twice, and a toy mixer with state of its own that the test registers without touching the
-framework."""
+layer twice, and toy parts of every kind (a mixer with state of its own, a feed-forward with routing, a position
+encoding, a norm, an arrangement) that the tests register without touching the framework."""
 
 import pytest
 import torch
@@ -710,3 +710,128 @@ def test_layers_with_and_without_a_window_in_one_model(dtype):
         assert windowed.pool.peak_used < 20 and windowed.pool.num_used < [gr for gr in m.groups if not gr.window][0].pool.num_used
         for rid, toks in (("a", a), ("b", b)):
             close_to_plain(torch.cat(got[rid]), want(toks, P._same), want(toks, P.to_bf16), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_toy_norm_and_a_toy_arrangement_of_the_parts(dtype):
+    """The two remaining kinds of part, defined and registered here: a norm that centres on the mean and has a
+    bias (the framework's subtracts nothing and has none), and an arrangement in which the mixer and the
+    feed-forward read the same normed activations and their outputs are added together,
+    x += mixer(norm(x)) + ff(norm(x)), one norm a layer.  Mixer, feed-forward and position encoding are the
+    framework's.  The whole prompt equals a plain computation written out below, portions beside another request
+    equal the whole, and the entry point generates with the model from graphs as without."""
+    import tempfile
+    from pico_vllm_amd import LLM, SamplingParams
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.base import Block, Norm
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import LayerSpec, ModelSpec, ParamSpec, PartSpec, RunEntry
+    from pico_vllm_amd.weights.random_init import write_random_model
+
+    H, V, NQ, NKV, D, I, EPS, THETA = 48, 77, 3, 3, 16, 40, 1e-4, 300.0
+
+    def flat(delta):                 # a part's output: [T, H], or a float32 stack of partial sums
+        delta = delta.float()
+        return delta.sum(0) if delta.dim() == 3 else delta
+
+    @register_part("norm", "toy_centred_norm")
+    class CentredNorm(Norm):
+        def __init__(self, size, eps, act_dtype=torch.bfloat16):
+            self.size, self.eps, self.act_dtype = size, eps, act_dtype
+
+        def param_specs(self):
+            return [ParamSpec("weight", (self.size,), role="norm"), ParamSpec("bias", (self.size,), role="bias")]
+
+        def load(self, tensors, device, dtype):
+            self.weight, self.bias = tensors["weight"].to(device).float(), tensors["bias"].to(device).float()
+
+        def add_norm(self, resid, delta, rows=None):
+            if rows is None:
+                if delta is not None:
+                    resid += flat(delta)
+                x = resid
+            else:
+                x = resid[rows.long()] + (flat(delta)[rows.long()] if delta is not None else 0.0)
+            x = x - x.mean(-1, keepdim=True)
+            return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight + self.bias).to(self.act_dtype)
+
+    @register_part("block", "toy_side_by_side")
+    class SideBySide(Block):
+        slot_categories = {"norm": "norm", "mixer": "mixer", "ff": "feed_forward"}
+
+        def forward(self, resid, pending, ctx, cache):
+            h = self.parts["norm"].add_norm(resid, pending)
+            return resid, flat(self.parts["mixer"].forward(h, ctx, cache)) + flat(self.parts["ff"].forward(h, ctx))
+
+    def toy_spec(cfg):
+        norm = PartSpec("toy_centred_norm", {"size": H, "eps": EPS})
+        attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": D, "qkv_bias": True,
+                                          "window": 0, "position": PartSpec("rotary_half", {"rotary_dim": D, "theta": THETA})})
+        ff = PartSpec("swiglu_mlp", {"hidden_size": H, "intermediate_size": I})
+        layers = [LayerSpec(f"toy.layers.{i}", "toy_side_by_side", {"norm": ("ln", norm), "mixer": ("attn", attn), "ff": ("ff", ff)})
+                  for i in range(3)]
+        return ModelSpec(H, V, "toy.embed.weight", layers, [RunEntry(i) for i in range(3)], norm, "toy.norm", None)
+
+    register_architecture("ToySideBySideLM", lambda raw: raw, toy_spec)
+    rnd = P._same if dtype == torch.float32 else P.to_bf16
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, {"architectures": ["ToySideBySideLM"]}, seed=6,
+                           std_overrides={"attn": 0.4, "embed": 0.5, "ff.gate": 0.3, "ff.up": 0.3, "ff.down": 0.3, ".bias": 0.3})
+        w = {k: v.float() for k, v in P.read_weights(d).items()}
+        assert float(w["toy.layers.0.ln.bias"].abs().max()) > 0.1
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        assert not model.is_graph_safe(prompts=True) and model.is_graph_safe()      # the toy parts did not opt in for prompts
+        r = ModelRunner(model, 8, 16, 3, 64, 64)
+        toks = torch.randint(0, V, (41,), generator=torch.Generator().manual_seed(2)).tolist()
+
+        def centred(x, p):
+            x = x - x.mean(-1, keepdim=True)
+            return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + EPS) * w[f"{p}.weight"] + w[f"{p}.bias"]
+
+        def plain(rnd):              # the whole sequence, no cache
+            pos = torch.arange(len(toks))
+            x = w["toy.embed.weight"][toks]
+            cos, sin = P.rope_tables(pos, D, THETA)
+            for i in range(3):
+                p = f"toy.layers.{i}"
+                h = rnd(centred(x, f"{p}.ln"))
+                W = torch.cat([w[f"{p}.attn.{n}_proj.weight"] for n in "qkv"], 0)
+                b = torch.cat([w[f"{p}.attn.{n}_proj.bias"] for n in "qkv"], 0)
+                q, k, v = P.split_qkv(rnd(h @ W.T + b), NQ, NKV, D)
+                o = rnd(P.causal_attention(rnd(P.apply_rope(q, cos, sin)), rnd(P.apply_rope(k, cos, sin)), v,
+                                           rnd_p=None if rnd is P._same else rnd))
+                a = rnd(o.reshape(len(toks), NQ * D) @ w[f"{p}.attn.o_proj.weight"].T)
+                gu = torch.cat([w[f"{p}.ff.gate_proj.weight"], w[f"{p}.ff.up_proj.weight"]], 0)
+                f = rnd(rnd(P.swiglu(rnd(h @ gu.T))) @ w[f"{p}.ff.down_proj.weight"].T)
+                x = x + a + f                                            # both read h, neither the other's output
+            return rnd(centred(x, "toy.norm")) @ w["toy.embed.weight"].T
+
+        want = plain(P._same)
+        r.manager.add_request("w")
+        assert r.manager.grow("w", len(toks))
+        whole_logits = r.step([SeqStep("w", toks, list(range(len(toks))))])
+        r.manager.free_request("w")
+        close_to_plain(whole_logits, want, plain(rnd), dtype)
+        r.manager.add_request("a")
+        r.manager.add_request("b")
+        got, fed = [], 0
+        for n, nb in ((9, 2), (1, 1), (2, 5), (22, 1), (7, 1)):
+            assert r.manager.grow("a", fed + n) and r.manager.grow("b", r.manager.num_computed("b") + nb)
+            seqs = [SeqStep("b", toks[:nb], []), SeqStep("a", toks[fed:fed + n], list(range(n)))]
+            got.append(r.step(seqs))
+            r.advance(seqs)
+            fed += n
+        close(torch.cat(got), whole_logits, dtype, scale=float(whole_logits.std()) * 3)
+        del r, model
+        # through the entry point, decode steps from graphs and without: the same tokens, and the plain argmax
+        outs = []
+        for graphs in (True, False):
+            llm = LLM(model=d, dtype="float32" if dtype == torch.float32 else "bfloat16", max_seq_len=64, max_num_seqs=2,
+                      num_gpu_blocks=16, block_size=8, use_cuda_graph=graphs)
+            assert llm.engine.runner.use_graph == graphs and not llm.engine.runner.graph_prompts
+            outs.append([o.token_ids for o in llm.generate([toks[:9], toks[5:20]], SamplingParams(max_new_tokens=6, temperature=0.0))])
+            del llm
+        assert outs[0] == outs[1]
