@@ -50,7 +50,7 @@ def noise_draws(name, longest: int = 0) -> int:
     a request of thousands of tokens)."""
     c = CONFIGS[name]
     params = c["num_hidden_layers"] * c["hidden_size"] * (3 * c["intermediate_size"] + 4 * c["hidden_size"]) + c["vocab_size"] * c["hidden_size"]
-    return 32 if params <= 20e6 and longest <= 2048 else 16 if params <= 1e9 else 8
+    return 32 if params <= 20e6 and longest <= 2048 else 16 if params <= 100e6 else 8
 
 
 @functools.lru_cache(maxsize=None)
@@ -341,11 +341,11 @@ def test_a_context_of_thousands_of_tokens_in_portions_of_2048(monkeypatch):
         del _plain_cache[key]
 
 
-def test_fifty_more_drawn_configurations_in_every_way_of_cutting():
+def test_forty_more_drawn_configurations_in_every_way_of_cutting():
     # a sweep over sizes nobody looked at, in both precisions, whole, with the tail token by token and mixed in a
     # small pool; it stops at the first configuration that fails and names it
     import tiny_configs as TC
-    for seed in range(10, 60):
+    for seed in range(10, 50):
         name = f"S{seed}"
         TC.CONFIGS[name], TC.PAGE_SIZE[name] = TC.drawn(seed)
         for dtype in ("bfloat16", "float32"):
@@ -355,7 +355,7 @@ def test_fifty_more_drawn_configurations_in_every_way_of_cutting():
                 got, _ = replay(name, dtype, trace)
                 compare(name, dtype, reqs, got, f"sweep {label}")
         for key in [k for k in _plain_cache if k == name or (isinstance(k, tuple) and k[0] == name)]:
-            del _plain_cache[key]           # the weights of fifty models need not stay in memory
+            del _plain_cache[key]           # the weights of forty models need not stay in memory
 
 
 def test_float32_does_not_depend_on_the_cut_at_all():
