@@ -560,16 +560,46 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
                                           int reach = NO_WINDOW) {
   const int kq = (threadIdx.x & 63) >> 4;
   f32x4p s[NQB][2 * NPAIR];
+  // Two query blocks a wave: the operands of a 16-key block (PF_KS reads from LDS) are requested one block ahead of
+  // their products, so that a read's latency passes under the products of the block before; left to itself the
+  // compiler, short of registers, requests each operand just in front of its use (one query block a wave: it has
+  // the registers, and three waves a SIMD to hide the latency with).
+  constexpr bool AHEAD = NQB == 2;
+  if constexpr (AHEAD) {
+    u32x4 ka[2][PF_KS];
 #pragma unroll
-  for (int j = 0; j < 2 * NPAIR; j++) {
+    for (int step = 0; step < PF_KS; step++) ka[0][step] = *reinterpret_cast<const u32x4*>(krow + 32 * step);
 #pragma unroll
-    for (int b = 0; b < NQB; b++) s[b][j] = f32x4p{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 2 * NPAIR; j++) {
+      if (j + 1 < 2 * NPAIR) {
 #pragma unroll
-    for (int step = 0; step < PF_KS; step++) {
-      const bf16x8 a = __builtin_bit_cast(
-          bf16x8, *reinterpret_cast<const u32x4*>(krow + (32 * (j / 2) + 4 * (j % 2)) * KROW + 32 * step));
+        for (int step = 0; step < PF_KS; step++)
+          ka[(j + 1) & 1][step] =
+              *reinterpret_cast<const u32x4*>(krow + (32 * ((j + 1) / 2) + 4 * ((j + 1) % 2)) * KROW + 32 * step);
+      }
+      __builtin_amdgcn_sched_barrier(0);            // the next block's reads stay in front of this block's products
 #pragma unroll
-      for (int b = 0; b < NQB; b++) s[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[b][step], s[b][j], 0, 0, 0);
+      for (int b = 0; b < NQB; b++) s[b][j] = f32x4p{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int step = 0; step < PF_KS; step++) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, ka[j & 1][step]);
+#pragma unroll
+        for (int b = 0; b < NQB; b++) s[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[b][step], s[b][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 2 * NPAIR; j++) {
+#pragma unroll
+      for (int b = 0; b < NQB; b++) s[b][j] = f32x4p{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int step = 0; step < PF_KS; step++) {
+        const bf16x8 a = __builtin_bit_cast(
+            bf16x8, *reinterpret_cast<const u32x4*>(krow + (32 * (j / 2) + 4 * (j % 2)) * KROW + 32 * step));
+#pragma unroll
+        for (int b = 0; b < NQB; b++) s[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q[b][step], s[b][j], 0, 0, 0);
+      }
     }
   }
 #pragma unroll
@@ -609,20 +639,47 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
       }
     st[b].l += sum;
   }
+  bf16x8 pb[NPAIR][NQB];
 #pragma unroll
-  for (int m = 0; m < NPAIR; m++) {
-    bf16x8 pb[NQB];
+  for (int m = 0; m < NPAIR; m++)
 #pragma unroll
     for (int b = 0; b < NQB; b++)
-      pb[b] = __builtin_bit_cast(
+      pb[m][b] = __builtin_bit_cast(
           bf16x8, u32x4{pack2_bf16(s[b][2 * m][0], s[b][2 * m][1]), pack2_bf16(s[b][2 * m][2], s[b][2 * m][3]),
                         pack2_bf16(s[b][2 * m + 1][0], s[b][2 * m + 1][1]), pack2_bf16(s[b][2 * m + 1][2], s[b][2 * m + 1][3])});
+  if constexpr (AHEAD) {
+    // likewise the operands of V^T, in groups of four head-dimension tiles (of two where four do not divide them)
+    constexpr int GR = PF_DT % 4 == 0 ? 4 : 2, NG = NPAIR * PF_DT / GR;
+    static_assert(PF_DT % GR == 0, "whole groups of tiles");
+    u32x4 va[2][GR];
+    auto vsrc = [&](int g, int i) { return vrow + 16 * ((g * GR + i) % PF_DT) * PF_VROW + 32 * ((g * GR + i) / PF_DT); };
 #pragma unroll
-    for (int tt = 0; tt < PF_DT; tt++) {
-      const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(vrow + 16 * tt * PF_VROW + 32 * m));
+    for (int i = 0; i < GR; i++) va[0][i] = *reinterpret_cast<const u32x4*>(vsrc(0, i));
 #pragma unroll
-      for (int b = 0; b < NQB; b++) st[b].o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[b], st[b].o[tt], 0, 0, 0);
+    for (int g = 0; g < NG; g++) {
+      if (g + 1 < NG) {
+#pragma unroll
+        for (int i = 0; i < GR; i++) va[(g + 1) & 1][i] = *reinterpret_cast<const u32x4*>(vsrc(g + 1, i));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < GR; i++) {
+        const int tt = (g * GR + i) % PF_DT, m = (g * GR + i) / PF_DT;
+        const bf16x8 a = __builtin_bit_cast(bf16x8, va[g & 1][i]);
+#pragma unroll
+        for (int b = 0; b < NQB; b++) st[b].o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[m][b], st[b].o[tt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
+  } else {
+#pragma unroll
+    for (int m = 0; m < NPAIR; m++)
+#pragma unroll
+      for (int tt = 0; tt < PF_DT; tt++) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(vrow + 16 * tt * PF_VROW + 32 * m));
+#pragma unroll
+        for (int b = 0; b < NQB; b++) st[b].o[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[m][b], st[b].o[tt], 0, 0, 0);
+      }
   }
 }
 
