@@ -686,7 +686,7 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
 // grid: x = query head, y = (sequence, 64-query tile), late (long) tiles first.  One team keeps three
 // workgroups on a compute unit, which serves many long, equal tiles best; two or three teams cut the key
 // loop of the longest tile, which decides when the tiles are few or unequal (a causal triangle).
-// NQB = 2 (one team only): a wave owns two blocks of 16 queries and a workgroup 128, so every K and V^T
+// NQB = 2 (one or two teams): a wave owns two blocks of 16 queries and a workgroup 128, so every K and V^T
 // operand read from LDS feeds two products; LDS traffic, which bounds the kernel when there is work for
 // every compute unit, halves per product, at the price of registers for two waves per SIMD.
 template <int KT, int NQB = 1>
@@ -695,10 +695,14 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
     float scale, int reach, int chunk_len, int max_chunks, float* __restrict__ part) {
-  static_assert(NQB == 1 || KT == 1, "two query blocks a wave: one team");
+  static_assert(NQB == 1 || KT <= 2, "two query blocks a wave: one or two teams (three would leave a wave 170 registers)");
   constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
   constexpr int BMQ = PF_BM * NQB;            // queries per workgroup
-  __shared__ PfTiles<KT> tiles;
+  // the tiles of keys and values, and after the key loop the sums that the teams beyond the first hand to it
+  constexpr size_t MERGE_BYTES = (size_t)(KT - 1) * 4 * NQB * (PF_DT * 4 + 2) * 64 * sizeof(float);
+  constexpr size_t LDS_BYTES = sizeof(PfTiles<KT>) > MERGE_BYTES ? sizeof(PfTiles<KT>) : MERGE_BYTES;
+  __shared__ alignas(16) char lds[LDS_BYTES];
+  PfTiles<KT>& tiles = *reinterpret_cast<PfTiles<KT>*>(lds);
   int b = 0, tile = (int)blockIdx.y, ntiles = 0;
   for (; b < num_seqs; b++) {
     ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + BMQ - 1) / BMQ;
@@ -808,41 +812,47 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   }
   if constexpr (KT > 1) {
     // merge the teams through LDS (reusing the tile memory): lane-wise, the layouts agree
-    PfState& s0 = st[0];
     __syncthreads();
-    float* xo = reinterpret_cast<float*>(&tiles);              // [team - 1][wave][PF_DT * 4 + 2][64 lanes]
-    constexpr int PER_WAVE = (PF_DT * 4 + 2) * 64;
-    static_assert(sizeof(PfTiles<KT>) >= (size_t)(KT - 1) * 4 * PER_WAVE * sizeof(float) || KT == 1,
-                  "LDS tile memory too small for the merge");
+    float* xo = reinterpret_cast<float*>(lds);                 // [team - 1][wave][query block][PF_DT * 4 + 2][64 lanes]
+    constexpr int PER_BLOCK = (PF_DT * 4 + 2) * 64, PER_WAVE = NQB * PER_BLOCK;
+    static_assert(LDS_BYTES >= (size_t)(KT - 1) * 4 * PER_WAVE * sizeof(float), "LDS too small for the merge");
     if (team > 0) {
-      float* mine = xo + ((team - 1) * 4 + wave) * PER_WAVE + lane;
 #pragma unroll
-      for (int tt = 0; tt < PF_DT; tt++)
+      for (int qb = 0; qb < NQB; qb++) {
+        float* mine = xo + ((team - 1) * 4 + wave) * PER_WAVE + qb * PER_BLOCK + lane;
 #pragma unroll
-        for (int r = 0; r < 4; r++) mine[(4 * tt + r) * 64] = s0.o[tt][r];
-      mine[(PF_DT * 4) * 64] = s0.m;
-      mine[(PF_DT * 4 + 1) * 64] = s0.l;
+        for (int tt = 0; tt < PF_DT; tt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) mine[(4 * tt + r) * 64] = st[qb].o[tt][r];
+        mine[(PF_DT * 4) * 64] = st[qb].m;
+        mine[(PF_DT * 4 + 1) * 64] = st[qb].l;
+      }
     }
     __syncthreads();
     if (team > 0) return;
-    float M = s0.m;
 #pragma unroll
-    for (int t = 1; t < KT; t++) M = fmaxf(M, xo[((t - 1) * 4 + wave) * PER_WAVE + (PF_DT * 4) * 64 + lane]);
-    const float m_use = (M == -INFINITY) ? 0.f : M;
-    const float a0 = __builtin_amdgcn_exp2f((s0.m - m_use) * c);
-    s0.l *= a0;
-    s0.m = M;                                                  // what the merged sums are relative to (a chunk's part says so)
+    for (int qb = 0; qb < NQB; qb++) {
+      PfState& s0 = st[qb];
+      const float* base = xo + wave * PER_WAVE + qb * PER_BLOCK + lane;       // team t: base + (t - 1) * 4 * PER_WAVE
+      float M = s0.m;
 #pragma unroll
-    for (int tt = 0; tt < PF_DT; tt++) s0.o[tt] *= a0;
+      for (int t = 1; t < KT; t++) M = fmaxf(M, base[(t - 1) * 4 * PER_WAVE + (PF_DT * 4) * 64]);
+      const float m_use = (M == -INFINITY) ? 0.f : M;
+      const float a0 = __builtin_amdgcn_exp2f((s0.m - m_use) * c);
+      s0.l *= a0;
+      s0.m = M;                                                // what the merged sums are relative to (a chunk's part says so)
 #pragma unroll
-    for (int t = 1; t < KT; t++) {
-      const float* theirs = xo + ((t - 1) * 4 + wave) * PER_WAVE + lane;
-      const float at = __builtin_amdgcn_exp2f((theirs[(PF_DT * 4) * 64] - m_use) * c);
-      s0.l += at * theirs[(PF_DT * 4 + 1) * 64];
+      for (int tt = 0; tt < PF_DT; tt++) s0.o[tt] *= a0;
 #pragma unroll
-      for (int tt = 0; tt < PF_DT; tt++)
+      for (int t = 1; t < KT; t++) {
+        const float* theirs = base + (t - 1) * 4 * PER_WAVE;
+        const float at = __builtin_amdgcn_exp2f((theirs[(PF_DT * 4) * 64] - m_use) * c);
+        s0.l += at * theirs[(PF_DT * 4 + 1) * 64];
 #pragma unroll
-        for (int r = 0; r < 4; r++) s0.o[tt][r] += at * theirs[(4 * tt + r) * 64];
+        for (int tt = 0; tt < PF_DT; tt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) s0.o[tt][r] += at * theirs[(4 * tt + r) * 64];
+      }
     }
   }
   if (n_chunks > 1) {
@@ -1262,8 +1272,8 @@ static int check_common(const char* who, int nq, int nkv, int d, int P, int max_
 extern "C" int pico_attn_head_dim() { return D; }
 
 // teams: the shape of the workgroups (1 to 3 teams of four waves that share the key loop of a 64-query tile; 4: one
-// team of 128 queries; 0: two teams where the head size allows it); a hint, any value gives the same result up to
-// rounding.  chunk_len > 0 (a multiple of 128, no window, not three teams, head sizes in steps of 32): the keys of every tile are cut
+// team of 128 queries; 6: two teams of 128 queries; 0: two teams of 64 where the head size allows it); a hint, any
+// value gives the same result up to rounding.  chunk_len > 0 (a multiple of 128, no window, not three teams, head sizes in steps of 32): the keys of every tile are cut
 // into chunks of that many, each a workgroup of its own, and a second launch joins the chunks of a tile; part is
 // their workspace, float32 [num_tokens, nq, max_chunks, D + 4], and max_chunks at least ceil(longest context / chunk_len).
 extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
@@ -1295,7 +1305,11 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
     int bmq = PF_BM;
 #define PF_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, \
                 cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach, chunk_len, max_chunks, part
-    if (teams == 4 && PF_KT_MAX == 2) {      // 128 queries a workgroup, two blocks of 16 a wave
+    if (teams == 6 && PF_KT_MAX == 2) {      // 128 queries a workgroup and two key teams
+      grid.y = num_tokens / (2 * PF_BM) + num_seqs;
+      bmq = 2 * PF_BM;
+      prefill16_kernel<PF_KT_MAX == 2 ? 2 : 1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 512, 0, stream>>>(PF_ARGS);
+    } else if (teams == 4 && PF_KT_MAX == 2) {      // 128 queries a workgroup, two blocks of 16 a wave
       grid.y = num_tokens / (2 * PF_BM) + num_seqs;
       bmq = 2 * PF_BM;
       prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 256, 0, stream>>>(PF_ARGS);

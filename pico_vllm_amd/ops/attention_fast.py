@@ -60,7 +60,11 @@ class FastAttention:
         4: one team whose waves own two blocks of 16 queries, 128 queries a workgroup: half the LDS traffic
         per product, which is the bound when every compute unit has plenty to do (184 us for the eight
         prompts, 622 against 825 us for four portions of 2,048 tokens after 2,048 with 40 heads), but coarser
-        tiles, so only for much work in portions that fill them."""
+        tiles, so only for much work in portions that fill them.
+        6: such waves in two teams (eight waves a workgroup): between the two, when there is more than the longest
+        tile's worth of work for every unit but not 64 tiles' worth (two prompts of 2,048 tokens of 12 heads: 56 us
+        against 71 with 4 and 74 with 1; one prompt of 28 heads: 63 against 71 and 72; four portions of 512 after
+        512: 32 against 36 and 39)."""
         longest, total, tokens, padded = 1, 0, 0, 0
         window = getattr(self, "window", 0)
         for n, c in zip(new_lens, context_lens):
@@ -75,7 +79,9 @@ class FastAttention:
         cus = getattr(self, "cus", None) or compute_units()
         if total * self.nq < cus * longest:
             return 3
-        return 4 if total * self.nq >= cus * 64 and 4 * tokens >= 3 * padded else 1
+        if 4 * tokens < 3 * padded:
+            return 1
+        return 4 if total * self.nq >= cus * 64 else 6
 
     def prefill_chunks(self, new_lens, context_lens):
         """(shape, chunk_len, max_chunks) when the keys of the query tiles are better cut into chunks that run as

@@ -389,7 +389,7 @@ def test_fast_attention_with_a_window(K, nq, nkv, d, Pg, window):
         for q in qs:
             q *= 2.0
     new_lens, prefix_lens = [70, 1, 200, 2, 1, 130], [0, 300, 131, 63, 17, 500]
-    for teams in (1, 2, 3, 4):
+    for teams in (1, 2, 3, 4, 6):
         out, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=window, boost=boost, teams=teams, window=window)
         close(out, want, torch.bfloat16)
     for nsplit in (1, 3, 8):
@@ -438,11 +438,11 @@ def test_fast_prefill_other_sizes_and_long_portions(K, nq, nkv, d, Pg):
     close(out, want, torch.bfloat16)
 
 
-@pytest.mark.parametrize("teams", [1, 2, 3, 4])
+@pytest.mark.parametrize("teams", [1, 2, 3, 4, 6])
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(6, 3, 32, 8), (2, 2, 64, 8), (12, 2, 128, 16), (8, 2, 256, 64), (4, 1, 96, 32),
                                         (4, 1, 96, 16), (4, 1, 96, 8), (8, 2, 256, 16), (2, 1, 160, 8)])
 def test_fast_prefill_with_every_shape_of_workgroup(K, nq, nkv, d, Pg, teams):
-    # the shape of the workgroups (1 to 3 teams on a 64-query tile, 4: two query blocks a wave, 128-query tiles)
+    # the shape of the workgroups (1 to 3 teams on a 64-query tile, 4: two query blocks a wave, 128-query tiles, 6: two teams of those)
     # is a hint: every value gives the same attention; lengths around the 64- and 128-query tiles and the
     # 64-, 128- and 192-key tiles of one to three teams; pages of 8 and 16 keys take the short way in whole tiles
     out, want = _fast_case([63, 1, 65, 130, 2, 200, 193, 127, 257], [0, 127, 1, 62, 191, 129, 383, 1, 64], nq, nkv, d, Pg, seed=5,
@@ -488,7 +488,7 @@ def test_fast_attention_of_a_step_with_much_work(K):
     close(out, want, torch.bfloat16)
 
 
-@pytest.mark.parametrize("teams", [0, 1, 2, 4])
+@pytest.mark.parametrize("teams", [0, 1, 2, 4, 6])
 @pytest.mark.parametrize("nq,nkv,d,Pg,chunk_len", [(12, 2, 128, 16, 256), (6, 3, 32, 8, 128), (2, 2, 64, 8, 384), (4, 1, 96, 32, 128),
                                                   (4, 2, 256, 16, 512), (2, 1, 160, 8, 256)])
 def test_fast_prefill_with_the_keys_cut_into_chunks(K, nq, nkv, d, Pg, chunk_len, teams):
@@ -546,6 +546,9 @@ def test_fast_prefill_chooses_teams_by_the_shape_of_the_batch():
     assert fa.prefill_teams([1] * 8, [4000] * 8) == 3       # decode tokens inside a mixed step
     assert fa.prefill_teams([2048], [16384]) == 4           # many long, equal tiles that fill 128 queries
     assert fa.prefill_teams([32] * 64, [2032] * 64) == 1    # much work in short portions
+    assert fa.prefill_teams([2048] * 2, [2048] * 2) == 6    # more than the longest tile's worth for every unit, not much more
+    assert fa.prefill_teams([512] * 4, [1024] * 4) == 6
+    assert fa.prefill_teams([2048] * 4, [2048] * 4) == 4    # much work
 
 
 def test_fast_prefill_with_a_cache_of_4_gib(K):
