@@ -67,6 +67,7 @@ class LLMEngine:
             self.eos_token_id = getattr(tokenizer, "eos_token_id", None)
         self.tokenizer = tokenizer
         self._next_id = 0
+        self.no_more_requests = False
         self.requests: Dict[int, Request] = {}
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
         self.timers = PhaseTimers(args.profile_phases)
@@ -76,7 +77,9 @@ class LLMEngine:
     def submit(self, prompt: Union[str, Sequence[int]], max_new_tokens: int = 16, temperature: float = 0.0,
                top_p: float = 1.0, seed: Optional[int] = None, ignore_eos: bool = False,
                stop_token_ids: Sequence[int] = ()) -> int:
-        """Queue a request; returns its id (pico_vllm/engine.py:243-276)."""
+        """Queue a request; returns its id, or -1 once ``mark_finished`` has been called (pico_vllm/engine.py:243-276)."""
+        if self.no_more_requests:
+            return -1
         params = SamplingParams(max_new_tokens, temperature, top_p, seed, ignore_eos, [int(t) for t in stop_token_ids])
         params.validate()
         ids = self._encode(prompt)
@@ -130,7 +133,14 @@ class LLMEngine:
             done += self._resolve(launched)
         return done
 
+    def mark_finished(self) -> None:
+        """No further request will be submitted (pico_vllm/engine.py:278-280): ``submit`` returns -1 from now on."""
+        self.no_more_requests = True
+
     def is_done(self) -> bool:
+        """Nothing is queued, running or in flight.  (The reference's also waits for ``mark_finished``,
+        engine.py:472-475; here a loop over ``step`` may end whenever the engine has run dry, and more may be
+        submitted afterwards.)"""
         return self._inflight is None and not self.scheduler.has_unfinished()
 
     # ---- a step in two halves -------------------------------------------

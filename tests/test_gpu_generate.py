@@ -149,6 +149,13 @@ def test_submit_step_is_done_in_the_reference_manner():
         eng.submit([1] * 200, max_new_tokens=10)
     with pytest.raises(ValueError):
         eng.submit([999], max_new_tokens=1)
+    # after mark_finished nothing more is taken (the reference returns -1 then, engine.py:250-251)
+    c = eng.submit([7, 8], max_new_tokens=2, ignore_eos=True)
+    eng.mark_finished()
+    assert eng.submit([1, 2, 3], max_new_tokens=1) == -1 and not eng.is_done()
+    while not eng.is_done():
+        done += eng.step()
+    assert done[-1].request_id == c and len(done[-1].token_ids) == 2
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
