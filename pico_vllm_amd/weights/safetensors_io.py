@@ -36,10 +36,18 @@ class SafetensorsFile:
 
     def __init__(self, path: str):
         self.path = path
+        self._mm = None
+        self._f = open(path, "rb")
+        try:
+            self._read_header(path)
+        except BaseException:
+            self.close()
+            raise
+
+    def _read_header(self, path: str) -> None:
         size = os.path.getsize(path)
         if size < 8:
             raise SafetensorsError(f"{path}: file is truncated (no header length)")
-        self._f = open(path, "rb")
         (n,) = struct.unpack("<Q", self._f.read(8))
         if 8 + n > size:
             raise SafetensorsError(f"{path}: file is truncated (header of {n} bytes does not fit in {size})")
@@ -47,19 +55,24 @@ class SafetensorsFile:
             header = json.loads(self._f.read(n).decode("utf-8"))
         except (UnicodeDecodeError, json.JSONDecodeError) as e:
             raise SafetensorsError(f"{path}: header is not valid JSON: {e}") from None
+        if not isinstance(header, dict):
+            raise SafetensorsError(f"{path}: header is not a JSON object")
         self.metadata = header.pop("__metadata__", {})
         self._base = 8 + n
-        self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ) if size else None
+        self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ)
         self.entries: Dict[str, Tuple[str, Tuple[int, ...]]] = {}
         self._offsets: Dict[str, Tuple[int, int]] = {}
         for name, info in header.items():
-            dt, shape = info["dtype"], tuple(int(s) for s in info["shape"])
-            b, e = info["data_offsets"]
+            try:
+                dt, shape = info["dtype"], tuple(int(s) for s in info["shape"])
+                b, e = (int(x) for x in info["data_offsets"])
+            except (KeyError, TypeError, ValueError):
+                raise SafetensorsError(f"{path}: tensor {name!r}: entry needs dtype, shape and data_offsets") from None
             if dt not in _DTYPES:
                 raise SafetensorsError(f"{path}: tensor {name!r} has unsupported dtype {dt}")
             want = int(np.prod(shape, dtype=np.int64)) * _DTYPES[dt][1]
-            if e - b != want:
-                raise SafetensorsError(f"{path}: tensor {name!r}: {e - b} bytes stored, shape {shape} needs {want}")
+            if b < 0 or min(shape, default=0) < 0 or e - b != want:
+                raise SafetensorsError(f"{path}: tensor {name!r}: bytes {b}..{e} stored, shape {shape} needs {want}")
             if self._base + e > size:
                 raise SafetensorsError(f"{path}: file is truncated inside tensor {name!r}")
             self.entries[name] = (dt, shape)

@@ -103,7 +103,8 @@ def test_random_model_is_seeded_and_typed():
         assert q1.dtype == torch.bfloat16 and not torch.equal(q1, q2)
         n = f1.tensor("model.norm.weight")
         assert n.dtype == torch.float32 and float(n.min()) >= 0.9 and float(n.max()) <= 1.1
-    assert json.load(open(os.path.join(a1, "config.json")))["vocab_size"] == 256
+    with open(os.path.join(a1, "config.json")) as f:
+        assert json.load(f)["vocab_size"] == 256
     assert a1 == a2
 
 
@@ -188,10 +189,37 @@ def test_truncated_and_empty_folders(tmp_path):
     with pytest.raises(WeightsError, match="no .safetensors"):
         load_checkpoint(str(tmp_path), _specs("A"), torch.bfloat16)
     src = os.path.join(model_dir("A"), "model.safetensors")
-    data = open(src, "rb").read()
+    with open(src, "rb") as f:
+        data = f.read()
     (tmp_path / "model.safetensors").write_bytes(data[:len(data) // 2])
     with pytest.raises(WeightsError, match="truncated"):
         load_checkpoint(str(tmp_path), _specs("A"), torch.bfloat16)
+
+
+def test_a_malformed_header_is_one_clear_error_and_leaves_no_file_open(tmp_path):
+    import struct
+    import warnings
+
+    def stored(header: bytes, body: bytes = b""):
+        (tmp_path / "model.safetensors").write_bytes(struct.pack("<Q", len(header)) + header + body)
+
+    cases = {
+        b"[1, 2]": "not a JSON object",
+        b"{not json": "not valid JSON",
+        b'{"w": {"dtype": "BF16", "shape": [2, 2]}}': "needs dtype, shape and data_offsets",
+        b'{"w": {"dtype": "BF16", "shape": [2, 2], "data_offsets": [-8, 0]}}': "shape .* needs 8",
+        b'{"w": {"dtype": "BF16", "shape": [2, 2], "data_offsets": [0, 6]}}': "shape .* needs 8",
+        b'{"w": {"dtype": "F8_E4M3", "shape": [2, 2], "data_offsets": [0, 4]}}': "unsupported dtype",
+        b'{"w": {"dtype": "BF16", "shape": [2, 2], "data_offsets": [0, 8]}}': "truncated inside",
+    }
+    with warnings.catch_warnings():
+        warnings.simplefilter("error", ResourceWarning)
+        for header, message in cases.items():
+            stored(header, b"\0" * 4)
+            with pytest.raises(WeightsError, match=message):
+                load_checkpoint(str(tmp_path), _specs("A"), torch.bfloat16)
+        import gc
+        gc.collect()
 
 
 def test_named_configurations_parse_and_the_tiny_ones_differ_in_every_size():
