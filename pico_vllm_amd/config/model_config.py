@@ -22,6 +22,20 @@ _REQUIRED = ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_he
              "tie_word_embeddings")
 
 
+def _integer(d: Dict[str, Any], key: str, value: Any = None) -> int:
+    v = d[key] if value is None else value
+    if isinstance(v, bool) or not isinstance(v, int):
+        raise ConfigError(f"{key} must be an integer, got {v!r}")
+    return v
+
+
+def _number(d: Dict[str, Any], key: str) -> float:
+    v = d[key]
+    if isinstance(v, bool) or not isinstance(v, (int, float)):
+        raise ConfigError(f"{key} must be a number, got {v!r}")
+    return float(v)
+
+
 @dataclass(frozen=True)
 class Qwen2Config:
     vocab_size: int
@@ -54,25 +68,33 @@ class Qwen2Config:
         head_dim = d.get("head_dim")
         if head_dim is None:
             # pico_vllm/model.py:37-38
-            if d["hidden_size"] % d["num_attention_heads"]:
+            width, heads = _integer(d, "hidden_size"), _integer(d, "num_attention_heads")
+            if heads < 1 or width % heads:
                 raise ConfigError("hidden_size is not a multiple of num_attention_heads and head_dim is not given")
-            head_dim = d["hidden_size"] // d["num_attention_heads"]
+            head_dim = width // heads
         eos = d.get("eos_token_id")
         if isinstance(eos, (list, tuple)):
             eos = eos[0] if eos else None
+        if eos is not None:
+            eos = _integer(d, "eos_token_id", eos)
+        if not isinstance(d["tie_word_embeddings"], bool):
+            raise ConfigError(f"tie_word_embeddings must be true or false, got {d['tie_word_embeddings']!r}")
+        architectures = d.get("architectures") or ("Qwen2ForCausalLM",)
+        if isinstance(architectures, str) or not all(isinstance(a, str) for a in architectures):
+            raise ConfigError(f"architectures must be a list of names, got {architectures!r}")
         known = set(cls.__dataclass_fields__) | {"use_sliding_window", "sliding_window", "max_window_layers",
                                                  "rope_scaling", "attention_bias", "model_type"}
         cfg = cls(
-            vocab_size=int(d["vocab_size"]), hidden_size=int(d["hidden_size"]),
-            num_hidden_layers=int(d["num_hidden_layers"]),
-            num_attention_heads=int(d["num_attention_heads"]),
-            num_key_value_heads=int(d["num_key_value_heads"]),
-            intermediate_size=int(d["intermediate_size"]),
-            rms_norm_eps=float(d["rms_norm_eps"]), rope_theta=float(d["rope_theta"]),
-            tie_word_embeddings=bool(d["tie_word_embeddings"]), head_dim=int(head_dim),
-            max_position_embeddings=int(d.get("max_position_embeddings", 131072)),
+            vocab_size=_integer(d, "vocab_size"), hidden_size=_integer(d, "hidden_size"),
+            num_hidden_layers=_integer(d, "num_hidden_layers"),
+            num_attention_heads=_integer(d, "num_attention_heads"),
+            num_key_value_heads=_integer(d, "num_key_value_heads"),
+            intermediate_size=_integer(d, "intermediate_size"),
+            rms_norm_eps=_number(d, "rms_norm_eps"), rope_theta=_number(d, "rope_theta"),
+            tie_word_embeddings=d["tie_word_embeddings"], head_dim=_integer(d, "head_dim", head_dim),
+            max_position_embeddings=_integer(d, "max_position_embeddings", d.get("max_position_embeddings", 131072)),
             hidden_act=str(d.get("hidden_act", "silu")), eos_token_id=eos,
-            architectures=tuple(d.get("architectures", ("Qwen2ForCausalLM",))),
+            architectures=tuple(architectures),
             torch_dtype=str(d.get("torch_dtype", "bfloat16")),
             ignored_keys=tuple(sorted(k for k in d if k not in known)),
         )
@@ -81,7 +103,7 @@ class Qwen2Config:
 
     def _validate(self, raw: Dict[str, Any]) -> None:
         pos = ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
-               "num_key_value_heads", "intermediate_size", "head_dim")
+               "num_key_value_heads", "intermediate_size", "head_dim", "max_position_embeddings")
         for k in pos:
             least = 0 if k == "num_hidden_layers" else 1
             if getattr(self, k) < least:

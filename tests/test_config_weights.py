@@ -36,7 +36,11 @@ def test_config_reads_every_key_and_has_no_size_defaults():
     ({"num_key_value_heads": 3}, "multiple"), ({"hidden_act": "gelu"}, "hidden_act"),
     ({"use_sliding_window": True}, "sliding"), ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"),
     ({"hidden_size": 66}, "head_dim"), ({"head_dim": 15}, "even"), ({"attention_bias": False}, "bias"),
-    ({"vocab_size": 0}, "vocab_size"),
+    ({"vocab_size": 0}, "vocab_size"), ({"hidden_size": "64"}, "hidden_size must be an integer"),
+    ({"vocab_size": 255.5}, "vocab_size must be an integer"), ({"num_hidden_layers": True}, "must be an integer"),
+    ({"rms_norm_eps": "1e-6"}, "rms_norm_eps must be a number"), ({"tie_word_embeddings": "yes"}, "true or false"),
+    ({"max_position_embeddings": 0}, "max_position_embeddings"), ({"eos_token_id": "3"}, "eos_token_id"),
+    ({"architectures": "Qwen2ForCausalLM"}, "list of names"),
 ])
 def test_config_rejects_what_the_engine_cannot_run(patch, word):
     with pytest.raises(ConfigError, match=word):
