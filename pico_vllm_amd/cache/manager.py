@@ -170,12 +170,11 @@ class CacheManager:
         if num_tokens > s.num_computed:
             raise ValueError("the source has not computed that many tokens")
         n = num_tokens // self.page_size
+        if any(p < 0 for st in s.tables for p in st[:n]):                # before anything is changed
+            raise PagePoolError("a page of the prefix was already given back by its window")
         for g, st, dt in zip(self.groups, s.tables, d.tables):
-            pages = st[:n]
-            if any(p < 0 for p in pages):
-                raise PagePoolError("a page of the prefix was already given back by its window")
-            g.pool.share(pages)
-            dt.extend(pages)
+            g.pool.share(st[:n])
+            dt.extend(st[:n])
         for gi in range(len(self.groups)):
             _mirror(d, gi)
         d.num_computed = num_tokens

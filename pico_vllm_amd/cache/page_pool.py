@@ -87,11 +87,11 @@ class PagePool:
                 self._free.append(p)
 
     def check(self) -> None:
-        free = list(self._free)
-        if len(set(free)) != len(free):
+        free = set(self._free)
+        if len(free) != len(self._free):
             raise PagePoolError("a page is on the free list twice")
         for p in range(self.num_pages):
-            if (self._refs[p] == 0) != (p in set(free)):
+            if (self._refs[p] == 0) != (p in free):
                 raise PagePoolError(f"page {p}: count {self._refs[p]} disagrees with the free list")
 
 

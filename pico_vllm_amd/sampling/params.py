@@ -9,7 +9,12 @@ request like the end-of-sequence token; the token is kept) have no counterpart t
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from numbers import Integral
 from typing import List, Optional
+
+
+def _whole(x) -> bool:
+    return isinstance(x, Integral) and not isinstance(x, bool)
 
 
 @dataclass
@@ -22,9 +27,11 @@ class SamplingParams:
     stop_token_ids: List[int] = field(default_factory=list)
 
     def validate(self) -> None:
-        if self.max_new_tokens < 1:
-            raise ValueError("max_new_tokens must be at least 1")
-        if self.temperature < 0:
-            raise ValueError("temperature must not be negative")
-        if not (0 < self.top_p):
-            raise ValueError("top_p must be positive")
+        if not _whole(self.max_new_tokens) or self.max_new_tokens < 1:
+            raise ValueError(f"max_new_tokens must be an integer of at least 1, got {self.max_new_tokens!r}")
+        if not (0 <= self.temperature < float("inf")):               # refuses not-a-number too
+            raise ValueError(f"temperature must be a number that is not negative, got {self.temperature!r}")
+        if not (0 < self.top_p < float("inf")):
+            raise ValueError(f"top_p must be a positive number, got {self.top_p!r}")
+        if not all(_whole(t) for t in self.stop_token_ids):
+            raise ValueError(f"stop_token_ids must be token ids, got {self.stop_token_ids!r}")

@@ -196,3 +196,77 @@ def test_a_model_with_state_cannot_share_a_prefix():
     with pytest.raises(PagePoolError, match="state"):
         m.fork_prefix("a", "b", 16)
     m.check()
+
+
+def test_the_checks_find_every_kind_of_damage():
+    # the tests above trust PagePool.check and CacheManager.check: each kind of damage, done by hand, is found
+    def damaged():
+        m = CacheManager({0: FULL, 1: WIN}, 8, 12, 3)
+        for r, n in (("a", 30), ("b", 9)):
+            m.add_request(r); m.grow(r, n); m.advance(r, n)
+        m.check()
+        return m
+
+    m = damaged()
+    m.groups[0].pool._free.append(m.groups[0].pool._free[0])             # a page twice on the free list
+    with pytest.raises(PagePoolError, match="free list twice"):
+        m.check()
+    m = damaged()
+    m.groups[0].pool._free.append(m.block_table("a")[0])                 # a held page that is also free
+    with pytest.raises(PagePoolError, match="disagrees with the free list"):
+        m.check()
+    m = damaged()
+    m.groups[0].pool._free.popleft()                                     # a page lost: neither free nor held
+    with pytest.raises(PagePoolError, match="disagrees with the free list"):
+        m.check()
+    m = damaged()
+    m.block_table("a")[1] = m.block_table("a")[0]                        # one page twice in a table
+    with pytest.raises(PagePoolError, match="twice in one table"):
+        m.check()
+    m = damaged()
+    m.block_table("b")[0] = m.block_table("a")[0]                        # held by two tables, counted once
+    with pytest.raises(PagePoolError, match="held by 2 tables"):
+        m.check()
+    m = damaged()
+    m.groups[0].pool.share(m.block_table("a")[:1])                       # counted twice, held by one table
+    with pytest.raises(PagePoolError, match="count 2, held by 1"):
+        m.check()
+    m.check(other_holders=[{m.block_table("a")[0]: 1}, {}])              # unless another holder is named
+    m = damaged()
+    m.requests["b"].slot = m.requests["a"].slot                          # a slot held twice
+    with pytest.raises(PagePoolError, match="slot is held twice"):
+        m.check()
+    m = damaged()
+    m.free_request("b")
+    m.slots._free.pop()                                                  # a slot lost
+    with pytest.raises(PagePoolError, match="slot was lost"):
+        m.check()
+
+
+def test_what_the_manager_refuses():
+    m = CacheManager({0: FULL, 1: WIN}, 8, 12, 3)
+    with pytest.raises(ValueError, match="unknown cache kind"):
+        CacheManager({0: CacheSpec("ring")}, 8, 12, 3)
+    with pytest.raises(ValueError, match="at least one page"):
+        PagePool(0)
+    with pytest.raises(ValueError, match="negative"):
+        PagePool(2).allocate(-1)
+    assert m.add_request("a")
+    with pytest.raises(PagePoolError, match="already in the cache"):
+        m.add_request("a")
+    m.grow("a", 64); m.advance("a", 64)
+    assert m.num_free_pages() == min(12 - 8, 12 - 3)                      # of the group that has fewest
+    assert list(m.block_table_array("a", 0, 3)) == m.block_table("a")[:3]
+    with pytest.raises(PagePoolError, match="9 pages are needed, 8 are allocated"):
+        m.block_table_array("a", 0, 9)
+    m.add_request("b")
+    with pytest.raises(ValueError, match="not computed that many"):
+        m.fork_prefix("a", "b", 72)
+    with pytest.raises(PagePoolError, match="given back by its window"):
+        m.fork_prefix("a", "b", 48)                                       # the window's group has dropped pages 0..4
+    assert m.block_table("b", 0) == [] and m.block_table("b", 1) == []    # and nothing was shared before it was refused
+    m.check()
+    m.grow("b", 3); m.advance("b", 3)
+    with pytest.raises(PagePoolError, match="must be empty"):
+        m.fork_prefix("a", "b", 8)
+    m.check()

@@ -47,6 +47,23 @@ def test_config_rejects_what_the_engine_cannot_run(patch, word):
         Qwen2Config.from_dict({**TINY_A, **patch})
 
 
+def test_a_config_file_that_is_missing_or_broken_and_the_way_back_to_a_file(tmp_path):
+    from pico_vllm_amd.config.model_config import read_config_json
+    with pytest.raises(ConfigError, match="does not exist"):
+        read_config_json(str(tmp_path))
+    (tmp_path / "config.json").write_text('{"vocab_size": 256,')
+    with pytest.raises(ConfigError, match="not valid JSON"):
+        read_config_json(str(tmp_path))
+    cfg = Qwen2Config.from_dict({**TINY_A, "eos_token_id": [7, 9], "some_future_key": 1})
+    assert cfg.eos_token_id == 7 and cfg.ignored_keys == ("some_future_key",) and cfg.num_kv_groups == 4
+    assert Qwen2Config.from_dict({**TINY_A, "eos_token_id": []}).eos_token_id is None
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+    assert Qwen2Config.from_dict(read_config_json(str(tmp_path))) == cfg      # what it writes, it reads
+    for key, word in (("rms_norm_eps", "rms_norm_eps"), ("rope_theta", "rope_theta")):
+        with pytest.raises(ConfigError, match=word):
+            Qwen2Config.from_dict({**TINY_A, key: 0.0})
+
+
 def test_registry_resolves_by_name_and_lists_known_names():
     assert "Qwen2ForCausalLM" in known_architectures()
     assert resolve_architecture(TINY_A).name == "Qwen2ForCausalLM"
@@ -187,6 +204,27 @@ def test_tied_model_ignores_a_stored_lm_head_and_untied_needs_it(tmp_path):
     with pytest.raises(WeightsError) as e:
         load_checkpoint(d, _specs("A") + [ParamSpec("lm_head.weight", (256, 64))], torch.bfloat16)
     assert e.value.missing == ["lm_head.weight"]
+
+
+def test_a_tensor_stored_twice_or_as_the_wrong_kind_of_number(tmp_path):
+    from pico_vllm_amd.weights.safetensors_io import write_safetensors
+    specs = [ParamSpec("w", (2, 4)), ParamSpec("table", (3,), role="table")]
+    made = {"w": torch.ones(2, 4, dtype=torch.bfloat16), "table": torch.arange(3, dtype=torch.int64)}
+
+    def store(name, names, tensors=made):
+        write_safetensors(str(tmp_path / name), [(n, tuple(tensors[n].shape), tensors[n].dtype) for n in names], tensors.__getitem__)
+
+    store("model-1.safetensors", ["w", "table"])
+    out = load_checkpoint(str(tmp_path), specs, torch.bfloat16)
+    assert out["w"].dtype == torch.bfloat16 and out["table"].dtype == torch.int32 and out["table"].tolist() == [0, 1, 2]
+    store("model-2.safetensors", ["w"])
+    with pytest.raises(WeightsError, match="tensor w is stored twice"):
+        load_checkpoint(str(tmp_path), specs, torch.bfloat16)
+    (tmp_path / "model-2.safetensors").unlink()
+    store("model-1.safetensors", ["w", "table"], {"w": torch.ones(2, 4, dtype=torch.int32), "table": torch.ones(3)})
+    with pytest.raises(WeightsError) as e:
+        load_checkpoint(str(tmp_path), specs, torch.bfloat16)
+    assert "tensor w is stored as I32" in str(e.value) and "tensor table is stored as F32" in str(e.value)
 
 
 def test_truncated_and_empty_folders(tmp_path):

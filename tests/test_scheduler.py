@@ -190,3 +190,29 @@ def test_a_windowed_group_is_sized_by_its_window_not_by_the_length():
     full, s2 = make(num_pages=8, budget=32, max_seqs=2)
     with pytest.raises(ValueError, match="could never finish"):
         s2.add_request(req(1, 300, 100))
+
+
+def test_no_admission_without_a_state_slot_and_what_the_scheduler_refuses():
+    m = CacheManager(SPEC, 16, 64, 1)                       # one slot for per-request state, though two may run
+    s = Scheduler(m, 2, 64, 512)
+    s.add_request(req(0, 5, 3)); s.add_request(req(1, 5, 3))
+    assert [x.request.request_id for x in s.schedule().seqs] == [0] and [r.request_id for r in s.waiting] == [1]
+    assert drive(s, None) == [0, 1]                         # the second one runs when the first has given its slot back
+    with pytest.raises(ValueError, match="starve"):
+        Scheduler(m, 8, 4, 512)
+    with pytest.raises(ValueError, match="at least one prompt token"):
+        s.add_request(Request(2, [], SamplingParams(max_new_tokens=1)))
+    with pytest.raises(ValueError, match="exceeds max_seq_len"):
+        s.add_request(req(3, 510, 3))
+
+
+@pytest.mark.parametrize("field,value", [("max_new_tokens", 0), ("max_new_tokens", 2.5), ("max_new_tokens", True),
+                                         ("temperature", -0.1), ("temperature", float("nan")), ("temperature", float("inf")),
+                                         ("top_p", 0.0), ("top_p", float("nan")), ("top_p", -1.0),
+                                         ("stop_token_ids", [3, "4"]), ("stop_token_ids", [1.0])])
+def test_sampling_options_that_make_no_sense_are_refused(field, value):
+    SamplingParams().validate()
+    SamplingParams(max_new_tokens=1, temperature=0.0, top_p=1.0).validate()
+    SamplingParams(temperature=3, top_p=5, stop_token_ids=[0, 7]).validate()       # top_p >= 1: no nucleus filter
+    with pytest.raises(ValueError, match=field):
+        SamplingParams(**{field: value}).validate()
