@@ -67,6 +67,8 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
     lens = [len(s.tokens) for s in seqs]
     if min(lens) < 1:
         raise BatchError("every sequence of a step brings at least one token")
+    if len({s.req for s in seqs}) != B:
+        raise BatchError("a request stands twice in one step: its tokens would take the same places in the cache")
     filler = 0
     if pad_tokens_to is not None:
         filler = pad_tokens_to - sum(lens)
