@@ -278,3 +278,54 @@ def test_named_configurations_parse_and_the_tiny_ones_differ_in_every_size():
     with pytest.raises(ValueError):
         preset("3b")
 
+
+
+def test_the_command_line_writes_a_model_folder_from_a_named_size_or_a_config_file(tmp_path, capsys):
+    from pico_vllm_amd import run
+    from pico_vllm_amd.config.presets import preset
+    from pico_vllm_amd.weights.safetensors_io import SafetensorsFile
+    a, b = str(tmp_path / "a"), str(tmp_path / "b")
+    assert run.main(["--write-random", a, "--random-config", "tiny-b", "--seed", "3"]) == 0
+    (tmp_path / "cfg.json").write_text(json.dumps(preset("tiny-b")))
+    assert run.main(["--write-random", b, "--config", str(tmp_path / "cfg.json"), "--seed", "3"]) == 0
+    assert capsys.readouterr().out.splitlines() == [f"wrote {a}", f"wrote {b}"]
+    with SafetensorsFile(os.path.join(a, "model.safetensors")) as fa, SafetensorsFile(os.path.join(b, "model.safetensors")) as fb:
+        assert fa.entries == fb.entries and len(fa.entries) > 10
+        assert all(torch.equal(fa.tensor(n), fb.tensor(n)) for n in fa.entries)
+    load_checkpoint(a, model_param_specs(load_model_description(a)[2]), torch.bfloat16)
+    for argv in (["--write-random", a], [], ["--random-config", "tiny-a"]):      # no size; no model; no prompt
+        with pytest.raises(SystemExit) as e:
+            run.main(argv)
+        assert e.value.code == 2
+    capsys.readouterr()
+
+
+def test_parts_are_found_by_category_and_kind_and_unknown_ones_are_named():
+    from pico_vllm_amd.parts.registry import CATEGORIES, part_class, register_part
+    assert part_class("position", "none").__name__ == "NoPosition"
+    assert {part_class(c, k).__name__ for c, k in (("mixer", "gqa_attention"), ("feed_forward", "swiglu_mlp"), ("norm", "rms_norm"),
+                                                     ("position", "rotary_half"), ("block", "prenorm"))} \
+        == {"GQAAttention", "SwiGLUMLP", "RMSNorm", "RotaryHalf", "PreNormBlock"}
+    with pytest.raises(KeyError, match="no mixer part of kind 'mamba' is registered; known: .*gqa_attention"):
+        part_class("mixer", "mamba")
+    with pytest.raises(KeyError, match="unknown part category 'router'"):
+        register_part("router", "top2")
+    with pytest.raises(KeyError, match="no router part"):
+        part_class("router", "top2")
+    assert set(CATEGORIES) == {"mixer", "feed_forward", "norm", "position", "block"}
+
+
+def test_parts_refuse_sizes_that_make_no_sense_when_they_are_built():
+    from pico_vllm_amd.parts.attention import GQAAttention
+    from pico_vllm_amd.parts.rotary import RotaryHalf
+    from pico_vllm_amd.parts.spec import PartSpec
+    none = PartSpec("none", {})
+    GQAAttention(64, 4, 2, 16, True, none)
+    for args, message in (((64, 4, 3, 16, True, none), "not a multiple"), ((64, 4, 2, 272, True, none), "head size"),
+                          ((64, 4, 2, 0, True, none), "head size")):
+        with pytest.raises(ValueError, match=message):
+            GQAAttention(*args)
+    with pytest.raises(ValueError, match="window must not be negative"):
+        GQAAttention(64, 4, 2, 16, True, none, window=-1)
+    with pytest.raises(ValueError, match="rotary_dim must be even"):
+        RotaryHalf(15, 10000.0)

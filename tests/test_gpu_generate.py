@@ -290,3 +290,38 @@ def test_phase_timers_behind_their_flag_change_nothing():
     assert rep["phases"]["model"]["device_ms"] > 0 and rep["phases"]["model"]["host_ms_per_call"] > 0
     assert rep["phases"]["schedule"]["calls"] >= steps and rep["phases"]["read"]["calls"] == steps
     assert rep["pages"][0]["in_use"] == 0 and rep["pages"][0]["peak"] > 0 and rep["graphs"]
+
+
+def test_what_generate_and_the_step_refuse_and_the_defaults_they_fall_back_to():
+    from pico_vllm_amd import LLM, SamplingParams
+    from pico_vllm_amd.engine.batch import BatchError, SeqStep
+    # no number of pages given: room for max_num_seqs requests of max_seq_len tokens
+    eng = LLM(model=model_dir("A"), dtype="float32", block_size=16, max_seq_len=100, max_num_seqs=3, max_num_batched_tokens=64,
+              use_cuda_graph=False)
+    assert eng.engine.runner.manager.groups[0].pool.num_pages == 3 * 7
+    prompts = prompts_for("A", [5, 9], seed=2)
+    outs = eng.generate(prompts)                                       # no options given: greedy, 16 tokens at most
+    assert all(1 <= len(o.token_ids) <= 16 for o in outs)
+    check_greedy("A", "float32", prompts, outs)
+    with pytest.raises(ValueError, match="one SamplingParams per prompt"):
+        eng.generate(prompts, [SamplingParams()] * 3)
+    with pytest.raises(ValueError, match="needs a tokenizer"):
+        eng.generate(["some text"])
+    with pytest.raises(ValueError, match="temperature"):
+        eng.generate(prompts, SamplingParams(temperature=float("nan")))
+    assert eng.engine.is_done()
+    # the step function itself
+    r = eng.engine.runner
+    m = r.manager
+    m.add_request("a"); m.add_request("b")
+    assert m.grow("a", 4) and m.grow("b", 1)
+    with pytest.raises(BatchError, match="single-token sequences only"):
+        r.step([SeqStep("a", [1, 2, 3, 4], [3]), SeqStep("b", [1], [0])], device_tokens=torch.zeros(2, dtype=torch.int32, device="cuda"))
+    m.advance("a", 4)
+    assert m.grow("a", 100)
+    with pytest.raises(BatchError, match="beyond max_seq_len=100"):
+        r.step([SeqStep("a", [1] * 97, [])])
+    logits = r.step([SeqStep("a", [1] * 60, [59]), SeqStep("b", [1], [0])])
+    assert logits.shape == (2, CONFIGS["A"]["vocab_size"]) and bool(torch.isfinite(logits).all())
+    m.free_request("a"); m.free_request("b")
+    m.check()

@@ -62,6 +62,15 @@ def test_add_rmsnorm(K, dtype, H):
     close(out, P.rms_norm(want_sum[rows.long()], w, eps), dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_residual_add(K, dtype):
+    # the add without a norm, for an arrangement of parts that ends on an add
+    resid, delta = torch.randn(7, 136) * 3, torch.randn(7, 136).to(dtype)
+    r = resid.clone().to(DEV)
+    assert K.residual_add(r, delta.to(DEV)) is r
+    assert torch.equal(r.cpu(), resid + delta.float())
+
+
 def test_rmsnorm_eps_is_inside_the_root(K):
     x = torch.full((1, 64), 1e-4)
     out = K.add_rmsnorm(x.to(DEV), None, torch.ones(64, device=DEV), 1e-2, torch.float32)
@@ -815,3 +824,116 @@ def test_gemm_skinny_refuses_misaligned_operands(K):
     assert not K.skinny_ok(torch.randn(257, 64).bfloat16().to(DEV), small)
     with pytest.raises(K.KernelError):
         K.gemm_skinny(torch.randn(257, 64).bfloat16().to(DEV), small)
+
+
+def test_the_wrappers_refuse_operands_that_do_not_fit_before_anything_is_launched(K):
+    # a kernel trusts the sizes it is given; what does not fit them is refused on the host, by name
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    bf, f32, i32 = torch.bfloat16, torch.float32, torch.int32
+
+    def dev(*shape, dtype=f32):
+        return torch.zeros(*shape, dtype=dtype, device=DEV)
+
+    def refused(message, fn, *args, **kw):
+        with pytest.raises(K.KernelError, match=message):
+            fn(*args, **kw)
+
+    T, H, V = 5, 64, 30
+    ids, table = dev(T, dtype=i32), dev(V, H)
+    refused("GPU only", K.embedding, table.cpu(), ids)
+    refused("not supported", K.embedding, table.half(), ids)
+    refused("contiguous int32", K.embedding, table, ids.long())
+    refused("table must be contiguous", K.embedding, dev(V, 2 * H)[:, ::2], ids)
+    refused("out must be", K.embedding, table, ids, out=dev(T, H, dtype=bf))
+    refused("softcap", K.softcap, dev(4, 4, dtype=bf), 2.0)
+    refused("softcap", K.softcap, dev(4, 4), 0.0)
+    resid, w = dev(T, H), dev(H)
+    refused("residual stream", K.add_rmsnorm, resid.to(bf), None, w, 1e-6, bf)
+    refused("norm weight", K.add_rmsnorm, resid, None, dev(H + 1), 1e-6, bf)
+    refused("partial sums must be float32", K.add_rmsnorm, resid, dev(2, T, H, dtype=bf), w, 1e-6, bf)
+    refused("shaped like the residual", K.add_rmsnorm, resid, dev(T, H + 8), w, 1e-6, bf)
+    refused("rows must be a contiguous int32", K.add_rmsnorm, resid, None, w, 1e-6, bf, rows=dev(2, dtype=torch.int64))
+    refused("out has the wrong shape", K.add_rmsnorm, resid, None, w, 1e-6, bf, out=dev(T, H))
+    refused("residual_add", K.residual_add, resid, dev(T, H + 8))
+    refused("swiglu: input", K.swiglu, dev(T, 7))
+    refused("swiglu: out", K.swiglu, dev(T, 8), out=dev(T, 8))
+    a, wf = dev(T, H), dev(9, H)
+    refused("inner sizes differ", K.gemm_f32, a, dev(9, H + 1))
+    refused("w must be float32", K.gemm_f32, a, wf.to(bf))
+    refused("bias must be", K.gemm_f32, a, wf, dev(8))
+    refused("out has the wrong", K.gemm_f32, a, wf, None, dev(T, 9, dtype=bf))
+    ab, wb = dev(T, H, dtype=bf), dev(16, H, dtype=bf)
+    refused("inner sizes differ", K.gemm_bf16, ab, dev(16, H + 8, dtype=bf))
+    refused("must be bfloat16", K.gemm_bf16, a, wb)
+    refused("bias must be", K.gemm_bf16, ab, wb, dev(16, dtype=bf))
+    refused("out has the wrong", K.gemm_bf16, ab, wb, None, bf, dev(T, 16))
+    refused("inner sizes differ", K.gemm_skinny, ab, dev(16, H + 8, dtype=bf))
+    refused("skinny_ok", K.gemm_skinny, dev(65, H, dtype=bf), dev((1 << 16) + 8, H, dtype=bf))   # many rows, a large matrix
+    refused("skinny_ok", K.gemm_skinny, dev(T, 60, dtype=bf), dev(16, 60, dtype=bf))       # K no multiple of 8
+    refused("bias must be", K.gemm_skinny, ab, wb, dev(15))
+    refused("partial sums", K.gemm_skinny, ab, wb, None, K.EPI_BF16, 2)
+    refused("even number", K.gemm_skinny, ab, dev(15, H, dtype=bf), None, K.EPI_SWIGLU)
+    assert not K.skinny_norm_ok(dev(2, H), None, wb) and not K.skinny_norm_ok(dev(1, H), dev(9, 1, H), wb)
+    assert K.skinny_norm_ok(dev(1, H), dev(3, 1, H), wb)
+    refused("skinny_norm_ok", K.gemm_skinny_norm, dev(2, H), None, w, 1e-6, wb)
+    refused("norm weight", K.gemm_skinny_norm, dev(1, H), None, dev(H + 1), 1e-6, wb)
+    refused("even number", K.gemm_skinny_norm, dev(1, H), None, w, 1e-6, dev(15, H, dtype=bf), K.EPI_SWIGLU)
+    # rotation and the cache: 2 query heads, 1 kv head of size 32, pages of 8
+    nq, nkv, d, Pg = 2, 1, 32, 8
+    kc, vc = dev(4, nkv, Pg, d, dtype=bf), dev(4, nkv, d, Pg, dtype=bf)
+    qkv, slots, cs = dev(T, (nq + 2 * nkv) * d, dtype=bf), dev(T, dtype=i32), dev(T, d // 2, 2)
+    K.rope_kv_store(qkv, cs, slots, kc, vc, nq, nkv, d, d)
+    refused("qkv must be contiguous", K.rope_kv_store, dev(T, 100, dtype=bf), cs, slots, kc, vc, nq, nkv, d, d)
+    refused("4-dimensional", K.rope_kv_store, qkv, cs, slots, kc[0], vc, nq, nkv, d, d)
+    refused("do not fit", K.rope_kv_store, qkv, cs, slots, kc, dev(4, nkv, Pg, d, dtype=bf), nq, nkv, d, d)
+    refused("differ in dtype", K.rope_kv_store, qkv, cs, slots, kc.float(), vc.float(), nq, nkv, d, d)
+    refused("slots has 5 entries, 6 are needed", K.rope_kv_store, dev(6, (nq + 2 * nkv) * d, dtype=bf), cs, slots, kc, vc, nq, nkv, d, d)
+    refused("table of cosines", K.rope_kv_store, qkv, dev(T, d // 2), slots, kc, vc, nq, nkv, d, d)
+    refused("table of cosines", K.rope_kv_store, qkv, None, slots, kc, vc, nq, nkv, d, d)
+    refused("inv_freq", K.rope_table, slots, dev(4, dtype=bf))
+    wq, bq = dev((nq + 2 * nkv) * d, H, dtype=bf), dev((nq + 2 * nkv) * d)
+    K.gemm_skinny_rope(ab, wq, bq, cs, slots, kc, vc, nq, nkv, d)
+    refused("weight .* is not", K.gemm_skinny_rope, ab, wb, None, cs, slots, kc, vc, nq, nkv, d)
+    refused("skinny_ok", K.gemm_skinny_rope, a, wq.float(), bq, cs, slots, kc, vc, nq, nkv, d)
+    refused("bias must be", K.gemm_skinny_rope, ab, wq, bq[:-1], cs, slots, kc, vc, nq, nkv, d)
+    refused("cache must be bfloat16", K.gemm_skinny_rope, ab, wq, bq, cs, slots, kc.float(), vc.float(), nq, nkv, d)
+    refused("multiple of 32", K.gemm_skinny_rope, ab, dev(4 * 16, H, dtype=bf), None, dev(T, 8, 2), slots,
+            dev(4, 1, Pg, 16, dtype=bf), dev(4, 1, 16, Pg, dtype=bf), 2, 1, 16)
+    r1, cs1 = dev(1, H), dev(1, d // 2, 2)
+    K.gemm_skinny_rope_norm(r1, None, w, 1e-6, wq, bq, cs1, slots, kc, vc, nq, nkv, d)
+    refused("skinny_norm_ok", K.gemm_skinny_rope_norm, dev(2, H), None, w, 1e-6, wq, bq, cs1, slots, kc, vc, nq, nkv, d)
+    refused("weight .* is not", K.gemm_skinny_rope_norm, r1, None, w, 1e-6, wb, None, cs1, slots, kc, vc, nq, nkv, d)
+    refused("bias must be", K.gemm_skinny_rope_norm, r1, None, w, 1e-6, wq, bq[:-1], cs1, slots, kc, vc, nq, nkv, d)
+    refused("cache must be bfloat16", K.gemm_skinny_rope_norm, r1, None, w, 1e-6, wq, bq, cs1, slots, kc.float(), vc.float(), nq, nkv, d)
+    refused("multiple of 32", K.gemm_skinny_rope_norm, r1, None, w, 1e-6, dev(4 * 16, H, dtype=bf), None, dev(1, 8, 2), slots,
+            dev(4, 1, Pg, 16, dtype=bf), dev(4, 1, 16, Pg, dtype=bf), 2, 1, 16)
+    # attention
+    q, bt, pos, seq = dev(T, nq * d, dtype=bf), dev(1, 4, dtype=i32), dev(T, dtype=i32), dev(T, dtype=i32)
+    K.paged_attention_ref(q, kc, vc, bt, pos, seq, nq, nkv, d, 0.1)
+    refused("unit stride", K.paged_attention_ref, q[:, :d], kc, vc, bt, pos, seq, nq, nkv, d, 0.1)
+    refused("differ in dtype", K.paged_attention_ref, q.float(), kc, vc, bt, pos, seq, nq, nkv, d, 0.1)
+    refused("block_table", K.paged_attention_ref, q, kc, vc, bt.long(), pos, seq, nq, nkv, d, 0.1)
+    refused("out has the wrong", K.paged_attention_ref, q, kc, vc, bt, pos, seq, nq, nkv, d, 0.1, out=dev(T, nq * d))
+    fa = FastAttention(nq, nkv, d)
+    ctxl, cu = torch.ones(T, dtype=i32, device=DEV), torch.arange(T + 1, dtype=i32, device=DEV)
+    bt5 = dev(T, 4, dtype=i32)
+    fa.decode(q, kc, vc, bt5, ctxl, T, 0.1, 1)
+    refused("one query token per sequence", fa.decode, q, kc, vc, bt5, ctxl, T - 1, 0.1, 1)
+    refused("at most 32 query heads", FastAttention(33, 1, d).decode, dev(T, 33 * d, dtype=bf), kc, vc, bt5, ctxl, T, 0.1, 1)
+    refused("bfloat16 tensors", fa.decode, q.float(), kc, vc, bt5, ctxl, T, 0.1, 1)
+    refused("unit stride", fa.prefill, q[:, :d], kc, vc, bt5, cu, ctxl, T, 0.1)
+    refused("block_table", fa.prefill, q, kc, vc, bt, cu, ctxl, T, 0.1)              # a table for one sequence, five given
+    refused("sequence metadata", fa.prefill, q, kc, vc, bt5, cu.long(), ctxl, T, 0.1)
+    refused("sequence metadata", fa.decode, q, kc, vc, bt5, ctxl[:2], T, 0.1, 1)
+    # sampling
+    logits, t1 = dev(3, V), dev(3)
+    K.sample(logits, t1, t1 + 1, t1)
+    refused("logits must be float32", K.sample, logits.to(bf), t1, t1, t1)
+    refused("top_p must be", K.sample, logits, t1, dev(2), t1)
+    refused("out must be", K.sample, logits, t1, t1, t1, dev(3))
+    work = K.argmax_workspace(3, DEV)
+    K.argmax(logits, dev(3, dtype=i32), work)
+    refused("logits must be float32", K.argmax, logits.to(bf), dev(3, dtype=i32), work)
+    refused("out must be", K.argmax, logits, dev(2, dtype=i32), work)
+    refused("workspace", K.argmax, logits, dev(3, dtype=i32), K.argmax_workspace(2, DEV))
+    torch.cuda.synchronize()

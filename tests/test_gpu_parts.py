@@ -713,6 +713,75 @@ def test_layers_with_and_without_a_window_in_one_model(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_layer_without_position_encoding_between_layers_with_rotation(dtype):
+    """The framework's own "none" position encoding in layer 1, rotation in the others: keys and values of that layer are
+    stored as they are.  A prompt in portions, then token by token (in bfloat16 a single row reaches the attention as a
+    norm still to be run, which this encoding does not take over), with and without recorded steps; against the plain
+    computation of that model, which differs from the one with rotation everywhere."""
+    import dataclasses
+    import tempfile
+    from pico_vllm_amd.config.model_config import Qwen2Config
+    from pico_vllm_amd.config.qwen2 import qwen2_spec
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.spec import LayerSpec, PartSpec
+    from pico_vllm_amd.weights.random_init import write_random_model
+    from tiny_configs import TINY_B, strong
+
+    def spec_with_a_bare_layer(cfg):
+        spec = qwen2_spec(cfg)
+        l1 = spec.layers[1]
+        name, attn = l1.slots["mixer"]
+        bare = PartSpec(attn.kind, dict(attn.params, position=PartSpec("none", {})))
+        layers = list(spec.layers)
+        layers[1] = LayerSpec(l1.prefix, l1.block, {**l1.slots, "mixer": (name, bare)})
+        return dataclasses.replace(spec, layers=layers)
+    register_architecture("ToyBareLayerLM", Qwen2Config.from_dict, spec_with_a_bare_layer)
+    cfg = dict(TINY_B, architectures=["ToyBareLayerLM"])
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=12, std_overrides=strong(cfg))
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        plain = P.PlainModel(d)
+        w, c = plain.w, plain.cfg
+
+        def want(toks, rnd):
+            nq, nkv, hd = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+            pos = torch.arange(len(toks))
+            x = w["model.embed_tokens.weight"][toks].float()
+            for i in range(c.num_hidden_layers):
+                p = f"model.layers.{i}"
+                h = rnd(P.rms_norm(x, w[f"{p}.input_layernorm.weight"], c.rms_norm_eps))
+                Wm = torch.cat([w[f"{p}.self_attn.{n}_proj.weight"] for n in "qkv"])
+                b = torch.cat([w[f"{p}.self_attn.{n}_proj.bias"] for n in "qkv"])
+                q, k, v = P.split_qkv(rnd(h @ Wm.T + b), nq, nkv, hd)
+                if i != 1:
+                    cos, sin = P.rope_tables(pos, hd, c.rope_theta)
+                    q, k = rnd(P.apply_rope(q, cos, sin)), rnd(P.apply_rope(k, cos, sin))
+                o = rnd(P.causal_attention(q, k, v, rnd_p=None if rnd is P._same else rnd))
+                x = x + rnd(o.reshape(len(toks), nq * hd) @ w[f"{p}.self_attn.o_proj.weight"].T)
+                x = x + P.mlp_layer(rnd(P.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], c.rms_norm_eps)), w, p, rnd)
+            return rnd(P.rms_norm(x, w["model.norm.weight"], c.rms_norm_eps)) @ w["lm_head.weight"].T
+        toks = torch.randint(0, 383, (70,), generator=torch.Generator().manual_seed(5)).tolist()
+        assert float((want(toks, P._same) - plain.logits(toks)).abs().max()) > 0.05 * float(plain.logits(toks).std())
+        for graphs in (False, True):
+            r = ModelRunner(model, 8, 24, 2, 64, 96, use_graph=graphs, max_graph_batch=2)
+            assert r.use_graph == graphs
+            r.manager.add_request("a")
+            got, fed = [], 0
+            for n in [23, 2, 17] + [1] * 28:
+                assert r.manager.grow("a", fed + n)
+                seqs = [SeqStep("a", toks[fed:fed + n], [n - 1] if graphs else list(range(n)))]
+                got.append(r.step(seqs).clone())
+                r.advance(seqs)
+                fed += n
+            assert fed == 70
+            rows = [22, 24, 41] + list(range(42, 70)) if graphs else list(range(70))
+            close_to_plain(torch.cat(got), want(toks, P._same)[rows], want(toks, P.to_bf16)[rows], dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_a_toy_norm_and_a_toy_arrangement_of_the_parts(dtype):
     """The two remaining kinds of part, defined and registered here: a norm that centres on the mean and has a
     bias (the framework's subtracts nothing and has none), and an arrangement in which the mixer and the
