@@ -329,3 +329,45 @@ def test_parts_refuse_sizes_that_make_no_sense_when_they_are_built():
         GQAAttention(64, 4, 2, 16, True, none, window=-1)
     with pytest.raises(ValueError, match="rotary_dim must be even"):
         RotaryHalf(15, 10000.0)
+
+
+def test_a_description_that_does_not_hold_together_is_refused_when_the_model_is_built():
+    import dataclasses
+    from pico_vllm_amd.config.qwen2 import qwen2_spec
+    from pico_vllm_amd.ops.linear import Linear
+    from pico_vllm_amd.parts.model import DecoderModel, load_model
+    from pico_vllm_amd.parts.spec import LayerSpec, PartSpec, RunEntry
+    from tiny_configs import TINY_B
+    spec = qwen2_spec(Qwen2Config.from_dict(TINY_B))
+    assert len(spec.layers) == 3
+    model = DecoderModel(spec, torch.float32, "cpu")               # building needs no GPU, only running does
+    assert sorted(model.cache_specs()) == [0, 1, 2]
+
+    def refused(message, **changes):
+        with pytest.raises(ValueError, match=message):
+            DecoderModel(dataclasses.replace(spec, **changes), torch.float32, "cpu")
+
+    refused("run order names layer 5, the model has 3", run_order=[RunEntry(0), RunEntry(5)])
+    refused("run entry 1: cache_of must name an earlier entry", run_order=[RunEntry(0), RunEntry(1, cache_of=1)])
+    refused("run entry 2: cache_of must name an earlier entry that owns its cache",
+            run_order=[RunEntry(0), RunEntry(1, cache_of=0), RunEntry(2, cache_of=1)])
+    shared = DecoderModel(dataclasses.replace(spec, run_order=[RunEntry(0), RunEntry(1, cache_of=0), RunEntry(0)]), torch.float32, "cpu")
+    assert sorted(shared.cache_specs()) == [0, 2]                  # the second run reads the first one's cache
+    l1 = spec.layers[1]
+    name, attn = l1.slots["mixer"]
+    windowed = LayerSpec(l1.prefix, l1.block, {**l1.slots, "mixer": (name, PartSpec(attn.kind, dict(attn.params, window=8)))})
+    refused("run entry 1 cannot use the cache of entry 0: different cache needs",
+            layers=[spec.layers[0], windowed, spec.layers[2]], run_order=[RunEntry(0), RunEntry(1, cache_of=0), RunEntry(2)])
+    no_ff = LayerSpec(l1.prefix, l1.block, {k: v for k, v in l1.slots.items() if k != "ff"})
+    refused(r"layer model.layers.1: block 'prenorm' needs slots \['ff'\]", layers=[spec.layers[0], no_ff, spec.layers[2]])
+    with pytest.raises(ValueError, match="dtype must be one of"):
+        load_model(model_dir("A"), "float16", "cpu")
+    # the matrix product's own refusals
+    with pytest.raises(ValueError, match="a linear weight is a matrix"):
+        Linear(torch.zeros(8))
+    lin = Linear(torch.zeros(4, 8, dtype=torch.bfloat16), torch.zeros(4))
+    assert (lin.out_features, lin.in_features) == (4, 8) and lin.bias.dtype == torch.bfloat16 and lin.bias_f32.dtype == torch.float32
+    with pytest.raises(ValueError, match="input has 6 features, the weight wants 8"):
+        lin(torch.zeros(2, 6, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="bfloat16 weights need bfloat16 activations"):
+        lin(torch.zeros(2, 8))

@@ -325,3 +325,40 @@ def test_what_generate_and_the_step_refuse_and_the_defaults_they_fall_back_to():
     assert logits.shape == (2, CONFIGS["A"]["vocab_size"]) and bool(torch.isfinite(logits).all())
     m.free_request("a"); m.free_request("b")
     m.check()
+
+
+def test_the_sizes_that_reports_are_made_of_and_the_measured_peaks():
+    from pico_vllm_amd.ops import peaks
+    from pico_vllm_amd.sampling.sampler import Sampler
+    eng = llm("B", "bfloat16").engine
+    c = CONFIGS["B"]
+    H, I, V, L = c["hidden_size"], c["intermediate_size"], c["vocab_size"], c["num_hidden_layers"]
+    nq, nkv = c["num_attention_heads"], c["num_key_value_heads"]
+    d = c.get("head_dim", H // nq)
+    per_layer = (nq + 2 * nkv) * d * H + H * nq * d + 2 * I * H + H * I          # q/k/v, o, gate/up, down
+    assert not c["tie_word_embeddings"]
+    assert eng.model.num_weight_bytes() == 2 * (L * per_layer + V * H)           # and the output matrix once
+    per_token = L * 2 * nkv * d * 2
+    assert eng.runner.storage.bytes_per_token() == per_token
+    assert eng.runner.storage.num_bytes() == per_token * 64 * PAGE_SIZE["B"]     # 64 pages
+    assert eng.runner.decode_bytes([10, 300]) == eng.model.num_weight_bytes() + 310 * per_token
+    tied = llm("A", "bfloat16").engine
+    a = CONFIGS["A"]
+    assert a["tie_word_embeddings"]
+    da = a.get("head_dim", a["hidden_size"] // a["num_attention_heads"])
+    per_layer = ((a["num_attention_heads"] + 2 * a["num_key_value_heads"]) * da * a["hidden_size"]
+                 + a["hidden_size"] * a["num_attention_heads"] * da + 3 * a["intermediate_size"] * a["hidden_size"])
+    assert tied.model.num_weight_bytes() == 2 * (a["num_hidden_layers"] * per_layer + a["vocab_size"] * a["hidden_size"])
+    # the two yardsticks of the benchmark: what a read stream and a loop of matrix-core products reach on this GPU
+    stream = peaks.read_bandwidth(num_bytes=1 << 30, reps=5)
+    flops, seconds = peaks.mfma_peak(reps=3, iters=4000)
+    assert 2e12 < stream < 8e12 and 0.8e15 < flops < 2.6e15 and seconds > 0, (stream, flops)
+    # the sampler's own refusals, and one call that launches and reads
+    sm = Sampler(torch.device("cuda:0"), 2)
+    logits = torch.zeros(3, 50, device="cuda")
+    logits[0, 7] = logits[1, 9] = 1.0
+    assert sm.sample(logits[:2], [0.0, 0.0], [1.0, 1.0], [1, 2], [0, 0]) == [7, 9]
+    with pytest.raises(ValueError, match="one set of sampling parameters per row"):
+        sm.launch(logits[:2], [0.0], [1.0, 1.0], [1, 2], [0, 0])
+    with pytest.raises(ValueError, match="3 rows to sample, the sampler was made for 2"):
+        sm.launch(logits, [0.0] * 3, [1.0] * 3, [1, 2, 3], [0] * 3)

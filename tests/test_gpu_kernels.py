@@ -937,3 +937,28 @@ def test_the_wrappers_refuse_operands_that_do_not_fit_before_anything_is_launche
     refused("out must be", K.argmax, logits, dev(2, dtype=i32), work)
     refused("workspace", K.argmax, logits, dev(3, dtype=i32), K.argmax_workspace(2, DEV))
     torch.cuda.synchronize()
+
+
+def test_the_library_product_with_its_tuner_on_gives_the_same_and_hands_the_mode_back():
+    # rows in multiples of 512 are timed by the library's tuner when asked; other counts take its default; off again
+    # torch's own mode is as it was
+    from pico_vllm_amd.ops import linear as L
+    g = torch.Generator().manual_seed(0)
+    x, w, b = torch.randn(1024, 320, generator=g).bfloat16(), torch.randn(200, 320, generator=g).bfloat16(), torch.randn(200, generator=g)
+    lin = L.Linear(w.to(DEV), b.to(DEV))
+    want = x.double() @ w.double().T + b.bfloat16().double()
+    before = lin(x.to(DEV))
+    assert not torch.cuda.tunable.is_enabled()
+    L.set_library_tuning(True)
+    try:
+        tuned = lin(x.to(DEV))                    # 1,024 rows: tuned
+        assert torch.cuda.tunable.is_enabled() and torch.cuda.tunable.tuning_is_enabled()
+        other = lin(x[:300].to(DEV))              # 300 rows: the library's default choice, nothing is timed
+        assert not torch.cuda.tunable.tuning_is_enabled()
+        no_bias = L.Linear(w.to(DEV))(x[:512].to(DEV))
+    finally:
+        L.set_library_tuning(False)
+    assert not torch.cuda.tunable.is_enabled() and not torch.cuda.tunable.tuning_is_enabled()
+    for got, ref in ((before, want), (tuned, want), (other, want[:300]), (no_bias, want[:512] - b.bfloat16().double())):
+        assert got.dtype == torch.bfloat16
+        assert torch.allclose(got.cpu().double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(320))

@@ -405,3 +405,29 @@ def test_the_program_itself_in_a_subprocess():
                 for row, key in zip(a, rows):
                     got[key] = row
         compare("A", "float32", reqs, got, "program")
+
+
+def test_the_program_says_what_is_wrong_with_a_trace(tmp_path):
+    import io
+    from pico_vllm_amd.engine.batch import BatchError
+    from pico_vllm_amd.engine.replay import TraceReplayer, main
+    V = CONFIGS["A"]["vocab_size"]
+    rp = TraceReplayer(model_dir("A"), "float32", max_tokens=64, page_size=PAGE_SIZE["A"])
+    pool = rp.runner.manager.groups[0].pool
+    out = rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3], "want": [2]}], "end": []})
+    assert out.shape == (1, V) and out.dtype == np.float32
+    assert rp.run_step({"step": 1, "entries": [{"id": "a", "tokens": [4, 5]}]}) is None          # nothing wanted: no file
+    with pytest.raises(RuntimeError, match="step 2: out of cache pages for request b"):
+        rp.run_step({"step": 2, "entries": [{"id": "b", "tokens": [1] * 80, "want": []}], "end": []})
+    with pytest.raises(BatchError, match="token id outside"):
+        rp.run_step({"step": 3, "entries": [{"id": "a", "tokens": [V], "want": [0]}], "end": []})
+    with pytest.raises(BatchError, match="wanted place 5"):
+        rp.run_step({"step": 4, "entries": [{"id": "a", "tokens": [1, 2], "want": [5]}], "end": []})
+    with pytest.raises(BatchError, match="stands twice"):
+        rp.run_step({"step": 5, "entries": [{"id": "a", "tokens": [1], "want": [0]}, {"id": "a", "tokens": [2], "want": [0]}]})
+    assert rp.run_step({"step": 6, "entries": [], "end": ["a", "b", "never seen"]}) is None
+    rp.runner.manager.check()
+    assert pool.num_free == pool.num_pages and not rp.live
+    with pytest.raises(json.JSONDecodeError):
+        main(["--model", model_dir("A"), "--dtype", "float32", "--out", str(tmp_path), "--max-tokens", "64"],
+             stdin=io.StringIO("{\"step\": 0, \"entries\": [\n"), stdout=io.StringIO())
