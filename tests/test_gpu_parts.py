@@ -313,6 +313,109 @@ def test_a_toy_mixer_with_state_of_its_own_registers_builds_and_steps(dtype):
         assert one_slot == eager or dtype != torch.float32
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_toy_mixer_that_keeps_nothing_beside_a_layer_with_attention(dtype):
+    """A mixer that works on every token by itself (y = (x Wv) * sigmoid(x Wg)) says nothing about a cache: the
+    default is none, its run gets no pages and no state, and the attention layer behind it has the model's only
+    group of pages.  Whole against a plain computation, portions against whole, and generation with recorded decode
+    steps against generation without."""
+    import tempfile
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.base import Mixer
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import LayerSpec, ModelSpec, ParamSpec, PartSpec, RunEntry
+    from pico_vllm_amd.weights.random_init import write_random_model
+    H, V, NQ, NKV, D, I = 48, 120, 3, 1, 16, 80
+
+    @register_part("mixer", "toy_gated_linear")
+    class GatedLinear(Mixer):
+        def __init__(self, hidden_size, act_dtype=torch.bfloat16):
+            self.H = hidden_size
+
+        def param_specs(self):
+            return [ParamSpec("value.weight", (self.H, self.H), std=0.3), ParamSpec("gate.weight", (self.H, self.H), std=0.3)]
+
+        def load(self, tensors, device, dtype):
+            self.wv, self.wg = tensors["value.weight"].to(device), tensors["gate.weight"].to(device)
+
+        def forward(self, x, ctx, cache):
+            assert cache is None
+            return ((x @ self.wv.T).float() * torch.sigmoid((x @ self.wg.T).float())).to(x.dtype)
+
+    def toy_spec(cfg):
+        norm = PartSpec("rms_norm", {"size": H, "eps": 1e-5})
+        attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": D, "qkv_bias": True,
+                                          "window": 0, "position": PartSpec("rotary_half", {"rotary_dim": D, "theta": 100.0})})
+        ff = PartSpec("swiglu_mlp", {"hidden_size": H, "intermediate_size": I})
+        mixers = [PartSpec("toy_gated_linear", {"hidden_size": H}), attn]
+        layers = [LayerSpec(f"toy.layers.{i}", "prenorm", {"norm1": ("ln1", norm), "mixer": ("mix", mixers[i]), "norm2": ("ln2", norm),
+                                                          "ff": ("ff", ff)}) for i in range(2)]
+        return ModelSpec(H, V, "toy.embed.weight", layers, [RunEntry(0), RunEntry(1)], norm, "toy.norm", None)
+
+    register_architecture("ToyGatedLinearLM", lambda raw: raw, toy_spec)
+    rnd = P._same if dtype == torch.float32 else P.to_bf16
+    kind = "float32" if dtype == torch.float32 else "bfloat16"
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, {"architectures": ["ToyGatedLinearLM"]}, seed=6, std_overrides={"mix": 0.3, "embed": 0.5, "ff": 0.3})
+        w = {k: v.float() for k, v in P.read_weights(d).items()}
+        model = load_model(d, kind, DEV)
+        r = ModelRunner(model, 8, 16, 3, 64, 64)
+        assert [g.layers for g in r.manager.groups] == [[1]] and not r.manager.state_layers
+        assert r.storage.layer(0) is None and r.storage.layer(1) is not None
+        toks = torch.randint(0, V, (37,), generator=torch.Generator().manual_seed(2)).tolist()
+
+        def plain(rnd):
+            pos = torch.arange(len(toks))
+            x = w["toy.embed.weight"][toks]
+            h = rnd(P.rms_norm(x, w["toy.layers.0.ln1.weight"], 1e-5))
+            x = x + rnd(rnd(h @ w["toy.layers.0.mix.value.weight"].T) * torch.sigmoid(rnd(h @ w["toy.layers.0.mix.gate.weight"].T)))
+            for i in range(2):
+                p = f"toy.layers.{i}"
+                if i == 1:
+                    h = rnd(P.rms_norm(x, w[f"{p}.ln1.weight"], 1e-5))
+                    W = torch.cat([w[f"{p}.mix.{n}_proj.weight"] for n in "qkv"], 0)
+                    b = torch.cat([w[f"{p}.mix.{n}_proj.bias"] for n in "qkv"], 0)
+                    q, k, v = P.split_qkv(rnd(h @ W.T + b), NQ, NKV, D)
+                    cos, sin = P.rope_tables(pos, D, 100.0)
+                    o = rnd(P.causal_attention(rnd(P.apply_rope(q, cos, sin)), rnd(P.apply_rope(k, cos, sin)), v,
+                                               rnd_p=None if rnd is P._same else rnd))
+                    x = x + rnd(o.reshape(len(toks), NQ * D) @ w[f"{p}.mix.o_proj.weight"].T)
+                h = rnd(P.rms_norm(x, w[f"{p}.ln2.weight"], 1e-5))
+                gu = torch.cat([w[f"{p}.ff.gate_proj.weight"], w[f"{p}.ff.up_proj.weight"]], 0)
+                x = x + rnd(rnd(P.swiglu(rnd(h @ gu.T))) @ w[f"{p}.ff.down_proj.weight"].T)
+            return rnd(P.rms_norm(x, w["toy.norm.weight"], 1e-5)) @ w["toy.embed.weight"].T
+
+        r.manager.add_request("w")
+        assert r.manager.grow("w", len(toks))
+        whole = r.step([SeqStep("w", toks, list(range(len(toks))))])
+        r.manager.free_request("w")
+        close_to_plain(whole, plain(P._same), plain(rnd), dtype)
+        r.manager.add_request("a")
+        got, fed = [], 0
+        for n in (11, 1, 2, 20, 1, 1, 1):
+            assert r.manager.grow("a", fed + n)
+            seqs = [SeqStep("a", toks[fed:fed + n], list(range(n)))]
+            got.append(r.step(seqs))
+            r.advance(seqs)
+            fed += n
+        close(torch.cat(got), whole, dtype, scale=float(whole.std()) * 3)
+        r.manager.check()
+        del r, model
+        from pico_vllm_amd import LLM, SamplingParams
+        prompts = [toks[:9], toks[9:12], toks[12:]]
+        sp = SamplingParams(max_new_tokens=10, temperature=0.0, ignore_eos=True)
+
+        def run(**kw):
+            llm = LLM(model=d, dtype=kind, block_size=8, num_gpu_blocks=24, max_seq_len=64, max_num_seqs=2, max_num_batched_tokens=64, **kw)
+            return [o.token_ids for o in llm.generate(prompts, sp)], llm.engine.runner
+        graphed, runner = run(use_cuda_graph=True, max_batch_size=2)
+        assert runner.use_graph and runner._graphs
+        assert graphed == run(use_cuda_graph=False)[0]
+
+
 def test_a_part_that_decides_on_the_host_keeps_the_model_out_of_graphs():
     """``graph_safe = False`` on any part: the runner never records a graph, whatever the options say."""
     import dataclasses
