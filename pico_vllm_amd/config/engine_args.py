@@ -26,7 +26,7 @@ class EngineArgs:
     max_num_batched_tokens: int = 2048   # token budget of one step
     use_cuda_graph: bool = True          # replay pure-decode steps from a captured HIP graph
     max_batch_size: int = 8              # largest decode batch that has a graph
-    graph_prompts: bool = True           # with use_cuda_graph: a prompt portion that is a step of its own replays a graph too
+    graph_prompts: bool = True           # with use_cuda_graph: a step that is one prompt portion, alone or behind decoding requests, replays a graph too
     manual_seed: int = 42
     pipeline_decode: bool = True         # keep one decode step in flight while the host prepares the next
     tune_library_gemm: bool = False      # let the library time its solutions for whole prompt portions (stalls the first such step)

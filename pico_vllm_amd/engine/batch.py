@@ -58,28 +58,39 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
     recorded at that size) with one more sequence of filler tokens behind the given ones: positions
     from 0, a context of its own length, a block table of -1, slots of -1, the spare state slot,
     nothing wanted; it may be empty.
+    Both: single-token sequences followed by ONE prompt portion.  The single tokens are padded with empty rows to
+    ``pad_to`` of them (the empty rows stand between the real ones and the portion, and are wanted like them), and
+    the portion with filler to ``pad_tokens_to`` tokens: ``pad_to + pad_tokens_to`` tokens in ``pad_to + 2`` sequences.
     """
     B = len(seqs)
     if B == 0:
         raise BatchError("a step needs at least one sequence")
-    if pad_to and pad_tokens_to:
-        raise BatchError("a step is padded with rows or with tokens, not with both")
     lens = [len(s.tokens) for s in seqs]
     if min(lens) < 1:
         raise BatchError("every sequence of a step brings at least one token")
     if len({s.req for s in seqs}) != B:
         raise BatchError("a request stands twice in one step: its tokens would take the same places in the cache")
+    mixed = bool(pad_to) and pad_tokens_to is not None
     filler = 0
-    if pad_tokens_to is not None:
+    if mixed:
+        if max(lens[:-1], default=1) != 1 or pad_to < B - 1:
+            raise BatchError(f"a step padded both ways is single tokens (at most {pad_to}) followed by one prompt portion")
+        filler = pad_tokens_to - lens[-1]
+        empty = pad_to - (B - 1)
+        rows = pad_to + 2
+        T = pad_to + pad_tokens_to
+    elif pad_tokens_to is not None:
         filler = pad_tokens_to - sum(lens)
-        if filler < 0:
-            raise BatchError(f"the step has {sum(lens)} tokens, more than the {pad_tokens_to} it is to be padded to")
+        empty = 0
         rows = B + 1
         T = pad_tokens_to
     else:
         rows = max(B, pad_to or 0)
-        T = sum(lens) + (rows - B)
-    R = sum(len(s.want) for s in seqs) + (rows - B if pad_to else 0)
+        empty = rows - B
+        T = sum(lens) + empty
+    if filler < 0:
+        raise BatchError(f"the step has {sum(lens) if not mixed else lens[-1]} tokens, more than the {pad_tokens_to} it is to be padded to")
+    R = sum(len(s.want) for s in seqs) + (empty if pad_to else 0)
     P = manager.page_size
     if T > buf.max_tokens or rows > buf.max_seqs or R > buf.max_want:
         raise BatchError(f"step of {T} tokens / {rows} sequences / {R} wanted rows exceeds the buffers "
@@ -101,8 +112,25 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
     t = 0
     r = 0
     h_cu[0] = 0
-    for b, s in enumerate(seqs):
-        n = lens[b]
+    spare = manager.slots.num_slots                # the state slot that no request ever holds
+    # the rows of the step: the given sequences in their order; empty rows behind them, or (padded both ways) in front
+    # of the portion that stands last; the filler at the very end
+    row_of = list(range(B)) if not mixed else list(range(B - 1)) + [pad_to]
+
+    def empty_rows(first: int, end: int) -> None:
+        nonlocal t, r
+        for e in range(first, end):
+            h_tok[t] = 0; h_pos[t] = 0; h_seq[t] = e
+            h_want[r] = t; r += 1
+            t += 1
+            h_cu[e + 1] = t
+            h_ctx[e] = 0
+            h_slot[e] = spare
+
+    for b, s in zip(row_of, seqs):
+        if mixed and b == pad_to:
+            empty_rows(B - 1, pad_to)              # between the single tokens and the portion
+        n = len(s.tokens)
         cached = manager.num_computed(s.req)
         if n == 1:
             tok = s.tokens[0]
@@ -140,27 +168,25 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         h_slot[b] = manager.slot(s.req)
         max_ctx = max(max_ctx, cached + n)
         need_pages = max(need_pages, -(-(cached + n) // P))
+    last = row_of[-1] + 1                          # the first row behind the given sequences
     if pad_tokens_to is not None:                  # the sequence of filler tokens of a recorded prompt step
         h_tok[t:T] = 0
         h_pos[t:T] = np.arange(filler)
-        h_seq[t:T] = B
-        h_cu[B + 1] = T
-        h_ctx[B] = filler
-        h_slot[B] = manager.slots.num_slots
+        h_seq[t:T] = last
+        h_cu[last + 1] = T
+        h_ctx[last] = filler
+        h_slot[last] = spare
     else:
-        for b in range(B, rows):                   # padding rows of a captured decode batch
-            h_tok[t] = 0; h_pos[t] = 0; h_seq[t] = b
-            h_want[r] = t; r += 1
-            t += 1
-            h_cu[b + 1] = t
-            h_ctx[b] = 0
-            h_slot[b] = manager.slots.num_slots   # the spare slot that no request ever holds
+        empty_rows(last, rows)                     # padding rows of a captured decode batch
     width = buf.max_pages if (pad_to or pad_tokens_to is not None) else need_pages
     if width > buf.max_pages:
         raise BatchError(f"a sequence needs {width} pages, the buffers hold {buf.max_pages} per sequence")
     tables = h[bt_off:bt_off + G * rows * width].reshape(G, rows, width)
     tables[:] = -1
-    for b, s in enumerate(seqs):
+    if rows > B:
+        for g in range(G):
+            h_slots[g][:] = -1                                          # padding rows and filler store nothing
+    for b, s in zip(row_of, seqs):
         need = -(-int(h_ctx[b]) // P)
         lo, hi = int(h_cu[b]), int(h_cu[b + 1])
         for g in range(G):
@@ -168,8 +194,6 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
             tables[g, b, :need] = table
             pos = h_pos[lo:hi]
             h_slots[g][lo:hi] = table[pos // P] * P + pos % P          # pico_vllm/cache.py:143-156
-    for g in range(G):
-        h_slots[g][int(h_cu[B]):T] = -1                               # padding rows store nothing
     used = bt_off + G * rows * width
     buf.dev[:used].copy_(buf.host[:used], non_blocking=True)
     if buf.copied is not None:

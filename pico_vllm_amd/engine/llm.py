@@ -214,7 +214,7 @@ class LLMEngine:
         out["pages"] = [{"window": g.window, "layers": len(g.layers), "total": g.pool.num_pages, "in_use": g.pool.num_used,
                          "peak": g.pool.peak_used, "reused": g.pool.reuse_count} for g in m.groups]
         out["graphs"] = sorted(self.runner._graphs)
-        out["prompt_graphs"] = sorted(key[0] for key in self.runner._prompt_graphs)
+        out["prompt_graphs"] = sorted((key[0], key[1]) for key in self.runner._prompt_graphs)   # (single tokens, portion)
         if self.timers.enabled:
             out["phases"] = self.timers.report()
         return out

@@ -12,7 +12,10 @@ of 8, engine.py:98-137).  A step that is one prompt portion alone replays a
 graph too, recorded at the next of a few sizes and padded to it with filler
 tokens in a sequence of their own: such a step is a few hundred launches and
 library calls that cost the host more than they cost the GPU (4.1 ms against
-1.6 ms for 300 tokens of the 1.5B shape).
+1.6 ms for 300 tokens of the 1.5B shape).  So does a step of a few decoding
+requests and one prompt portion of up to ``MIXED_GRAPH_TOKENS`` tokens (what
+continuous serving under a small token budget consists of), its single tokens
+padded to a power of two as in a decode step.
 """
 from __future__ import annotations
 
@@ -44,6 +47,11 @@ def prompt_sizes(most: int) -> List[int]:
     return [s for s in out if s <= most]
 
 
+# A step of single tokens and one prompt portion is recorded only up to this many tokens of the portion: beyond it
+# the GPU's work outweighs what the launches cost the host, and every recorded shape costs two warm-up runs.
+MIXED_GRAPH_TOKENS = 1024
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_size: int, num_pages: int, max_seqs: int,
                  max_tokens_per_step: int, max_seq_len: int, use_graph: bool = False, max_graph_batch: int = 8,
@@ -56,17 +64,19 @@ class ModelRunner:
         self.max_pages = -(-max_seq_len // page_size)
         self.max_seq_len = max_seq_len
         # a decode batch is padded to the power of two its graph was captured at: rows for that too
-        # (and a recorded prompt step has a second sequence, of filler)
-        rows = max(max_seqs, _bucket(min(max_seqs, max_graph_batch)), 2) if use_graph else max_seqs
-        self.buffers = BatchBuffers(self.device, max(max_tokens_per_step, rows), rows, self.max_pages,
-                                    max(1, len(self.manager.groups)))
+        # (and a recorded prompt step has a sequence of filler, and may have padded single tokens in front)
+        padded = _bucket(min(max_seqs, max_graph_batch))
+        rows = max(max_seqs, padded + 2) if use_graph else max_seqs
+        self.buffers = BatchBuffers(self.device, max(max_tokens_per_step + (padded if use_graph else 0), rows), rows,
+                                    self.max_pages, max(1, len(self.manager.groups)))
         # a part that decides on the host per step (``Part.graph_safe`` False) keeps the whole model out of graphs
         self.use_graph = use_graph and model.is_graph_safe()
         self.graph_prompts = self.use_graph and graph_prompts and model.is_graph_safe(prompts=True)
         self.prompt_sizes = prompt_sizes(min(max_tokens_per_step, self.max_pages * page_size))
         self.max_graph_batch = max_graph_batch
         self._graphs: Dict[int, tuple] = {}
-        self._prompt_graphs: Dict[tuple, tuple] = {}       # (recorded size, wanted rows, the parts' choices) -> (graph, logits)
+        # (padded single tokens, recorded size of the portion, its wanted rows, the parts' choices) -> (graph, logits)
+        self._prompt_graphs: Dict[tuple, tuple] = {}
         # all graphs take their intermediate tensors from one pool (they never run at the same time), so that a
         # dozen recorded sizes hold the memory of the largest, not of all
         self._graph_pool = torch.cuda.graph_pool_handle() if self.use_graph else None
@@ -107,14 +117,15 @@ class ModelRunner:
         if self.use_graph and decode_only and len(seqs) <= self.max_graph_batch:
             logits = self._step_graph(seqs, device_tokens)
         elif size:
-            logits = self._step_prompt_graph(seqs[0], size)
+            logits = self._step_prompt_graph(seqs, size)
+            if back is not None:
+                logits = logits.index_select(0, torch.tensor(back, dtype=torch.long, device=logits.device))
         else:
             ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size)
-            if decode_only:
-                # the kernel choices of a recorded decode step (how the context is split over workgroups) hold for
-                # any context; a decode step that is not replayed makes the same ones, so that a request gets the
-                # same tokens with and without graphs
-                ctx.max_context = self.max_seq_len
+            # the kernel choices of a recorded step for its single tokens (how their contexts are split over
+            # workgroups) hold for any context; a step that is not replayed makes the same ones, so that a request
+            # gets the same tokens with and without graphs
+            ctx.max_context = self.max_seq_len
             if device_tokens is not None:
                 ctx.token_ids[:len(seqs)].copy_(device_tokens[:len(seqs)])
             logits = self.model.forward(ctx, self.storage)
@@ -143,27 +154,38 @@ class ModelRunner:
 
     # ---- graph replay of a prompt portion alone ---------------------------
     def _prompt_size(self, seqs: List[SeqStep]) -> int:
-        """The recorded size that serves this step, or 0: one sequence of two tokens or more and at most one
-        wanted row.  (The filler is a sequence of its own with positions from 0, so it needs no room behind the
-        request's tokens.)"""
-        if len(seqs) != 1 or len(seqs[0].tokens) < 2 or len(seqs[0].want) > 1:
+        """The recorded size that serves this step's prompt portion, or 0.  What is recorded: one sequence of two
+        tokens or more with at most one wanted row, alone or behind single tokens (each wanted, no more of them than
+        a recorded decode step takes) if the portion is short enough for the launches to outweigh the work.  (The
+        filler is a sequence of its own with positions from 0, so it needs no room behind the request's tokens.)"""
+        last = seqs[-1]
+        if len(last.tokens) < 2 or len(last.want) > 1:
             return 0
-        n = len(seqs[0].tokens)
+        singles = len(seqs) - 1
+        if singles and (singles > self.max_graph_batch or any(len(s.tokens) != 1 or list(s.want) != [0] for s in seqs[:-1])):
+            return 0
+        n = len(last.tokens)
         for size in self.prompt_sizes:
             if size >= n:
-                return size
+                return size if not singles or size <= MIXED_GRAPH_TOKENS else 0
         return 0
 
-    def _step_prompt_graph(self, seq: SeqStep, size: int) -> torch.Tensor:
-        ctx = build_context([seq], self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
-                            pad_tokens_to=size)
+    def _step_prompt_graph(self, seqs: List[SeqStep], size: int) -> torch.Tensor:
+        singles = len(seqs) - 1
+        rows = _bucket(singles) if singles else 0
+        ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size,
+                            pad_to=rows or None, pad_tokens_to=size)
+        if rows:
+            ctx.max_context = self.max_seq_len      # as in a recorded decode step: choices that hold for any context
         # what parts choose on the host for this step (a kernel's shape for a short or a long context) is part of
         # the key: a replay runs what the step would run unrecorded
-        key = (size, len(seq.want), self.model.graph_variant(ctx))
+        key = (rows, size, len(seqs[-1].want), self.model.graph_variant(ctx))
         if key not in self._prompt_graphs:
             self._prompt_graphs[key] = self._record(ctx)        # leaves the step's arrays as they are
         graph, out = self._prompt_graphs[key]
         graph.replay()
+        if rows > singles:                                       # drop the rows of the padding
+            out = torch.cat([out[:singles], out[rows:]])
         return out
 
     def _capture(self, size: int, seqs: List[SeqStep]) -> None:

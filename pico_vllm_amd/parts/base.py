@@ -60,9 +60,11 @@ class Part:
 
     ``graph_safe_prompts``: the same for a step that is one prompt portion, which is recorded padded: behind the
     portion's sequence stands a second one of filler tokens (slot -1, a block table of -1, outputs ignored) that
-    brings the step to a recorded size.  A part that says True does device work only in such a step, may take what
-    it decides on the host from the step that was recorded (``ctx.host`` is that step's), and keeps nothing of the
-    filler.  The default is False: prompt steps of a model with such a part run unrecorded.
+    brings the step to a recorded size; in front of the portion there may be sequences of one token each, the last
+    of them empty rows as in a recorded decode step (context 0, a block table of -1, the spare state slot).  A part
+    that says True does device work only in such a step, may take what it decides on the host from the step that
+    was recorded (``ctx.host`` is that step's), and keeps nothing of the filler or the empty rows.  The default is
+    False: prompt steps of a model with such a part run unrecorded.
 
     ``graph_variant(ctx)``: what such a part decides on the host for a prompt step (a kernel's shape, say), as
     something hashable.  Steps whose variants differ are recorded apart, so that a replayed step runs what the

@@ -79,6 +79,38 @@ def test_rows_of_padding_and_a_sequence_of_filler():
     assert build_context([SeqStep("r0", [1] * 5, [])], m, buf, torch.bfloat16, VOCAB, pad_tokens_to=5).num_tokens == 5
 
 
+def test_single_tokens_and_one_portion_padded_both_ways():
+    # three requests with one token each, padded to four rows, in front of a portion of 5 tokens padded to 16
+    m, buf = setup([10, 3, 30, 24], [1, 1, 1, 5])
+    seqs = [SeqStep(f"r{i}", [i + 1], [0]) for i in range(3)] + [SeqStep("r3", [1, 2, 3, 4, 5], [4])]
+    ctx = build_context(seqs, m, buf, torch.bfloat16, VOCAB, pad_to=4, pad_tokens_to=16)
+    assert (ctx.num_tokens, ctx.num_seqs, ctx.all_decode, ctx.max_new_tokens) == (20, 6, False, 5)
+    assert ctx.token_ids.tolist() == [1, 2, 3, 0, 1, 2, 3, 4, 5] + [0] * 11
+    assert ctx.positions.tolist() == [10, 3, 30, 0, 24, 25, 26, 27, 28] + list(range(11))
+    assert ctx.token_seq.tolist() == [0, 1, 2, 3] + [4] * 5 + [5] * 11
+    assert ctx.cu_seqlens.tolist() == [0, 1, 2, 3, 4, 9, 20]
+    assert ctx.context_lens.tolist() == [11, 4, 31, 0, 29, 11]
+    assert ctx.want_rows.tolist() == [0, 1, 2, 3, 8]                  # the empty row is wanted like the real ones
+    spare = m.slots.num_slots
+    assert ctx.state_slots.tolist() == [m.slot("r0"), m.slot("r1"), m.slot("r2"), spare, m.slot("r3"), spare]
+    for g in range(2):
+        assert ctx.block_tables[g].shape == (6, buf.max_pages)
+        assert ctx.block_tables[g][3].tolist() == [-1] * buf.max_pages == ctx.block_tables[g][5].tolist()
+        want = [m.token_slot(f"r{i}", c, g) for i, c in enumerate([10, 3, 30])] + [-1] \
+            + [m.token_slot("r3", 24 + j, g) for j in range(5)] + [-1] * 11
+        assert ctx.slot_mapping[g].tolist() == want
+        assert ctx.block_tables[g][4].tolist()[:4] == m.block_table("r3", g)[:4]
+    assert ctx.host["cu_seqlens"].tolist() == ctx.cu_seqlens.tolist() and ctx.host["context_lens"].tolist() == ctx.context_lens.tolist()
+    # no single token at all is allowed too (rows of padding only), and so is a full house
+    ctx = build_context(seqs[3:], m, buf, torch.bfloat16, VOCAB, pad_to=2, pad_tokens_to=8)
+    assert ctx.cu_seqlens.tolist() == [0, 1, 2, 7, 10] and ctx.context_lens.tolist() == [0, 0, 29, 3] and ctx.want_rows.tolist() == [0, 1, 6]
+    ctx = build_context(seqs, m, buf, torch.bfloat16, VOCAB, pad_to=3, pad_tokens_to=5)
+    assert ctx.cu_seqlens.tolist() == [0, 1, 2, 3, 8, 8] and ctx.want_rows.tolist() == [0, 1, 2, 7]
+    # a step after it that is not padded leaves nothing of it behind
+    ctx = build_context(seqs, m, buf, torch.bfloat16, VOCAB)
+    assert ctx.cu_seqlens.tolist() == [0, 1, 2, 3, 8] and ctx.slot_mapping[0].tolist()[3:] == [m.token_slot("r3", 24 + j, 0) for j in range(5)]
+
+
 def test_what_a_step_refuses():
     m, buf = setup([10, 3], [4, 1])
     a, b = SeqStep("r0", [1, 2, 3, 4], [3]), SeqStep("r1", [5], [0])
@@ -88,7 +120,10 @@ def test_what_a_step_refuses():
             build_context(seqs, m, buf, torch.bfloat16, VOCAB, **pad)
 
     refused([], "at least one sequence")
-    refused([a, b], "not with both", pad_to=4, pad_tokens_to=16)
+    refused([a, b], "followed by one prompt portion", pad_to=4, pad_tokens_to=16)        # the portion stands last
+    m.add_request("r2"); m.grow("r2", 1)
+    refused([b, SeqStep("r2", [1], [0]), a], "followed by one prompt portion", pad_to=1, pad_tokens_to=16)   # more single tokens than rows
+    refused([b, a], "more than the 2", pad_to=2, pad_tokens_to=2)
     refused([a, SeqStep("r1", [], [])], "at least one token")
     refused([a, SeqStep("r0", [9], [0])], "stands twice")
     refused([a], "more than the 2", pad_tokens_to=2)

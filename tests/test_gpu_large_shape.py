@@ -267,13 +267,69 @@ def test_prompt_steps_replayed_from_graphs_at_sizes_that_take_the_library_produc
             r.manager.free_request(rid)
     assert sizes_seen.count(320) >= 3 and 1024 in sizes_seen          # a recorded size was replayed after other work
     assert len(rec._prompt_graphs) >= 4 and not raw._prompt_graphs
+    # Steps of decoding requests and one prompt portion are recorded too: the single tokens padded to a power of two
+    # with empty rows, the portion to a recorded size with filler.  Each replay against the same padded step unrecorded,
+    # bit for bit, and against the plain implementation.
+    def both_mixed(seqs):
+        outs = []
+        singles = len(seqs) - 1
+        for r in (rec, raw):
+            m = r.manager
+            for q in seqs:
+                if q.req not in m.requests:
+                    assert m.add_request(q.req)
+                assert m.grow(q.req, m.num_computed(q.req) + len(q.tokens))
+            if r is rec:
+                size = r._prompt_size(seqs)
+                before = len(r._prompt_graphs)
+                outs.append(r.step(seqs).clone())
+            else:
+                rows = 1
+                while rows < singles:
+                    rows *= 2
+                ctx = build_context(seqs, m, wide, model.dtype, V, pad_to=rows, pad_tokens_to=size)
+                ctx.max_context = r.max_seq_len
+                out = model.forward(ctx, r.storage)
+                outs.append(torch.cat([out[:singles], out[rows:]]).clone())
+            r.advance(seqs)
+        torch.cuda.synchronize()
+        return outs[0], outs[1], size, len(rec._prompt_graphs) - before
+
+    from pico_vllm_amd.engine.batch import BatchBuffers
+    wide = BatchBuffers(model.device, 2048 + 4, 6, raw.max_pages, 1)      # room for the padding, which the unrecording runner never needs
+    lens = {"d0": 40, "d1": 333, "d2": 7}
+    text = {rid: [rng.randrange(V) for _ in range(n + 8)] for rid, n in lens.items()}
+    text["new"] = [rng.randrange(V) for _ in range(700)]
+    at = dict(lens, new=0)
+    for rid, n in lens.items():
+        both(rid, text[rid][:n], [n - 1])
+    recorded = 0
+    for live, n in ((["d0", "d1", "d2"], 100), (["d1"], 37), (["d0", "d2"], 250), (["d2", "d0", "d1"], 2), (["d1", "d0", "d2"], 120),
+                    (["d0"], 40), (["d1", "d2"], 110)):
+        seqs = [SeqStep(rid, text[rid][at[rid]:at[rid] + 1], [0]) for rid in live] + [SeqStep("new", text["new"][at["new"]:at["new"] + n], [n - 1])]
+        a, b, size, fresh = both_mixed(seqs)
+        recorded += fresh
+        assert size >= n and a.shape == (len(live) + 1, V) and torch.equal(a, b), (live, n, size)
+        for q, row in zip(seqs, a):
+            at[q.req] += len(q.tokens)
+            ref = plain.logits(text[q.req][:at[q.req]])[-1]
+            assert float((row.cpu() - ref).abs().max()) < 0.1 * float(ref.std()), (live, n, q.req)
+    # seven steps, five shapes: (4 rows, 128), (1, 64), (2, 256), (4, 16) and (2, 128) were recorded, two were replays of them
+    assert recorded == 5 and sorted(k[:2] for k in rec._prompt_graphs if k[0]) == [(1, 64), (2, 128), (2, 256), (4, 16), (4, 128)]
+    big = [SeqStep("d0", [1], [0]), SeqStep("new", [1] * 140, [139])]
+    assert rec._prompt_size(big[1:]) == 192 and rec._prompt_size(big) == 192
+    big[1] = SeqStep("new", [1] * 1100, [0])
+    assert rec._prompt_size(big[1:]) == 1280 and not rec._prompt_size(big)              # beyond 1,024 tokens only alone
+    for r in (rec, raw):
+        for rid in at:
+            r.manager.free_request(rid)
     # What the attention chooses on the host (the shape of its prefill workgroups) differs between a first portion and
     # one behind thousands of tokens: the two are recorded apart, and each replay is the unrecorded step bit for bit.
     toks = [rng.randrange(V) for _ in range(6000)]
     for at, n in ((0, 2048), (2048, 2048), (4096, 1900)):
         a, b, size = both("long", toks[at:at + n], [n - 1])
         assert size == 2048 and torch.equal(a, b), (at, n)
-    variants = {key[2] for key in rec._prompt_graphs if key[0] == 2048}
+    variants = {key[3] for key in rec._prompt_graphs if key[1] == 2048}
     assert len(variants) >= 2, variants
     del rec, raw, model
     torch.cuda.empty_cache()
