@@ -168,20 +168,20 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
     return res, model
 
 
-def prefill_point(model_dir, model, dtype, reps=7):
+def prefill_point(model_dir, model, dtype, reps=7, tokens=PREFILL_TOKENS):
     import torch
     from pico_vllm_amd.engine.batch import SeqStep
     peak = measured_peaks()[1] if dtype == "bfloat16" else None       # before the timed steps: a profile ends with them
     eng = make_engine(model_dir, dtype, 1, model)
     V = CONFIG["vocab_size"]
-    ids = torch.randint(0, V, (PREFILL_TOKENS,), generator=torch.Generator().manual_seed(7)).tolist()
+    ids = torch.randint(0, V, (tokens,), generator=torch.Generator().manual_seed(7)).tolist()
     m = eng.runner.manager
     times = []
     for i in range(reps + 1):
         rid = f"p{i}"
         m.add_request(rid)
-        assert m.grow(rid, PREFILL_TOKENS)
-        seq = [SeqStep(rid, ids, [PREFILL_TOKENS - 1])]
+        assert m.grow(rid, tokens)
+        seq = [SeqStep(rid, ids, [tokens - 1])]
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record()
@@ -192,8 +192,8 @@ def prefill_point(model_dir, model, dtype, reps=7):
         m.free_request(rid)
     times = sorted(times[1:])                         # the first run builds, tunes and warms
     dt = times[len(times) // 2]
-    flops = prefill_flops(CONFIG, PREFILL_TOKENS)
-    out = {"value": PREFILL_TOKENS / dt, "tokens": PREFILL_TOKENS, "ms": dt * 1e3, "ms_min": times[0] * 1e3,
+    flops = prefill_flops(CONFIG, tokens)
+    out = {"value": tokens / dt, "tokens": tokens, "ms": dt * 1e3, "ms_min": times[0] * 1e3,
            "tflops": flops / dt / 1e12, "frac": flops / dt / MFMA_PEAK[dtype]}
     if peak is not None:
         out["measured_peak_tflops"] = peak / 1e12
@@ -348,6 +348,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill (long workload: the decode points)")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="with --prefill-only: the prompt's length (2 to 2048; the contract's prefill is of 2,048 tokens)")
     ap.add_argument("--write-model", metavar="DIR", default=None,
                     help="only write the random-weights model folder to DIR (to reuse with --model) and exit")
     ap.add_argument("--model", default=None, help="reuse a model folder instead of writing random weights")
@@ -377,6 +379,9 @@ def main() -> int:
     CONTEXT = a.context
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
+        return 2
+    if not 2 <= a.prefill_tokens <= PREFILL_TOKENS:
+        print(f"bench.py: --prefill-tokens must be 2..{PREFILL_TOKENS}")
         return 2
     if CONTEXT < 2 * PREFILL_TOKENS or a.steps + a.warmup >= CONTEXT // 2 - 200:
         print(f"bench.py: the context must be at least {2 * PREFILL_TOKENS} and steps + warmup below {CONTEXT // 2 - 200}")
@@ -430,7 +435,7 @@ def main() -> int:
                            "preemptions": r["preemptions"]}}), flush=True)
             return 0
         if a.prefill_only:
-            print(json.dumps({"prefill": prefill_point(model_dir, preloaded, a.dtype)}), flush=True)
+            print(json.dumps({"prefill": prefill_point(model_dir, preloaded, a.dtype, tokens=a.prefill_tokens)}), flush=True)
             return 0
         if a.workload == "sweep":
             rows = sweep_point(model_dir, preloaded, a.dtype, a.batch)
