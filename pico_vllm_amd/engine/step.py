@@ -38,13 +38,18 @@ def _bucket(n: int) -> int:
 
 def prompt_sizes(most: int) -> List[int]:
     """The sizes at which prompt steps are recorded: 16, 32, 64, then steps of 64 to 512, of 128 to 1,024 and of
-    256 beyond, up to ``most``: at most a quarter of a recorded step is filler, beyond 64 tokens an eighth."""
+    256 beyond, up to ``most``, and ``most`` itself (a step's token budget: the size of most portions of a long
+    prompt): less than half of a recorded step is filler for portions of 16 tokens or more, a third from 128 on,
+    a fifth from 512 on."""
     out = [16, 32]
     n = 64
     while n <= most:
         out.append(n)
         n += 64 if n < 512 else 128 if n < 1024 else 256
-    return [s for s in out if s <= most]
+    out = [s for s in out if s <= most]
+    if most >= 2 and most not in out:
+        out.append(most)
+    return out
 
 
 # A step of single tokens and one prompt portion is recorded only up to this many tokens of the portion: beyond it

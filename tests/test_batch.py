@@ -137,3 +137,17 @@ def test_what_a_step_refuses():
     with pytest.raises(BatchError, match="needs 2 pages, the buffers hold 1"):
         build_context([a], m, small, torch.bfloat16, VOCAB)
     build_context([a, b], m, buf, torch.bfloat16, VOCAB)              # and the step itself is fine
+
+
+def test_the_sizes_at_which_prompt_steps_are_recorded():
+    from pico_vllm_amd.engine.step import prompt_sizes
+    assert prompt_sizes(2048) == [16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1280, 1536, 1792, 2048]
+    assert prompt_sizes(24) == [16, 24] and prompt_sizes(300) == [16, 32, 64, 128, 192, 256, 300] and prompt_sizes(8) == [8]
+    assert prompt_sizes(1) == [] and prompt_sizes(16) == [16] and prompt_sizes(64) == [16, 32, 64]
+    for most in (24, 300, 2048, 5000):
+        sizes = prompt_sizes(most)
+        assert sizes == sorted(set(sizes)) and sizes[-1] == most
+        for n in range(2, most + 1):                     # every portion finds a size, with little filler
+            size = next(s for s in sizes if s >= n)
+            filler = size - n
+            assert filler < 16 if n < 16 else 2 * filler < size if n < 128 else 3 * filler <= size if n < 512 else 5 * filler <= size

@@ -115,6 +115,30 @@ def test_decode_steps_replayed_from_a_graph_give_the_same_tokens(dtype):
     check_greedy("A", dtype, prompts[:2], more)
 
 
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
+def test_steps_of_decoding_requests_and_a_prompt_portion_replayed_from_graphs_give_the_same_tokens(name, dtype):
+    # a small token budget: while prompts are still coming in, most steps are a few decoding requests and one portion of a
+    # prompt; those are recorded with the single tokens padded to a power of two and the portion to a recorded size
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for(name, [40, 9, 77, 23, 51, 30, 64], seed=5)
+    sps = [SamplingParams(max_new_tokens=n, temperature=t, top_p=0.9, seed=i, ignore_eos=True)
+           for i, (n, t) in enumerate([(30, 0.0), (45, 0.0), (12, 0.7), (40, 0.0), (25, 0.0), (33, 0.9), (8, 0.0)])]
+    kw = dict(num_gpu_blocks=160, max_num_seqs=4, max_num_batched_tokens=32, max_seq_len=128)
+    eager = llm(name, dtype, **kw).generate(prompts, sps)
+    graph_llm = llm(name, dtype, use_cuda_graph=True, max_batch_size=4, **kw)
+    graphed = graph_llm.generate(prompts, sps)
+    keys = list(graph_llm.engine.runner._prompt_graphs)
+    assert any(k[0] > 0 for k in keys), "no step of single tokens and a portion went through a graph"
+    assert any(k[0] == 0 for k in keys) and graph_llm.engine.runner._graphs
+    assert {k[0] for k in keys} <= {0, 1, 2, 4}
+    assert [o.token_ids for o in graphed] == [o.token_ids for o in eager]
+    check_greedy(name, dtype, [prompts[i] for i in (0, 1, 3, 4, 6)], [graphed[i] for i in (0, 1, 3, 4, 6)])
+    # nothing is recorded when the option says so
+    off = llm(name, dtype, use_cuda_graph=True, max_batch_size=4, graph_prompts=False, **kw)
+    assert [o.token_ids for o in off.generate(prompts, sps)] == [o.token_ids for o in eager]
+    assert not off.engine.runner._prompt_graphs and off.engine.runner._graphs
+
+
 def test_running_out_of_pages_preempts_and_recomputes_to_the_same_tokens():
     from pico_vllm_amd import SamplingParams
     prompts = prompts_for("A", [30, 30, 30], seed=4)
