@@ -157,7 +157,7 @@ class ModelRunner:
         graph.replay()
         return out[:B]
 
-    # ---- graph replay of a prompt portion alone ---------------------------
+    # ---- graph replay of a prompt portion, alone or behind single tokens --
     def _prompt_size(self, seqs: List[SeqStep]) -> int:
         """The recorded size that serves this step's prompt portion, or 0.  What is recorded: one sequence of two
         tokens or more with at most one wanted row, alone or behind single tokens (each wanted, no more of them than
