@@ -461,11 +461,20 @@ def paged_attention_ref(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     return out
 
 
+def sample_workspace(rows: int, device) -> torch.Tensor:
+    """What ``sample`` needs beside its output for up to ``rows`` rows (partial results of its chain of launches)."""
+    lib = library.core()
+    lib.pico_sample_workspace_words.restype = ctypes.c_longlong
+    return torch.empty(max(2, int(lib.pico_sample_workspace_words(rows))), dtype=torch.int32, device=device)
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, u: torch.Tensor,
-           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+           out: Optional[torch.Tensor] = None, work: Optional[torch.Tensor] = None, top_p_rows: bool = True) -> torch.Tensor:
     """One token id per row of float32 logits; per-row temperature (0 = greedy), top_p and
-    uniform number."""
-    _gpu(logits, temperature, top_p, u)
+    uniform number.  ``work``: ``sample_workspace`` for at least as many rows (made here if not given).
+    ``top_p_rows=False``: the caller knows that no row has top_p < 1, and the launches that look for the
+    threshold of such rows are left out (a top_p below 1 is then taken as 1)."""
+    _gpu(logits, temperature, top_p, u, work)
     R, V = logits.shape
     if logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise KernelError("sample: logits must be float32 with unit stride along the vocabulary")
@@ -477,8 +486,15 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     elif out.dtype != torch.int32 or out.numel() < R or not out.is_contiguous():
         raise KernelError("sample: out must be contiguous int32 with one entry per row")
     lib = library.core()
+    if work is None:
+        work = sample_workspace(R, logits.device)
+    else:
+        lib.pico_sample_workspace_words.restype = ctypes.c_longlong
+        if work.dtype != torch.int32 or not work.is_contiguous() or work.numel() < int(lib.pico_sample_workspace_words(R)) \
+                or work.data_ptr() % 8:
+            raise KernelError("sample: the workspace must come from sample_workspace for at least as many rows")
     _check(lib, lib.pico_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature),
-                                _ptr(top_p), _ptr(u), _ptr(out), _stream()))
+                                _ptr(top_p), _ptr(u), _ptr(out), _ptr(work), int(bool(top_p_rows)), _stream()))
     return out
 
 

@@ -42,6 +42,7 @@ class Sampler:
         self._dev = torch.zeros(3, max_rows, dtype=torch.float32, device=device)
         self._out = torch.zeros(max_rows, dtype=torch.int32, device=device)
         self._argmax_work = kernels.argmax_workspace(max_rows, device) if torch.cuda.is_available() else None
+        self._sample_work = kernels.sample_workspace(max_rows, device) if torch.cuda.is_available() else None
         self._host_np = [h.numpy() for h in self._host]
         self._landing = [torch.zeros(max_rows, dtype=torch.int32, pin_memory=torch.cuda.is_available()) for _ in range(2)]
         self._landed = [torch.cuda.Event() if torch.cuda.is_available() else None for _ in range(2)]
@@ -85,7 +86,8 @@ class Sampler:
             h[1, :R] = top_ps
             h[2, :R] = [uniform(s, i) if t > 0 else 0.0 for s, i, t in zip(seeds, indices, temperatures)]
             self._dev.copy_(self._host[self._turn], non_blocking=True)
-            kernels.sample(logits, self._dev[0], self._dev[1], self._dev[2], self._out)
+            kernels.sample(logits, self._dev[0], self._dev[1], self._dev[2], self._out, self._sample_work,
+                           top_p_rows=any(t > 0 and p < 1 for t, p in zip(temperatures, top_ps)))
         turn = self._turn
         self._turn ^= 1
         self._landing[turn][:R].copy_(self._out[:R], non_blocking=True)

@@ -323,6 +323,42 @@ def test_sampling_top_p_keeps_a_prefix_of_tied_tokens(K):
         assert seen == kept, (probs.tolist()[:5], top_p, sorted(seen))
 
 
+def test_sampling_at_the_real_vocabulary_row_by_row(K):
+    # 151,936 logits a row, rows of every kind side by side: greedy, plain temperature, wide and narrow nuclei, flat and
+    # peaked distributions.  Every row against the plain rule, and the same token when the row is sampled alone.
+    g = torch.Generator().manual_seed(21)
+    R, V = 14, 151936
+    logits = torch.randn(R, V, generator=g) * torch.tensor([1, 1, 3, 3, 3, 8, 8, 0.1, 0.1, 20, 20, 3, 3, 3.0])[:, None]
+    temps = torch.tensor([0.0, 1.0, 0.7, 0.7, 1.3, 1.0, 0.5, 1.0, 1.0, 1.0, 2.0, 0.0, 0.9, 1.1])
+    top_ps = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.05, 0.95, 0.3, 0.9, 0.999, 0.8, 0.6, 0.5, 1.0, 0.99])
+    us = torch.rand(R, generator=g)
+    dev = logits.to(DEV)
+    work = K.sample_workspace(R, DEV)
+    out = K.sample(dev, temps.to(DEV), top_ps.to(DEV), us.to(DEV), work=work).tolist()
+    assert out == K.sample(dev, temps.to(DEV), top_ps.to(DEV), us.to(DEV), work=work).tolist()      # and again: the same
+    exact = 0
+    for r in range(R):
+        alone = K.sample(dev[r:r + 1], temps[r:r + 1].to(DEV), top_ps[r:r + 1].to(DEV), us[r:r + 1].to(DEV))
+        assert int(alone[0]) == out[r], (r, int(alone[0]), out[r])
+        if temps[r] == 0:
+            assert out[r] == P.sample_greedy(logits[r])
+            continue
+        p = P.top_p_probs(logits[r].double(), float(temps[r]), float(top_ps[r]))
+        assert float(p[out[r]]) > 0, (r, "a token outside the kept set")
+        want = P.inverse_cdf(p, float(us[r]))
+        cum = torch.cumsum(p, 0)
+        exact += out[r] == want
+        # equal, or u falls within rounding of a boundary of the CDF (float32 exponentials against float64 ones)
+        assert out[r] == want or abs(float(cum[min(out[r], want)]) - float(us[r])) < 1e-4, (r, out[r], want)
+    assert exact >= R - 3
+    # rows that are known to have no nucleus skip the search for it
+    plain_rows = torch.ones(R, device=DEV)
+    assert K.sample(dev, temps.to(DEV), plain_rows, us.to(DEV), top_p_rows=False).tolist() \
+        == K.sample(dev, temps.to(DEV), plain_rows, us.to(DEV)).tolist()
+    with pytest.raises(K.KernelError, match="workspace"):
+        K.sample(dev, temps.to(DEV), top_ps.to(DEV), us.to(DEV), work=K.sample_workspace(R - 1, DEV))
+
+
 def test_sampling_top_p(K):
     probs = torch.tensor([[0.05, 0.5, 0.15, 0.3]])
     logits = torch.log(probs)
