@@ -115,6 +115,7 @@ __global__ __launch_bounds__(SAMPLE_ROUND_THREADS) void sample_round_kernel(
     const float* __restrict__ top_p, const float* __restrict__ part_val, const float* __restrict__ prev,
     float* __restrict__ next, uint32_t* __restrict__ state, int first) {
   __shared__ float hist[SAMPLE_CLASSES][SAMPLE_ROUND_THREADS];   // a column per thread: no two threads share an entry
+  __shared__ float halves[2][SAMPLE_CLASSES];
   __shared__ uint32_t result[4];
   const int row = blockIdx.x, c = blockIdx.y, tid = threadIdx.x;
   // everything the workgroup needs from memory is asked for at once, whatever it turns out to need: what the launch
@@ -173,15 +174,18 @@ __global__ __launch_bounds__(SAMPLE_ROUND_THREADS) void sample_round_kernel(
     for (int k = 0; k < 8; k++) v[k] = ahead[k];
   }
   __syncthreads();
-  float* mine = next + ((size_t)row * SAMPLE_CHUNKS + c) * SAMPLE_CLASSES;
-  const int wave = tid >> 6, lane = tid & 63;
-  for (int m = wave; m < SAMPLE_CLASSES; m += SAMPLE_ROUND_THREADS / 64) {
-    float v = hist[m][lane];
-#pragma unroll
-    for (int k = 1; k < SAMPLE_ROUND_THREADS / 64; k++) v += hist[m][lane + 64 * k];
-    v = wave_sum(v);
-    if (lane == 0) mine[m] = v;
-  }
+  // Thread (m, half) adds the entries of class m of one half of the threads, one after the other (no exchange between
+  // lanes: 32 reductions over a wave would be 32 chains of six exchanges); it starts at column m so that the lanes of a
+  // wave read different banks.
+  static_assert(SAMPLE_ROUND_THREADS == 128 && SAMPLE_CLASSES == 64, "two halves of 64 threads, a class a lane");
+  const int m = tid & 63, half = tid >> 6;
+  float sum = 0.f;
+#pragma unroll 16
+  for (int j = 0; j < 64; j++) sum += hist[m][half * 64 + ((j + m) & 63)];
+  halves[half][m] = sum;
+  __syncthreads();
+  if (tid < SAMPLE_CLASSES)
+    next[((size_t)row * SAMPLE_CHUNKS + c) * SAMPLE_CLASSES + tid] = halves[0][tid] + halves[1][tid];
 }
 
 __device__ __forceinline__ double wave_sum_f64(double v) {
