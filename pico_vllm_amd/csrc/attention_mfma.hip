@@ -181,7 +181,7 @@ __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf
     s[r] = v;
     mx = fmaxf(mx, v);
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = max_across_32(mx);
   const float m_new = fmaxf(st.m, mx);
   const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column with nothing visible yet
   const float alpha = __expf(st.m - m_use);
@@ -192,7 +192,7 @@ __device__ __forceinline__ void attend_subtile(const Tiles& t, int sub, const bf
     s[r] = p;
     sum += p;
   }
-  sum += __shfl_xor(sum, 32, 64);
+  sum = sum_across_32(sum);
   st.l = st.l * alpha + sum;
   st.m = m_new;
 #pragma unroll
@@ -257,7 +257,7 @@ __device__ __forceinline__ void attend_tile(const Tiles& t, int nsub, const bf16
       }
     }
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = max_across_32(mx);
   const float m_new = fmaxf(st.m, mx);
   const bool outgrown = (m_new - st.m) * c > 8.0f;          // also true while the reference is -inf
   if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {          // the same decision for the whole wave
@@ -283,7 +283,7 @@ __device__ __forceinline__ void attend_tile(const Tiles& t, int nsub, const bf16
       }
     }
   }
-  sum += __shfl_xor(sum, 32, 64);
+  sum = sum_across_32(sum);
   st.l += sum;
 #pragma unroll
   for (int sub = 0; sub < NS; sub++) {
@@ -615,8 +615,8 @@ __device__ __forceinline__ void pf_attend(const bf16_t* krow, const bf16_t* vrow
         }
         mx = fmaxf(mx, s[b][j][r]);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_across_16(mx);
+    mx = max_across_32(mx);
     const float m_new = fmaxf(st[b].m, mx);
     const bool outgrown = (m_new - st[b].m) * c > 8.0f;        // also true while the reference is -inf
     if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {          // the same decision for the whole wave
@@ -862,8 +862,8 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     for (int qb = 0; qb < NQB; qb++) {
       if (!q_ok[qb]) continue;
       float l = st[qb].l;
-      l += __shfl_xor(l, 16, 64);
-      l += __shfl_xor(l, 32, 64);
+      l = sum_across_16(l);
+      l = sum_across_32(l);
       float* prow = part + (((size_t)(tok0 + q_idx[qb]) * nq + head) * max_chunks + chunk) * PF_PART_ROW + 4 * kq;
 #pragma unroll
       for (int tt = 0; tt < PF_DT; tt++) *reinterpret_cast<f32x4p*>(prow + 16 * tt) = st[qb].o[tt];
@@ -878,8 +878,8 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   for (int qb = 0; qb < NQB; qb++) {
     if (!q_ok[qb]) continue;
     float l = st[qb].l;
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = sum_across_16(l);
+    l = sum_across_32(l);
     const float inv_l = 1.0f / l;
     bf16_t* orow = out + ((size_t)(tok0 + q_idx[qb]) * nq + head) * D + 4 * kq;
 #pragma unroll
@@ -1117,8 +1117,8 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
         sv[r] = v;
         mx = fmaxf(mx, v);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_across_16(mx);
+      mx = max_across_32(mx);
       const float m_new = fmaxf(m, mx);                        // finite: the block holds at least one key in lo .. k_end - 1
       const float alpha = __expf(m - m_new);
       float sum = 0.f;
@@ -1127,8 +1127,8 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
         sv[r] = __expf(sv[r] - m_new);
         sum += sv[r];
       }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
+      sum = sum_across_16(sum);
+      sum = sum_across_32(sum);
       l = l * alpha + sum;
       m = m_new;
       const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack2_bf16(sv[0], sv[1]), pack2_bf16(sv[2], sv[3]),

@@ -50,17 +50,52 @@ template <typename T> __device__ __forceinline__ void store_f32(T* p, float v);
 template <> __device__ __forceinline__ void store_f32<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
-// Reductions over a 64-lane wave; every lane gets the result.  The order of the
-// additions is fixed, so results do not depend on anything but the inputs.
+// A value combined with the one 16 (32) lanes across, in both lanes: one vector instruction of gfx950
+// (v_permlane16_swap / v_permlane32_swap give both values in two registers) where an exchange through the LDS crossbar
+// (what __shfl_xor compiles to) waits in line behind the tiles' reads.  Maximum and sum are symmetric, so both lanes
+// get the same bits.
+__device__ __forceinline__ float max_across_16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_across_32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_across_16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_across_32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// The value of another lane of the same row of 16, by a pattern that is part of the instruction (DPP): lane ^ 1,
+// lane ^ 2, 7 - lane within a half row, 15 - lane within the row.
+template <int PATTERN>
+__device__ __forceinline__ float lane_pattern(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), PATTERN, 0xf, 0xf, true));
+}
+constexpr int LANE_XOR_1 = 0xB1, LANE_XOR_2 = 0x4E, HALF_ROW_MIRROR = 0x141, ROW_MIRROR = 0x140;
+
+// Reductions over a 64-lane wave; every lane gets the result, the same bits in every lane (each step combines two
+// values that are the same on both sides).  The order of the additions is fixed, so results do not depend on
+// anything but the inputs.  Pairs, quads, half rows and rows of 16 by lane patterns, then the rows by the lane
+// swaps above: six vector instructions, where six exchanges through the LDS crossbar made a chain of their latencies.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+  v += lane_pattern<LANE_XOR_1>(v);
+  v += lane_pattern<LANE_XOR_2>(v);
+  v += lane_pattern<HALF_ROW_MIRROR>(v);
+  v += lane_pattern<ROW_MIRROR>(v);
+  return sum_across_32(sum_across_16(v));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
+  v = fmaxf(v, lane_pattern<LANE_XOR_1>(v));
+  v = fmaxf(v, lane_pattern<LANE_XOR_2>(v));
+  v = fmaxf(v, lane_pattern<HALF_ROW_MIRROR>(v));
+  v = fmaxf(v, lane_pattern<ROW_MIRROR>(v));
+  return max_across_32(max_across_16(v));
 }
 
 // Sum over a workgroup of up to 1024 threads (blockDim.x a multiple of 64);
