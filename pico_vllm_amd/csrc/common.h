@@ -98,6 +98,35 @@ __device__ __forceinline__ float wave_max(float v) {
   return max_across_32(max_across_16(v));
 }
 
+// The first maximum of a wave (the lowest index among equal values); every lane gets it.  The same steps as above.
+__device__ __forceinline__ void keep_first_max(float& mx, int& mi, float ov, int oi) {
+  if (ov > mx || (ov == mx && oi < mi)) { mx = ov; mi = oi; }
+}
+template <int PATTERN>
+__device__ __forceinline__ void first_max_step(float& mx, int& mi) {
+  const float ov = lane_pattern<PATTERN>(mx);
+  const int oi = (int)__builtin_amdgcn_update_dpp(0u, (uint32_t)mi, PATTERN, 0xf, 0xf, true);
+  keep_first_max(mx, mi, ov, oi);
+}
+__device__ __forceinline__ void wave_first_max(float& mx, int& mi) {
+  first_max_step<LANE_XOR_1>(mx, mi);
+  first_max_step<LANE_XOR_2>(mx, mi);
+  first_max_step<HALF_ROW_MIRROR>(mx, mi);
+  first_max_step<ROW_MIRROR>(mx, mi);
+  {
+    const auto v = __builtin_amdgcn_permlane16_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+    const auto i = __builtin_amdgcn_permlane16_swap((uint32_t)mi, (uint32_t)mi, false, false);
+    mx = __uint_as_float(v[0]); mi = (int)i[0];
+    keep_first_max(mx, mi, __uint_as_float(v[1]), (int)i[1]);
+  }
+  {
+    const auto v = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+    const auto i = __builtin_amdgcn_permlane32_swap((uint32_t)mi, (uint32_t)mi, false, false);
+    mx = __uint_as_float(v[0]); mi = (int)i[0];
+    keep_first_max(mx, mi, __uint_as_float(v[1]), (int)i[1]);
+  }
+}
+
 // Sum over a workgroup of up to 1024 threads (blockDim.x a multiple of 64);
 // scratch holds 16 floats of LDS.  All threads get the result.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

@@ -297,12 +297,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
   // the row's first maximum: what a greedy row gives, and what a draw falls back on
   float mx = lane < SAMPLE_CHUNKS ? part_val[row * SAMPLE_CHUNKS + lane] : -INFINITY;
   int mi = lane < SAMPLE_CHUNKS ? part_idx[row * SAMPLE_CHUNKS + lane] : 0x7fffffff;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const float ov = __shfl_xor(mx, off, 64);
-    const int oi = __shfl_xor(mi, off, 64);
-    if (ov > mx || (ov == mx && oi < mi)) { mx = ov; mi = oi; }
-  }
+  wave_first_max(mx, mi);
   const float temp = temperature[row];
   if (!(temp > 0.f)) {
     if (tid == 0) out[row] = mi;
@@ -395,10 +390,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
 // one compute unit takes data in (19 us for 151,936 logits); ARGMAX_CHUNKS workgroups per row find the
 // first maximum of a chunk each, a second launch picks among them (the lowest index on a tie, as above).
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ void keep_first_max(float& mx, int& mi, float ov, int oi) {
-  if (ov > mx || (ov == mx && oi < mi)) { mx = ov; mi = oi; }
-}
-
 __global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits, int ld, int V,
                                                           float* __restrict__ part_val, int* __restrict__ part_idx) {
   __shared__ float vals[4];
@@ -421,8 +412,7 @@ __global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restric
     for (int j = 0; j < 4; j++)
       if (v[j] > mx) { mx = v[j]; mi = i0 + j * 256; }
   }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) keep_first_max(mx, mi, __shfl_xor(mx, off, 64), __shfl_xor(mi, off, 64));
+  wave_first_max(mx, mi);
   if ((tid & 63) == 0) { vals[tid >> 6] = mx; idxs[tid >> 6] = mi; }
   __syncthreads();
   if (tid == 0) {
@@ -437,8 +427,7 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
   const int row = blockIdx.x, lane = threadIdx.x;
   float mx = lane < ARGMAX_CHUNKS ? part_val[row * ARGMAX_CHUNKS + lane] : -INFINITY;
   int mi = lane < ARGMAX_CHUNKS ? part_idx[row * ARGMAX_CHUNKS + lane] : 0x7fffffff;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) keep_first_max(mx, mi, __shfl_xor(mx, off, 64), __shfl_xor(mi, off, 64));
+  wave_first_max(mx, mi);
   if (lane == 0) out[row] = mi;
 }
 
