@@ -359,6 +359,25 @@ def test_sampling_at_the_real_vocabulary_row_by_row(K):
         K.sample(dev, temps.to(DEV), top_ps.to(DEV), us.to(DEV), work=K.sample_workspace(R - 1, DEV))
 
 
+def test_sampling_at_the_edges_of_its_options(K):
+    # a nucleus so small that only the likeliest token fits, a temperature so low that it holds all the mass, one so high
+    # that the distribution is flat, and a vocabulary smaller than the number of chunks a row is read in
+    g = torch.Generator().manual_seed(3)
+    for V in (5, 31, 33, 1000, 151936):
+        logits = torch.randn(6, V, generator=g) * 2
+        best = logits.argmax(1).tolist()
+        temps = torch.tensor([1.0, 1e-4, 1.0, 50.0, 50.0, 0.3])
+        top_ps = torch.tensor([1e-6, 1.0, 1e-6, 1.0, 0.999999, 1e-3])
+        for u in (0.0, 0.37, 0.999999):
+            us = torch.full((6,), u)
+            out = K.sample(logits.to(DEV), temps.to(DEV), top_ps.to(DEV), us.to(DEV)).tolist()
+            assert [out[0], out[1], out[2], out[5]] == [best[0], best[1], best[2], best[5]], (V, u, out, best)
+            for r in (3, 4):                                   # nearly flat: the token at which the CDF passes u
+                p = P.top_p_probs(logits[r].double(), 50.0, float(top_ps[r]))
+                want = P.inverse_cdf(p, u)
+                assert 0 <= out[r] < V and (out[r] == want or abs(float(torch.cumsum(p, 0)[min(out[r], want)]) - u) < 1e-4), (V, u, r, out[r], want)
+
+
 def test_sampling_top_p(K):
     probs = torch.tensor([[0.05, 0.5, 0.15, 0.3]])
     logits = torch.log(probs)
