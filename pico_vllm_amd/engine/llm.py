@@ -118,6 +118,11 @@ class LLMEngine:
             done = self._resolve(prev)
             if plan is not None:
                 plan.seqs = [s for s in plan.seqs if s.request.status is RequestStatus.RUNNING]
+                if not plan.seqs:
+                    # everything it planned has ended with the tokens just read (a stop token cannot be foreseen), and
+                    # what it preempted waits: plan anew
+                    self.stats["preemptions"] += len(plan.preempted)
+                    plan = None
         if plan is None:
             with self.timers.phase("schedule"):
                 plan = self.scheduler.schedule()

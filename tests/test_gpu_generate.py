@@ -386,3 +386,32 @@ def test_the_sizes_that_reports_are_made_of_and_the_measured_peaks():
         sm.launch(logits[:2], [0.0], [1.0, 1.0], [1, 2], [0, 0])
     with pytest.raises(ValueError, match="3 rows to sample, the sampler was made for 2"):
         sm.launch(logits, [0.0] * 3, [1.0] * 3, [1, 2, 3], [0] * 3)
+
+
+def test_a_stop_token_that_arrives_while_the_other_request_is_being_preempted():
+    # With a step in flight the next step is planned before the tokens of the one in flight are read.  Two requests, so
+    # few pages that the younger one is preempted when both want their third page; the older one's stop token is placed
+    # at every position in turn, so that at one of them it arrives in the very step whose plan preempted the younger:
+    # all that the plan held has then ended, and the engine has to plan anew instead of finding nothing to run.
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for("A", [20, 20], seed=11)
+    free = SamplingParams(max_new_tokens=40, temperature=0.0, ignore_eos=True)
+    roomy = dict(num_gpu_blocks=16, max_num_seqs=2, max_num_batched_tokens=64, max_seq_len=64, use_cuda_graph=False)
+    ref = [o.token_ids for o in llm("A", "float32", **roomy).generate(prompts, free)]
+    assert len(ref[0]) == 40 and len(ref[1]) == 40
+    tight = dict(roomy, num_gpu_blocks=5)
+    preempted = 0
+    for k in range(40):
+        stop = ref[0][k]
+        first = ref[0].index(stop)                              # the request ends where the token first appears
+        sps = [SamplingParams(max_new_tokens=40, temperature=0.0, ignore_eos=True, stop_token_ids=[stop]), free]
+        for pipe in (True, False):
+            eng = llm("A", "float32", pipeline_decode=pipe, **tight)
+            outs = eng.generate(prompts, sps)
+            assert [o.token_ids for o in outs] == [ref[0][:first + 1], ref[1]], (k, pipe)
+            assert outs[0].finish_reason == ("stop" if first < 39 or stop == ref[0][39] else "length") and outs[1].finish_reason == "length"
+            preempted += eng.engine.stats["preemptions"]
+            m = eng.engine.runner.manager
+            m.check()
+            assert all(g.pool.num_free == g.pool.num_pages for g in m.groups)
+    assert preempted > 0
