@@ -415,3 +415,38 @@ def test_a_stop_token_that_arrives_while_the_other_request_is_being_preempted():
             m.check()
             assert all(g.pool.num_free == g.pool.num_pages for g in m.groups)
     assert preempted > 0
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_drawn_serving_scenarios_give_the_same_tokens_in_every_mode(seed):
+    # requests of drawn lengths and options (greedy and sampled, stop tokens, the end-of-sequence token honoured or not)
+    # served with and without recorded steps, with and without the step in flight, in a roomy and in a tight pool that
+    # forces preemption: in float32 the same tokens and finish reasons in all eight, no page lost, nothing left behind
+    import random
+    from pico_vllm_amd import LLM, SamplingParams
+    rng = random.Random(1000 + seed)
+    for _ in range(8):
+        name = rng.choice(["A", "B", "C", "D", "E"])
+        V, page = CONFIGS[name]["vocab_size"], PAGE_SIZE[name]
+        n = rng.randint(2, 7)
+        prompts = [[rng.randrange(V - 1) for _ in range(rng.choice([1, 2, 3, 7, 15, 16, 17, 33, 64, 65, 100]))] for _ in range(n)]
+        sps = [SamplingParams(max_new_tokens=rng.choice([1, 2, 5, 17, 40]), temperature=rng.choice([0.0, 0.0, 0.8]), top_p=rng.choice([1.0, 0.9]),
+                              seed=rng.randrange(1000), ignore_eos=rng.random() < 0.7,
+                              stop_token_ids=[rng.randrange(V)] if rng.random() < 0.3 else []) for _ in range(n)]
+        longest = max(len(p) + sp.max_new_tokens for p, sp in zip(prompts, sps))
+        need = -(-longest // page)
+        max_seqs, budget = rng.randint(2, 5), rng.choice([16, 33, 64, 128])
+        tight = need + rng.randint(0, need)
+        ref = None
+        for graphs in (False, True):
+            for pipe in (False, True):
+                for pages in (need * max_seqs + 4, tight):
+                    eng = LLM(model=model_dir(name), dtype="float32", block_size=page, num_gpu_blocks=pages, max_seq_len=max(longest, 16),
+                              max_num_seqs=max_seqs, max_num_batched_tokens=budget, use_cuda_graph=graphs, pipeline_decode=pipe,
+                              max_batch_size=4)
+                    got = [(o.token_ids, o.finish_reason) for o in eng.generate(prompts, sps)]
+                    m = eng.engine.runner.manager
+                    m.check()
+                    assert all(g.pool.num_free == g.pool.num_pages for g in m.groups) and not eng.engine.requests
+                    ref = ref or got
+                    assert got == ref, (name, graphs, pipe, pages, [len(p) for p in prompts])
