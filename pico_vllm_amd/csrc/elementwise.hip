@@ -301,6 +301,12 @@ extern "C" int pico_rope_table(const int* positions, const float* inv_freq, floa
   return 0;
 }
 
+// a cos - b sin and b cos + a sin with the roundings spelled out (one product rounded, then one fused multiply-add), so
+// that the kernel for few tokens and the one with 16-byte accesses give the same bits: left to the compiler, which of
+// the two products is fused differs from kernel to kernel
+__device__ __forceinline__ float rotate_lo(float a, float b, float c, float s) { return __fmaf_rn(a, c, -__fmul_rn(b, s)); }
+__device__ __forceinline__ float rotate_hi(float a, float b, float c, float s) { return __fmaf_rn(b, c, __fmul_rn(a, s)); }
+
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, const float2* __restrict__ cos_sin,
                                   const int* __restrict__ slots,
@@ -326,8 +332,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float2* __restrict_
     }
     const float c = cs[j].x, s = cs[j].y;
     const float a = load_f32(x + j), b = load_f32(x + j + half);
-    store_f32(o + j, a * c - b * s);
-    store_f32(o + j + half, b * c + a * s);
+    store_f32(o + j, rotate_lo(a, b, c, s));
+    store_f32(o + j + half, rotate_hi(a, b, c, s));
   }
   if (!store) return;
   for (int u = threadIdx.x; u < nkv * (d - rot); u += blockDim.x) {      // what is not rotated of k
@@ -386,8 +392,8 @@ __global__ __launch_bounds__(256) void rope_store_bf16x8_kernel(bf16_t* __restri
         const float4 c2 = cs[e];
         const float a0 = __uint_as_float(lo[e] << 16), a1 = __uint_as_float(lo[e] & 0xffff0000u);
         const float b0 = __uint_as_float(hi[e] << 16), b1 = __uint_as_float(hi[e] & 0xffff0000u);
-        olo[e] = pack2_bf16(a0 * c2.x - b0 * c2.y, a1 * c2.z - b1 * c2.w);
-        ohi[e] = pack2_bf16(b0 * c2.x + a0 * c2.y, b1 * c2.z + a1 * c2.w);
+        olo[e] = pack2_bf16(rotate_lo(a0, b0, c2.x, c2.y), rotate_lo(a1, b1, c2.z, c2.w));
+        ohi[e] = pack2_bf16(rotate_hi(a0, b0, c2.x, c2.y), rotate_hi(a1, b1, c2.z, c2.w));
       }
       *reinterpret_cast<rs_u32x4*>(o + j) = olo;
       *reinterpret_cast<rs_u32x4*>(o + j + half) = ohi;

@@ -212,6 +212,7 @@ def build_context(seqs: List[SeqStep], manager: CacheManager, buf: BatchBuffers,
         slot_mapping=[d[(3 + g) * buf.max_tokens:(3 + g) * buf.max_tokens + T] for g in range(G)],
         act_dtype=act_dtype,
         max_new_tokens=max(lens), max_context=max_ctx, all_decode=max(lens) == 1 and pad_tokens_to is None,
-        host={"cu_seqlens": h_cu.copy(), "context_lens": h_ctx.copy()},
+        # (filler: how many sequences at the end are padding of a recorded step, whose size says nothing about the work)
+        host={"cu_seqlens": h_cu.copy(), "context_lens": h_ctx.copy(), "filler": int(pad_tokens_to is not None)},
     )
     return ctx

@@ -195,11 +195,14 @@ class FastAttention:
             if "cu_seqlens" in ctx.host and "context_lens" in ctx.host:
                 cu = ctx.host["cu_seqlens"]
                 lens = cu[1:B + 1] - cu[:B]
-                while lead < B and lens[lead] == 1:
+                # the filler behind a recorded step's portion does not count: the step gets the shapes it would get
+                # unrecorded, and so the same bits
+                real = B - int(ctx.host.get("filler", 0))
+                while lead < real and lens[lead] == 1:
                     lead += 1
-                if lead < B:
-                    teams = self.prefill_teams(lens[lead:], ctx.host["context_lens"][lead:B])
-                    cut = self.prefill_chunks(lens[lead:], ctx.host["context_lens"][lead:B])
+                if lead < real:
+                    teams = self.prefill_teams(lens[lead:real], ctx.host["context_lens"][lead:real])
+                    cut = self.prefill_chunks(lens[lead:real], ctx.host["context_lens"][lead:real])
                     if cut is not None:
                         teams, chunk_len, max_chunks = cut
             ctx.shared[key] = (int(teams), int(lead), int(chunk_len), int(max_chunks))

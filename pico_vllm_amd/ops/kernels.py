@@ -225,10 +225,15 @@ MAX_HEAD_DIM = 256          # the largest head size any attention kernel takes
 SKINNY_ROWS, SKINNY_MID_ROWS, SKINNY_MID_WEIGHT = 64, 256, 1 << 22
 
 
+def skinny_rows(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether a step of this many rows is one the weight-streaming kernel is meant for."""
+    return a.dim() == 2 and (a.shape[0] <= SKINNY_ROWS or (a.shape[0] <= SKINNY_MID_ROWS and w.numel() <= SKINNY_MID_WEIGHT))
+
+
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the weight-streaming kernel takes these operands (few rows, 16-byte aligned rows)."""
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2
-            and (a.shape[0] <= SKINNY_ROWS or (a.shape[0] <= SKINNY_MID_ROWS and w.numel() <= SKINNY_MID_WEIGHT))
+            and skinny_rows(a, w)
             and a.shape[1] % 8 == 0 and a.stride(1) == 1 and w.stride(1) == 1
             and (a.stride(0) % 8 == 0 or a.shape[0] == 1) and w.stride(0) % 8 == 0
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)

@@ -1,8 +1,8 @@
 """y = x W^T (+ b) with W stored [out, in] as in the checkpoint.
 
 bfloat16 weights: with up to 64 rows of activations (decode, small mixed
-steps) the weight-streaming matrix-core kernel of this package, with bias,
-SwiGLU or float32 output as its epilogue; with more rows the library GEMM
+steps; up to 256 for small matrices) the weight-streaming matrix-core kernel of this package, with bias,
+SwiGLU or float32 output as its epilogue (for shapes it refuses, this package's plain matrix-core product); with more rows the library GEMM
 (hipBLASLt through torch), as the reference uses the library for every
 projection (pico_vllm/model.py:200,225,316,318).  float32 weights: this package's plain-FMA kernel, never a library
 call, so the 32-bit engine has no reduced-precision matrix mode anywhere; if
@@ -92,6 +92,11 @@ class Linear:
             return kernels.gemm_skinny(x, self.weight, self.bias_f32, epi)
         if out_dtype == torch.float32:
             return kernels.gemm_bf16(x, self.weight, self.bias_f32, torch.float32)
+        if kernels.skinny_rows(x, self.weight):
+            # few rows of a shape that the weight-streaming kernel refuses (an inner size that is no multiple of 8):
+            # this package's plain matrix-core product, in which a row's result does not depend on the other rows of
+            # the step, as it does not in the weight-streaming kernel; the library's may
+            return kernels.gemm_bf16(x, self.weight, self.bias_f32, torch.bfloat16)
         _library_tuning(x.shape[0])
         if self.bias is not None:
             return torch.addmm(self.bias, x, self.weight.t())

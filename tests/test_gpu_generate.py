@@ -450,3 +450,41 @@ def test_drawn_serving_scenarios_give_the_same_tokens_in_every_mode(seed):
                     assert all(g.pool.num_free == g.pool.num_pages for g in m.groups) and not eng.engine.requests
                     ref = ref or got
                     assert got == ref, (name, graphs, pipe, pages, [len(p) for p in prompts])
+
+
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_a_recorded_prompt_step_gives_the_bits_of_the_step_unrecorded_and_unpadded(name):
+    # in bfloat16 too: the filler and the empty rows of a recorded step take no part in what the kernels choose (the
+    # attention's workgroup shapes, the splits of the single tokens' contexts), and with few rows every product is a
+    # kernel of this package in which a row does not depend on the others (A and D have inner sizes that are no
+    # multiple of 8: the plain matrix-core product instead of the weight-streaming one)
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.model import load_model
+    model = load_model(model_dir(name), "bfloat16", "cuda:0")
+    V, page = CONFIGS[name]["vocab_size"], PAGE_SIZE[name]
+    rec = ModelRunner(model, page, 64, 4, 64, 256, use_graph=True, max_graph_batch=4)
+    raw = ModelRunner(model, page, 64, 4, 64, 256, use_graph=False)
+    g = torch.Generator().manual_seed(4)
+    text = {r: torch.randint(0, V, (200,), generator=g).tolist() for r in "abcd"}
+    at = dict.fromkeys(text, 0)
+
+    def both(parts):
+        outs = []
+        for r in (rec, raw):
+            seqs = []
+            for rid, n in parts:
+                if rid not in r.manager.requests:
+                    assert r.manager.add_request(rid)
+                assert r.manager.grow(rid, at[rid] + n)
+                seqs.append(SeqStep(rid, text[rid][at[rid]:at[rid] + n], [n - 1]))
+            outs.append(r.step(seqs).clone())
+            r.advance(seqs)
+        for rid, n in parts:
+            at[rid] += n
+        assert torch.equal(outs[0], outs[1]), parts
+
+    for parts in ([("a", 15)], [("b", 40)], [("a", 1), ("b", 1), ("c", 23)], [("a", 1), ("c", 2)], [("a", 1), ("b", 1), ("c", 1), ("d", 50)],
+                  [("b", 1), ("d", 7)], [("a", 1), ("b", 1), ("c", 1), ("d", 1)], [("c", 33)], [("a", 1), ("b", 1), ("d", 1), ("c", 60)]):
+        both(parts)
+    assert {k[:2] for k in rec._prompt_graphs} >= {(0, 16), (2, 32), (1, 16), (4, 64)} and rec._graphs and not raw._prompt_graphs

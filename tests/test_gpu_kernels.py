@@ -254,6 +254,29 @@ def test_attention_window_edge(K, dtype, window):
     close(out, want, dtype)
 
 
+@pytest.mark.parametrize("nq,nkv,d,rot", [(8, 1, 16, 16), (12, 2, 128, 128), (2, 2, 64, 32)])
+def test_rotation_gives_a_token_the_same_bits_whatever_stands_beside_it(K, nq, nkv, d, rot):
+    # seven tokens alone take the kernel for few tokens, the same seven among twenty the one with 16-byte accesses: the
+    # same rotated queries and the same keys and values in the cache, bit for bit (a step padded for a recorded graph
+    # must not differ from the step unpadded)
+    g = torch.Generator().manual_seed(d)
+    T, n, Pg = 20, 7, 16
+    qkv = (torch.randn(T, (nq + 2 * nkv) * d, generator=g) * 2).bfloat16()
+    pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(4 * Pg, generator=g)[:T].to(torch.int32)
+    inv = (1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    got = []
+    for rows in (T, n):
+        x = qkv[:rows].clone().to(DEV)
+        kc = torch.zeros(4, nkv, Pg, d, dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros(4, nkv, d, Pg, dtype=torch.bfloat16, device=DEV)
+        K.rope_kv_store(x, K.rope_table(pos[:rows].to(DEV), inv), slots[:rows].to(DEV), kc, vc, nq, nkv, d, rot)
+        got.append((x[:n].cpu(), [(kc[int(s) // Pg, :, int(s) % Pg].cpu(), vc[int(s) // Pg, :, :, int(s) % Pg].cpu()) for s in slots[:n]]))
+    assert torch.equal(got[0][0], got[1][0])
+    for (k1, v1), (k2, v2) in zip(got[0][1], got[1][1]):
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
 def test_sampling_greedy_and_ties(K):
     logits = torch.randn(5, 1000)
     logits[1, 7] = logits[1, 900] = 50.0            # tie: the lower index wins
