@@ -55,3 +55,24 @@ def test_the_splits_of_a_decode_step(num_seqs, context, want):
 
 def test_a_window_bounds_the_splits():
     assert plan(12, window=100).num_splits(1, 32768) == 3                # 131 keys at most
+
+
+def test_the_filler_of_a_recorded_step_takes_no_part_in_the_plan():
+    # a recorded step has a sequence of filler behind its portion (and single tokens, some of them empty rows, in front):
+    # the plan is that of the real sequences, so that the step gets the shapes it would get unrecorded
+    import numpy as np
+    from types import SimpleNamespace
+    fa = plan(12)
+
+    def step(lens, contexts, filler):
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        return SimpleNamespace(num_seqs=len(lens), shared={},
+                               host={"cu_seqlens": cu, "context_lens": np.asarray(contexts, dtype=np.int32), "filler": filler})
+
+    for lens, contexts in (([2048], [16384]), ([300], [300]), ([1, 1, 1, 700], [50, 900, 0, 5000]), ([1, 1, 100], [4000, 4000, 2100])):
+        alone = fa.plan(step(lens, contexts, 0))
+        for fill in (0, 1, 13, 1900):
+            assert fa.plan(step(lens + [fill], contexts + [fill], 1)) == alone, (lens, fill)
+        assert alone[1] == sum(n == 1 for n in lens)                 # the single tokens that stand first
+    # counted as a sequence, a long filler would change the shapes: that is what leaving it out avoids
+    assert fa.plan(step([2048, 2048], [16384, 2048], 0)) != fa.plan(step([2048, 2048], [16384, 2048], 1))
