@@ -339,6 +339,35 @@ def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20, chunk_len=0):
     return {"us": round(us, 1), "shape": shape, "tflops": round(flops / us / 1e6, 1), "frac": round(flops / (us * 1e-6) / MFMA_PEAK["bfloat16"], 4)}
 
 
+def sampling_point(cfg, rows, top_p, reps=50):
+    """The sampling call alone on ``rows`` rows of float32 logits of the shape's vocabulary: greedy, temperature 0.8,
+    and temperature 0.8 with ``top_p``; microseconds a call."""
+    import torch
+    from pico_vllm_amd.ops import kernels
+    dev, V = "cuda", cfg["vocab_size"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.randn(rows, V, device=dev, generator=g) * 3.0
+    u = torch.rand(rows, device=dev, generator=g)
+    out = torch.empty(rows, dtype=torch.int32, device=dev)
+    work = kernels.sample_workspace(rows, dev)
+    res = {}
+    for name, temp, p in (("greedy", 0.0, 1.0), ("temperature", 0.8, 1.0), ("top_p", 0.8, top_p)):
+        t = torch.full((rows,), temp, device=dev)
+        pp = torch.full((rows,), p, device=dev)
+        run = lambda: kernels.sample(logits, t, pp, u, out=out, work=work, top_p_rows=temp > 0 and p < 1)
+        for _ in range(5):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name] = round(e0.elapsed_time(e1) / reps * 1e3, 1)
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -367,6 +396,8 @@ def main() -> int:
     ap.add_argument("--max-new", type=int, default=256, help="new tokens per request of the serve workload")
     ap.add_argument("--attention", metavar="SEQS,NEW,PREFIX[,SHAPE[,CHUNK]]", default=None,
                     help="time only the prefill attention kernel on SEQS portions of NEW tokens after PREFIX cached ones")
+    ap.add_argument("--sampling", metavar="ROWS[,TOP_P]", default=None,
+                    help="time only the sampling call on ROWS rows of the shape's vocabulary (greedy, temperature, top-p)")
     a = ap.parse_args()
     global CONFIG, CONTEXT
     shape_name, full = SHAPES[a.shape]
@@ -395,6 +426,17 @@ def main() -> int:
         print(json.dumps({"metric": "prefill attention kernel", "unit": "us", "value": r["us"], "workgroup_shape": r["shape"],
                           "tflops": r["tflops"], "frac_of_bf16_peak": r["frac"], "sequences": nums[0], "new_tokens": nums[1],
                           "prefix": nums[2], "heads": CONFIG["num_attention_heads"], "kv_heads": CONFIG["num_key_value_heads"]}))
+        return 0
+    if a.sampling:
+        parts = a.sampling.split(",")
+        rows, top_p = int(parts[0]), float(parts[1]) if len(parts) > 1 else 0.9
+        if not (1 <= rows <= 1024 and 0 < top_p <= 1):
+            print("bench.py: --sampling takes 1..1024 rows and a top-p in (0, 1]")
+            return 2
+        r = sampling_point(CONFIG, rows, top_p)
+        print(json.dumps({"metric": "sampling call", "unit": "us", "value": r["top_p"], "greedy": r["greedy"],
+                          "temperature": r["temperature"], "top_p": r["top_p"], "rows": rows, "vocab_size": CONFIG["vocab_size"],
+                          "p": top_p}))
         return 0
     if a.write_model:
         write_random_model(a.write_model, CONFIG, seed=0)

@@ -36,6 +36,7 @@
 #define SAMPLE_K 63                 // thresholds a round
 #define SAMPLE_CLASSES (SAMPLE_K + 1)
 #define SAMPLE_ROUNDS 5             // ceil(2^30 / 64^5) = 1
+#define SAMPLE_PIECE 32             // the elements of the chosen chunk that a thread of the last launch holds in registers
 #define SAMPLE_ONE 0x3f800000u      // the bit pattern of 1.0f: no e is above it
 
 struct SampleChunk {
@@ -199,6 +200,26 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
   return v;
 }
 
+// The terms e = exp((x - max) / t) of the elements begin + thread, begin + thread + SAMPLE_THREADS, ... of a chunk, in
+// that order, eight loads in flight a thread: one load at a time, each used at once, is a chain of memory latencies
+// (6 us for the 19 elements a thread has of a chunk of 151,936 logits).
+template <class Use>
+__device__ __forceinline__ void sample_each_term(const float* __restrict__ x, int begin, int end, float mx, float inv_t, Use use) {
+  for (int i0 = begin + (int)threadIdx.x; i0 < end; i0 += 8 * SAMPLE_THREADS) {
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const int i = i0 + k * SAMPLE_THREADS;
+      v[k] = i < end ? x[i] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const int i = i0 + k * SAMPLE_THREADS;
+      if (i < end) use(i, __expf((v[k] - mx) * inv_t));
+    }
+  }
+}
+
 // per chunk: the sum of e > t* (double) and the number of e == t*; the row's t* and how many ties it keeps
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_chunk_sums_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
@@ -227,11 +248,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_chunk_sums_kernel(
   const SampleChunk ch = sample_chunk(V, c);
   double s = 0.0;
   int n = 0;
-  for (int i = ch.begin + tid; i < ch.end; i += SAMPLE_THREADS) {
-    const float e = __expf((x[i] - mx) * inv_t);
+  sample_each_term(x, ch.begin, ch.end, mx, inv_t, [&](int, float e) {
     if (e > thr) s += (double)e;
     n += e == thr;
-  }
+  });
   s = wave_sum_f64(s);
   n = wave_sum_i32(n);
   if ((tid & 63) == 0) { ws[tid >> 6] = s; wn[tid >> 6] = n; }
@@ -289,7 +309,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
     int* __restrict__ out) {
   __shared__ double wave_tot[SAMPLE_THREADS / 64];
   __shared__ int wave_cnt[SAMPLE_THREADS / 64];
-  __shared__ int chosen_chunk, chosen_ties_before, chosen_thread, last_thread;
+  __shared__ int chosen_chunk, chosen_ties_before;
+  __shared__ int wave_first[SAMPLE_THREADS / 64], wave_last[SAMPLE_THREADS / 64];
   __shared__ int chunk_n[SAMPLE_CHUNKS];
   __shared__ double chunk_s[SAMPLE_CHUNKS];
   __shared__ double chosen_before, chosen_target;
@@ -298,7 +319,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
   float mx = lane < SAMPLE_CHUNKS ? part_val[row * SAMPLE_CHUNKS + lane] : -INFINITY;
   int mi = lane < SAMPLE_CHUNKS ? part_idx[row * SAMPLE_CHUNKS + lane] : 0x7fffffff;
   wave_first_max(mx, mi);
-  const float temp = temperature[row];
+  const float temp = temperature[row], u_row = u[row];    // (asked for here: where it is used, one thread would wait for it)
   if (!(temp > 0.f)) {
     if (tid == 0) out[row] = mi;
     return;
@@ -323,7 +344,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
       total += kept[c];
       ties += n;
     }
-    const double target = (double)u[row] * total;
+    const double target = (double)u_row * total;
     double run = 0.0, before_last = 0.0;
     int c = -1, last_nonzero = 0;
     for (int i = 0; i < SAMPLE_CHUNKS; i++) {
@@ -336,36 +357,69 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
     chosen_before = run;
     chosen_target = target;
     chosen_ties_before = before[c];
-    chosen_thread = 0x7fffffff;
-    last_thread = -1;
   }
   __syncthreads();
   const SampleChunk ch = sample_chunk(V, chosen_chunk);
   const float inv_t = 1.0f / temp;
   const float* x = logits + (size_t)row * ld;
-  // thread t owns a contiguous piece of the chunk
+  // A thread owns a contiguous piece of the chunk and goes through it three times.  One element after the other from
+  // memory, each pass is a chain of latencies (2 to 2.6 us each for the 19 elements a thread has of a chunk of
+  // 151,936 logits): a piece of up to SAMPLE_PIECE elements (vocabularies up to 262,144) is asked for at once and
+  // its terms wait in registers.
+  auto term = [&](int i) { return __expf((x[i] - mx) * inv_t); };
   const int piece = (ch.end - ch.begin + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
   const int b = min(ch.end, ch.begin + tid * piece), e_ = min(ch.end, b + piece);
+  const bool held = piece <= SAMPLE_PIECE;                                 // the same for all threads
+  float mine[SAMPLE_PIECE];
+  if (held) {
+#pragma unroll
+    for (int k = 0; k < SAMPLE_PIECE; k++) mine[k] = b + k < e_ ? x[b + k] : 0.f;
+#pragma unroll
+    for (int k = 0; k < SAMPLE_PIECE; k++) mine[k] = __expf((mine[k] - mx) * inv_t);
+  }
+  // use(i, e) for the elements of the piece in their order, until it returns false
+  auto each = [&](auto use) {
+    if (held) {
+#pragma unroll
+      for (int k = 0; k < SAMPLE_PIECE; k++) {
+        if (b + k >= e_ || !use(b + k, mine[k])) break;
+      }
+    } else {
+      for (int i = b; i < e_; i++)
+        if (!use(i, term(i))) break;
+    }
+  };
   int my_ties = 0;
-  for (int i = b; i < e_; i++) my_ties += __expf((x[i] - mx) * inv_t) == thr;
+  each([&](int, float e) { my_ties += e == thr; return true; });
   const int ties_before = chosen_ties_before + block_prefix_i32(my_ties, wave_cnt);
   double s = 0.0;
   {
     int tie = ties_before;
-    for (int i = b; i < e_; i++) {
-      const float e = __expf((x[i] - mx) * inv_t);
+    each([&](int, float e) {
       if (e > thr || (e == thr && tie++ < ties_kept)) s += (double)e;
-    }
+      return true;
+    });
   }
   double chunk_total;
   const double before = chosen_before + block_prefix_f64(s, wave_tot, chunk_total);
   const double target = chosen_target;
-  if (s > 0.0) {
-    atomicMax(&last_thread, tid);
-    if (before + s > target) atomicMin(&chosen_thread, tid);
+  // the first thread whose piece reaches the target, and the last that keeps anything (a vote in each wave, then
+  // the waves side by side: every thread asking for one word of LDS at once takes 4 us)
+  {
+    const unsigned long long keeps = __ballot(s > 0.0), reaches = __ballot(s > 0.0 && before + s > target);
+    if (lane == 0) {
+      wave_last[tid >> 6] = keeps ? (tid | 63) - __clzll(keeps) : -1;
+      wave_first[tid >> 6] = reaches ? tid + __ffsll(reaches) - 1 : 0x7fffffff;
+    }
   }
   __syncthreads();
-  const int who = chosen_thread != 0x7fffffff ? chosen_thread : last_thread;
+  int first = 0x7fffffff, last = -1;
+#pragma unroll
+  for (int w = 0; w < SAMPLE_THREADS / 64; w++) {
+    first = min(first, wave_first[w]);
+    last = max(last, wave_last[w]);
+  }
+  const int who = first != 0x7fffffff ? first : last;
   if (who < 0) {                              // nothing kept in the chunk (cannot be, but a token must come out)
     if (tid == 0) out[row] = mi;
     return;
@@ -373,14 +427,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
   if (tid == who) {
     double run = before;
     int pick = -1, last_kept = mi, tie = ties_before;
-    for (int i = b; i < e_; i++) {
-      const float e = __expf((x[i] - mx) * inv_t);
+    each([&](int i, float e) {
       if (e > thr || (e == thr && tie++ < ties_kept)) {
         last_kept = i;
         run += (double)e;
-        if (run > target) { pick = i; break; }
+        if (run > target) { pick = i; return false; }
       }
-    }
+      return true;
+    });
     out[row] = pick >= 0 ? pick : last_kept;
   }
 }

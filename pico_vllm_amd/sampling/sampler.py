@@ -1,8 +1,9 @@
 """Sampling one token per row of logits on the GPU.
 
 Strategy per row as in pico_vllm/sampler.py:40-88 (greedy / temperature /
-temperature with top-p), but in one kernel launch with per-row parameters
-instead of one torch call per group of equal parameters.  Randomness comes from
+temperature with top-p), but in one call with per-row parameters for the whole
+batch (a short chain of launches, several workgroups a row) instead of torch
+calls per group of equal parameters.  Randomness comes from
 a counter-based generator on the host: the uniform number of a draw depends
 only on (seed, index of the token in its request), so a request samples the
 same tokens whatever else is in the batch.
