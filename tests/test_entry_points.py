@@ -15,6 +15,13 @@ def test_the_benchmark_says_that_it_runs_on_one_gpu_and_exits_with_2():
         assert len(lines) == 1 and "one GPU" in lines[0] and f"--gpus {n}" in lines[0]
 
 
+def test_the_benchmark_refuses_sizes_of_its_single_points_that_it_does_not_run():
+    for args, said in ((["--sampling", "0"], "--sampling"), (["--sampling", "8,1.5"], "--sampling"),
+                       (["--prefill-only", "--prefill-tokens", "1"], "--prefill-tokens"), (["--layers", "99"], "--layers")):
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *args], capture_output=True, text=True, timeout=300, cwd=ROOT)
+        assert r.returncode == 2 and said in r.stdout, (args, r.returncode, r.stdout[-300:], r.stderr[-300:])
+
+
 def test_the_entry_file_has_build_and_smoke_and_the_replay_program_explains_itself():
     sys.path.insert(0, ROOT)
     try:
