@@ -117,9 +117,6 @@ class CacheManager:
         rc = self.requests[req]
         return [max(0, _cdiv(new_len, self.page_size) - len(t)) for t in rc.tables]
 
-    def can_grow(self, req: Hashable, new_len: int) -> bool:
-        return all(g.pool.ensure_free(n) for n, g in zip(self.pages_needed(req, new_len), self.groups))
-
     def grow(self, req: Hashable, new_len: int) -> bool:
         """Cover positions [0, new_len) in every group, or change nothing and return False."""
         need = self.pages_needed(req, new_len)

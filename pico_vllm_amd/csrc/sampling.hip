@@ -429,7 +429,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
     int pick = -1, last_kept = mi, tie = ties_before;
     each([&](int i, float e) {
       if (e > thr || (e == thr && tie++ < ties_kept)) {
-        last_kept = i;
+        if (e > 0.f) last_kept = i;           // a token whose probability underflowed to zero is never the fallback
         run += (double)e;
         if (run > target) { pick = i; return false; }
       }
@@ -499,7 +499,7 @@ extern "C" int pico_argmax(const float* logits, int ld, int R, int V, float* par
   return 0;
 }
 
-// work: pico_sample_workspace_words(R) 4-byte words, 8-byte aligned.  top_p_rows == 0: no row has top_p < 1 (every
+// work: pico_sample_workspace_words(R) 4-byte words, 16-byte aligned.  top_p_rows == 0: no row has top_p < 1 (every
 // row is treated so), and the rounds that look for the threshold are not launched.
 extern "C" long long pico_sample_workspace_words(int R) {
   return (long long)R * SAMPLE_CHUNKS * (2 + 1 + 1 + 2 * SAMPLE_CLASSES + 4 + 1 + 2);
@@ -511,7 +511,8 @@ extern "C" int pico_sample(const float* logits, int ld, int R, int V, const floa
   PICO_REQUIRE(R >= 0 && V > 0 && ld >= V, "pico_sample: bad sizes R=%d V=%d ld=%d", R, V, ld);
   PICO_REQUIRE(R <= 65535, "pico_sample: too many rows");
   if (R == 0) return 0;
-  PICO_REQUIRE(work != nullptr && (uintptr_t)work % 8 == 0, "pico_sample: the workspace is missing or misaligned");
+  // (the rounds read their state with 16-byte loads; every part of the workspace is a multiple of 16 bytes long)
+  PICO_REQUIRE(work != nullptr && (uintptr_t)work % 16 == 0, "pico_sample: the workspace is missing or not 16-byte aligned");
   const size_t n = (size_t)R * SAMPLE_CHUNKS;
   double* fin_s = (double*)work;
   float* part_val = (float*)(fin_s + n);

@@ -51,7 +51,10 @@ class LLMEngine:
         if args.max_seq_len > self.model.spec.max_position:
             raise ValueError(f"max_seq_len = {args.max_seq_len} exceeds the model's max_position_embeddings = "
                              f"{self.model.spec.max_position}")
-        linear.set_library_tuning(args.tune_library_gemm)
+        if args.tune_library_gemm:
+            # a mode of the whole process (torch's tuner): an engine only ever switches it on, so that building a
+            # second engine does not change what the first one runs
+            linear.set_library_tuning(True)
         num_pages = args.num_gpu_blocks
         if num_pages is None:
             num_pages = args.max_num_seqs * (-(-args.max_seq_len // args.block_size))
@@ -158,8 +161,7 @@ class LLMEngine:
             return False
         if [s.request for s in step.sampling] != self.scheduler.running:
             return False
-        return all(r.num_generated < r.params.max_new_tokens and r.total_len < self.args.max_seq_len
-                   for r in self.scheduler.running)
+        return all(not r.is_max_len_finished() and r.total_len < self.args.max_seq_len for r in self.scheduler.running)
 
     def _launch(self, plan, from_device: bool = False) -> "_Inflight":
         """Start the model step and the sampling of ``plan`` and advance what does not depend on the

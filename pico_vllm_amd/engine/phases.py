@@ -47,11 +47,17 @@ class _Phase:
             e1 = torch.cuda.Event(enable_timing=True)
             e1.record()
             o._pending.append((self.name, self.e0, e1))
+            if len(o._pending) >= PhaseTimers.COLLECT_EVERY:      # a long run that never asks for a report keeps few events
+                o._collect(wait=False)
+                if len(o._pending) >= 4 * PhaseTimers.COLLECT_EVERY:
+                    o._collect(wait=True)
         torch.cuda.nvtx.range_pop()
         return False
 
 
 class PhaseTimers:
+    COLLECT_EVERY = 64      # pending pairs of events beyond which finished ones are read (and all of them at four times that)
+
     def __init__(self, enabled: bool):
         self.enabled = enabled
         self.host_s: Dict[str, float] = {}

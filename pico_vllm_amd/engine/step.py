@@ -128,8 +128,11 @@ class ModelRunner:
         else:
             ctx = build_context(seqs, self.manager, self.buffers, self.model.dtype, self.model.spec.vocab_size)
             # the kernel choices of a recorded step for its single tokens (how their contexts are split over
-            # workgroups) hold for any context; a step that is not replayed makes the same ones, so that a request
-            # gets the same tokens with and without graphs
+            # workgroups) hold for any context; a step that is not replayed makes the same ones, so that a decoding
+            # request gets the same tokens with and without graphs.  (A recorded prompt step equals the same PADDED
+            # step unrecorded bit for bit; against the unpadded step that holds only while every product of the
+            # step is one of this package's, in which a row does not depend on the rows beside it: up to 64 rows.
+            # The library's products may round a row differently at another row count.)
             ctx.max_context = self.max_seq_len
             if device_tokens is not None:
                 ctx.token_ids[:len(seqs)].copy_(device_tokens[:len(seqs)])

@@ -496,7 +496,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     else:
         lib.pico_sample_workspace_words.restype = ctypes.c_longlong
         if work.dtype != torch.int32 or not work.is_contiguous() or work.numel() < int(lib.pico_sample_workspace_words(R)) \
-                or work.data_ptr() % 8:
+                or work.data_ptr() % 16:
             raise KernelError("sample: the workspace must come from sample_workspace for at least as many rows")
     _check(lib, lib.pico_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature),
                                 _ptr(top_p), _ptr(u), _ptr(out), _ptr(work), int(bool(top_p_rows)), _stream()))

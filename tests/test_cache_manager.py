@@ -122,7 +122,7 @@ def test_a_holder_of_spare_pages_is_asked_before_an_allocation_is_refused():
     m.add_request("c"); assert m.grow("c", 16) and asked == [1]         # one page short: the keeper gives its oldest
     assert kept == pages[1:2] and m.block_table("c") == [pages[0]]
     m.check([{p: 1 for p in kept}])
-    assert not m.can_grow("c", 48) and kept == []                       # asked again, gave its last, still short
+    assert not m.grow("c", 48) and kept == []                           # asked again, gave its last, still short: nothing taken
     assert m.grow("c", 32)
     m.check()
     assert not m.grow("b", 48) and asked[-1] == 1                       # nothing left to give: refused, nothing taken

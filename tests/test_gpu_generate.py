@@ -154,6 +154,27 @@ def test_running_out_of_pages_preempts_and_recomputes_to_the_same_tokens():
     assert m.groups[0].pool.num_free == 8 and m.groups[0].pool.reuse_count > 0
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_tokens_recomputed_after_a_preemption_in_bfloat16_are_still_the_plain_argmax(name):
+    # In bfloat16 a preempted request's earlier tokens come back through the prompt kernels, so its later tokens need
+    # not be the bits of an undisturbed run; they must still be right: every token the plain argmax given the
+    # engine's own prefix, within the rounding of the logits.
+    from pico_vllm_amd import SamplingParams
+    prompts = prompts_for(name, [30, 30, 30, 17], seed=14)
+    sp = SamplingParams(max_new_tokens=40, temperature=0.0, ignore_eos=True)
+    pages = 8 * 16 // PAGE_SIZE[name]                               # room for 128 tokens: four requests of up to 70 do not fit
+    for graphs in (False, True):
+        tight_llm = llm(name, "bfloat16", num_gpu_blocks=pages, use_cuda_graph=graphs, max_batch_size=4)
+        tight = tight_llm.generate(prompts, sp)
+        assert tight_llm.engine.stats["preemptions"] > 0 and sum(o.num_preemptions for o in tight) > 0
+        assert tight[0].num_preemptions == 0
+        assert [len(o.token_ids) for o in tight] == [40] * 4 and all(o.finish_reason == "length" for o in tight)
+        check_greedy(name, "bfloat16", prompts, tight)
+        m = tight_llm.engine.runner.manager
+        m.check()
+        assert m.groups[0].pool.num_free == pages and m.groups[0].pool.reuse_count > 0 and not m.requests
+
+
 def test_submit_step_is_done_in_the_reference_manner():
     from pico_vllm_amd import EngineArgs
     from pico_vllm_amd.engine.llm import LLMEngine
@@ -298,8 +319,10 @@ def test_a_finished_request_leaves_the_engine():
     assert eng.engine.requests == {} and not eng.engine.runner.manager.requests
 
 
-def test_phase_timers_behind_their_flag_change_nothing():
+def test_phase_timers_behind_their_flag_change_nothing(monkeypatch):
     from pico_vllm_amd import SamplingParams
+    from pico_vllm_amd.engine.phases import PhaseTimers
+    monkeypatch.setattr(PhaseTimers, "COLLECT_EVERY", 6)        # events are read while the run goes on, not only by a report
     prompts = prompts_for("A", [5, 30, 11], seed=6)
     sp = SamplingParams(max_new_tokens=12, temperature=0.0, ignore_eos=True)
     plain_run = llm("A", "bfloat16", use_cuda_graph=True, max_batch_size=4)
@@ -307,6 +330,7 @@ def test_phase_timers_behind_their_flag_change_nothing():
     a, b = plain_run.generate(prompts, sp), timed.generate(prompts, sp)
     assert [o.token_ids for o in a] == [o.token_ids for o in b]
     assert "phases" not in plain_run.engine.report()
+    assert len(timed.engine.timers._pending) < 4 * 6 and timed.engine.timers.device_s["model"] > 0
     rep = timed.engine.report()
     steps = rep["steps"]
     assert steps >= 12 and rep["decode_tokens"] > 0 and rep["prefill_tokens"] == 46

@@ -143,7 +143,8 @@ def test_gemm_bf16(K, M, N, K_, out_dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,rot,Pg", [(4, 1, 16, 16, 16), (6, 3, 32, 32, 8), (5, 5, 48, 48, 16), (2, 2, 64, 32, 32),
-                                            (12, 2, 128, 128, 16), (3, 1, 24, 8, 16), (28, 4, 128, 128, 16)])
+                                            (12, 2, 128, 128, 16), (3, 1, 24, 8, 16), (28, 4, 128, 128, 16),
+                                            (6, 2, 24, 24, 8), (5, 1, 40, 40, 16), (4, 4, 72, 72, 8), (2, 1, 250, 250, 16)])
 def test_rope_and_cache_store(K, dtype, nq, nkv, d, rot, Pg):
     theta = 10000.0
     new_lens, prefix_lens = [5, 1, 9], [14, 33, 0]          # 14..18 crosses a page edge of 16 (store_kvcache.py:107-118)
@@ -224,6 +225,33 @@ def test_plain_attention_kernel_on_the_reference_cases(K, dtype, case):
 def test_plain_attention_kernel_other_sizes(K, dtype, nq, nkv, d, Pg):
     out, want = _attn_case(K, dtype, [7, 1, 30, 2], [0, 70, 45, 129], nq, nkv, d, Pg, seed=3)
     close(out, want, dtype)
+
+
+# Head sizes that are no multiple of 16 (the configuration allows any even one): the matrix-core kernels do not take
+# them, so both engine precisions go through this kernel there.
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Pg", [8, 16])
+@pytest.mark.parametrize("nq,nkv,d", [(6, 2, 24), (5, 1, 40), (4, 4, 72), (3, 1, 2), (2, 1, 250)])
+@pytest.mark.parametrize("case", range(len(REFERENCE_CASES)))
+def test_plain_attention_kernel_at_head_sizes_between_the_steps_of_16(K, dtype, Pg, nq, nkv, d, case):
+    # the reference's own (new, prefix) cases (tests/test_prefill_paged_attn.py:183-260), with grouped heads
+    new_lens, prefix_lens = REFERENCE_CASES[case]
+    out, want = _attn_case(K, dtype, new_lens, prefix_lens, nq, nkv, d, Pg, seed=case + d)
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("d", [24, 40, 72])
+def test_attention_finds_one_far_key_at_head_sizes_between_the_steps_of_16(K, dtype, d):
+    # as below: a dropped key, page or tail of the head dimension would show
+    for far in (0, 7, 8, 63, 64, 301):
+        def boost(qs, ks, vs, far=far):
+            ks[0][far] = qs[0][-1, 0:1, :] * 8.0          # (a short head: a large factor makes the score stand out)
+            vs[0][far] = 100.0
+            vs[0][far][..., d - 1] = -100.0          # the last head dimension carries a value of its own
+        out, want = _attn_case(K, dtype, [3], [330], 3, 1, d, 8, seed=far, boost=boost)
+        assert float(want[-1, 0, :d - 1].mean()) > 50 and float(want[-1, 0, d - 1]) < -50
+        close(out, want, dtype, scale=100)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -399,6 +427,34 @@ def test_sampling_at_the_edges_of_its_options(K):
                 p = P.top_p_probs(logits[r].double(), 50.0, float(top_ps[r]))
                 want = P.inverse_cdf(p, u)
                 assert 0 <= out[r] < V and (out[r] == want or abs(float(torch.cumsum(p, 0)[min(out[r], want)]) - u) < 1e-4), (V, u, r, out[r], want)
+
+
+def test_sampling_never_returns_a_token_whose_probability_underflowed(K):
+    # a low temperature leaves a handful of tokens with a probability above zero; with u just below 1 the running sum
+    # of a thread may stop short of the target by rounding, and the fallback must then be the last token that has
+    # any probability, never one of the thousands behind it whose exp() is 0
+    g = torch.Generator().manual_seed(5)
+    for V in (1000, 151936):
+        logits = torch.randn(4, V, generator=g)
+        alive = [sorted(torch.randperm(V, generator=g)[:3].tolist()) for _ in range(4)]
+        for r, idx in enumerate(alive):
+            logits[r, idx] = torch.tensor([30.0, 30.5, 29.5])
+        temps = torch.full((4,), 0.05)                       # exp((x - 30.5) / 0.05) is 0 for every other token
+        for u in (0.0, 0.5, 0.9999999, 1.0 - 2.0 ** -24):
+            out = K.sample(logits.to(DEV), temps.to(DEV), torch.ones(4, device=DEV), torch.full((4,), u).to(DEV),
+                           top_p_rows=False).tolist()
+            assert all(out[r] in alive[r] for r in range(4)), (V, u, out, alive)
+            out = K.sample(logits.to(DEV), temps.to(DEV), torch.tensor([1.0, 0.9, 0.5, 1.0]).to(DEV),
+                           torch.full((4,), u).to(DEV)).tolist()
+            assert all(out[r] in alive[r] for r in range(4)), (V, u, out, alive)
+
+
+def test_sampling_refuses_a_workspace_that_is_not_16_byte_aligned(K):
+    logits = torch.randn(2, 100).to(DEV)
+    ones = torch.ones(2, device=DEV)
+    work = K.sample_workspace(3, DEV)
+    with pytest.raises(K.KernelError, match="workspace"):
+        K.sample(logits, ones, ones, ones * 0.5, work=work[2:])          # 8 bytes off
 
 
 def test_sampling_top_p(K):

@@ -256,11 +256,13 @@ def compare(name, dtype, reqs, got, label):
     print(f"[replay] {label} {name} {dtype}: worst position {worst:.2f}x the draws' rms there")
 
 
-LENGTHS = {"A": [70, 45, 100, 33, 64, 90], "B": [41, 97, 34, 80, 65, 50], "C": [50, 36, 81]}
+LENGTHS = {"A": [70, 45, 100, 33, 64, 90], "B": [41, 97, 34, 80, 65, 50], "C": [50, 36, 81],
+           # head sizes 24 and 40: no multiple of 16, so both precisions take the plain attention kernel
+           "G": [70, 41, 97, 33, 64, 50], "H": [45, 100, 34, 80]}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "G", "H"])
 def test_whole(name, dtype):
     reqs = make_requests(name, LENGTHS[name])
     got, _ = replay(name, dtype, whole(reqs))
@@ -268,7 +270,7 @@ def test_whole(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "G", "H"])
 def test_last_32_tokens_one_by_one(name, dtype):
     reqs = make_requests(name, LENGTHS[name][:3], seed=1)
     got, _ = replay(name, dtype, tail_one_by_one(reqs))
@@ -276,7 +278,7 @@ def test_last_32_tokens_one_by_one(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "G", "H"])
 def test_portions_of_changing_size(name, dtype):
     reqs = make_requests(name, LENGTHS[name][:4], seed=2)
     got, _ = replay(name, dtype, portions(reqs))
@@ -284,7 +286,7 @@ def test_portions_of_changing_size(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "G"])
 def test_mixed_with_pages_used_again(name, dtype):
     reqs = make_requests(name, LENGTHS[name] + [57, 38], seed=3)
     trace = mixed(reqs, seed=4)
@@ -295,7 +297,7 @@ def test_mixed_with_pages_used_again(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", [f"R{i}" for i in range(10)] + ["D"])
+@pytest.mark.parametrize("name", [f"R{i}" for i in range(10)] + ["D", "H"])
 def test_configurations_drawn_at_random_whole_and_mixed(name, dtype):
     # sizes nobody picked by hand: whole requests, and the same requests mixed in a small pool
     reqs = make_requests(name, [40, 77, 33, 60], seed=7)
@@ -385,12 +387,101 @@ def test_long_decoding_and_first_tokens():
         assert (np.abs(first - ref).max(axis=1) <= NOISIER[dtype] * noise_bounds(draws)[1] * n_max[:4]).all()
 
 
-def test_the_program_itself_in_a_subprocess():
-    reqs = make_requests("A", [40, 23], seed=8)
-    trace = mixed(reqs, seed=9)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_model_without_layers_is_norm_times_output_matrix(dtype):
+    # num_hidden_layers = 0 is a configuration the reader accepts: no cache group, no page, the final norm straight on
+    # the embedding rows and the untied output matrix (the formula of test_plain.py's test of the same name)
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    reqs = make_requests("Z", [40, 3, 21], seed=12)
+    w = {k: v.double() for k, v in P.read_weights(model_dir("Z")).items()}
+    E, g, W = w["model.embed_tokens.weight"], w["model.norm.weight"], w["lm_head.weight"]
+    for trace in (whole(reqs), mixed(reqs, seed=2, tail=4)):
+        rp = TraceReplayer(model_dir("Z"), dtype, trace.live_peak, PAGE_SIZE["Z"])
+        assert not rp.runner.manager.groups
+        for step in trace.steps:
+            out = rp.run_step(step)
+            for row, (rid, pos) in zip(out if out is not None else [], trace.rows[step["step"]]):
+                x = E[reqs[rid][pos]]
+                want = (x / torch.sqrt((x * x).mean() + CONFIGS["Z"]["rms_norm_eps"]) * g) @ W.T
+                err = float((torch.from_numpy(row).double() - want).abs().max())
+                assert err <= (2e-6 if dtype == "float32" else 2e-2) * float(want.abs().max()), (rid, pos, err)
+        rp.runner.manager.check()
+        assert not rp.live
+    compare("Z", dtype, reqs, replay_rows(TraceReplayer(model_dir("Z"), dtype, 256, PAGE_SIZE["Z"]), whole(reqs)), "no layers")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_two_requests_that_share_the_pages_of_a_prefix_in_one_step(name, dtype):
+    # ``fork_prefix`` lets a second request hold the whole pages of a first one's prefix (what an index of shared
+    # prefixes would do; the reference adopts matched blocks, pico_vllm/cache.py:170-192).  Two block tables then name
+    # the same pages in one step: a portion of one request beside single tokens and portions of the other.
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    page = PAGE_SIZE[name]
+    V = CONFIGS[name]["vocab_size"]
+    rng = random.Random(21)
+    shared = 5 * page
+    first = [rng.randrange(V) for _ in range(shared + 30)]
+    second = first[:shared] + [rng.randrange(V) for _ in range(41)]           # the same prefix, another continuation
+    reqs = {"a": first, "b": second}
+    rp = TraceReplayer(model_dir(name), dtype, 4 * 64 + 64, page)
+    run, m = rp.runner, rp.runner.manager
+    got = {}
+
+    def step(entries):
+        seqs = []
+        for rid, lo, hi in entries:
+            assert m.grow(rid, hi)
+            seqs.append(SeqStep(rid, reqs[rid][lo:hi], list(range(hi - lo))))
+        out = run.step(seqs).float().cpu().numpy()
+        run.advance(seqs)
+        at = 0
+        for rid, lo, hi in entries:
+            for p in range(lo, hi):
+                got[rid, p] = out[at]
+                at += 1
+
+    assert m.add_request("a") and m.add_request("b")
+    step([("a", 0, shared + 3)])                               # the prefix and a little more, alone
+    m.fork_prefix("a", "b", shared)
+    assert m.block_table("b")[:5] == m.block_table("a")[:5] and m.num_computed("b") == shared
+    pool = m.groups[0].pool
+    assert all(pool.ref_count(p) == 2 for p in m.block_table("a")[:5])
+    step([("a", shared + 3, shared + 4), ("b", shared, shared + 17)])           # a single token beside a portion
+    step([("b", shared + 17, shared + 19), ("a", shared + 4, shared + 20)])     # portions of both, the other way round
+    step([("a", shared + 20, shared + 21), ("b", shared + 19, shared + 20)])    # two single tokens
+    m.check()
+    step([("a", shared + 21, shared + 30)])
+    m.free_request("a")                                        # the shared pages stay: b still holds them
+    assert all(pool.ref_count(p) == 1 for p in m.block_table("b")[:5])
+    step([("b", shared + 20, shared + 41)])
+    m.check()
+    m.free_request("b")
+    assert pool.num_free == pool.num_pages
+    for rid in reqs:                                           # b's prefix positions were never run: a's rows stand for them
+        for p in range(shared):
+            got.setdefault((rid, p), got["a", p])
+    compare(name, dtype, reqs, got, "shared prefix")
+
+
+def replay_rows(rp, trace):
+    """The rows a replayer gives for a trace, by (request, position)."""
+    got = {}
+    for step in trace.steps:
+        out = rp.run_step(step)
+        for row, key in zip(out if out is not None else [], trace.rows[step["step"]]):
+            got[key] = row
+    return got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_program_itself_in_a_subprocess(dtype):
+    reqs = make_requests("A", [40, 23, 50, 31, 36], seed=8)
+    trace = mixed(reqs, seed=9, max_live=2)
     with tempfile.TemporaryDirectory() as out:
         inp = "\n".join(json.dumps(s) for s in trace.steps) + "\n"
-        r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir("A"), "--dtype", "float32",
+        r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir("A"), "--dtype", dtype,
                             "--out", out, "--max-tokens", str(trace.live_peak)],
                            input=inp, capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, r.stderr[-2000:]
@@ -404,7 +495,28 @@ def test_the_program_itself_in_a_subprocess():
                 a = np.fromfile(path, dtype="<f4").reshape(len(rows), -1)
                 for row, key in zip(a, rows):
                     got[key] = row
-        compare("A", "float32", reqs, got, "program")
+        compare("A", dtype, reqs, got, "program")
+        # from what the program wrote alone: every token landed on a page its request held, no page under two live
+        # requests at once, and pages that ended requests gave back were used again by later ones
+        with open(os.path.join(out, "pages.jsonl")) as f:
+            log = [json.loads(line) for line in f]
+        assert [e["step"] for e in log] == [s["step"] for s in trace.steps]
+        owner, owners_ever, fed = {}, {}, {}
+        for e, s in zip(log, trace.steps):
+            assert [x["id"] for x in e["entries"]] == [x["id"] for x in s["entries"]]
+            for x, y in zip(e["entries"], s["entries"]):
+                assert x["first_position"] == fed.get(x["id"], 0)
+                fed[x["id"]] = x["first_position"] + len(y["tokens"])
+                (pages,) = x["pages"]                       # one group of layers
+                lo, hi = x["first_position"] // PAGE_SIZE["A"], -(-fed[x["id"]] // PAGE_SIZE["A"])
+                assert len(pages) == hi - lo and all(p >= 0 for p in pages)
+                for p in pages:
+                    assert owner.setdefault(p, x["id"]) == x["id"], f"page {p} under two live requests"
+                    owners_ever.setdefault(p, set()).add(x["id"])
+            for rid in e["end"]:
+                owner = {p: o for p, o in owner.items() if o != rid}
+        assert any(len(o) > 1 for o in owners_ever.values()), "no page was used again"
+        assert len(owners_ever) <= trace.live_peak // PAGE_SIZE["A"]
 
 
 def test_the_program_says_what_is_wrong_with_a_trace(tmp_path):

@@ -52,7 +52,8 @@ def test_argmax_without_allocation_twice_in_a_row_the_second_smaller():
     logits = big.to(DEV)
     out, want = _both(lib, logits, 37, 5003)
     assert torch.equal(out, want)
-    assert torch.equal(out.long(), big.argmax(dim=1)) or int(out[7]) == 100
+    others = [r for r in range(37) if r != 7]           # (row 7 holds a tie, which torch's argmax need not break alike)
+    assert torch.equal(out.long()[others], big.argmax(dim=1)[others])
     assert int(out[5]) == 4999 and int(out[6]) == 0 and int(out[7]) == 100
     # a smaller input straight after: fewer rows, fewer columns, so that every chunk boundary moves and the
     # entries of rows 5 .. 36 in the library's memory are stale
@@ -65,7 +66,8 @@ def test_argmax_without_allocation_twice_in_a_row_the_second_smaller():
     # and the first input again, a row stride wider than the row
     out3, want3 = _both(lib, logits, 20, 4000)
     assert torch.equal(out3, want3)
-    assert torch.equal(out3.long(), big[:20, :4000].argmax(dim=1)) or int(out3[7]) == 100
+    others = [r for r in range(20) if r != 7]
+    assert torch.equal(out3.long()[others], big[:20, :4000].argmax(dim=1)[others]) and int(out3[7]) == 100
 
 
 def test_more_rows_than_the_library_holds_are_refused():

@@ -37,8 +37,22 @@ TINY_F = {   # for contexts of thousands of tokens: two heads of 64 on one kv he
     "num_key_value_heads": 1, "intermediate_size": 264, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
     "tie_word_embeddings": False, "max_position_embeddings": 16384, "hidden_act": "silu",
 }
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "F": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
+TINY_G = {   # head size 24, between the steps of 16 that the matrix-core attention takes: groups of 3, pages of 8
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 271, "hidden_size": 144, "num_hidden_layers": 2, "num_attention_heads": 6,
+    "num_key_value_heads": 2, "intermediate_size": 208, "rms_norm_eps": 1e-5,
+    "rope_theta": 10000.0, "tie_word_embeddings": False, "max_position_embeddings": 1024, "hidden_act": "silu",
+}
+TINY_H = {   # head size 40 given explicitly, five heads on one kv head, a width that is not heads * head
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "vocab_size": 263, "hidden_size": 120, "num_hidden_layers": 3, "num_attention_heads": 5,
+    "num_key_value_heads": 1, "head_dim": 40, "intermediate_size": 176, "rms_norm_eps": 1e-6,
+    "rope_theta": 1000000.0, "tie_word_embeddings": True, "max_position_embeddings": 1024, "hidden_act": "silu",
+}
+TINY_Z = dict(TINY_B, num_hidden_layers=0)       # no layer at all: embedding, final norm, untied output matrix
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "F": 16, "G": 8, "H": 16, "Z": 8}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F, "G": TINY_G, "H": TINY_H,
+           "Z": TINY_Z}
 
 
 def drawn(seed: int):
