@@ -18,7 +18,11 @@ decoded tokens a second as ``value`` (K steps between two synchronisations, the 
 ``ms_per_step_median`` from device events around every step; ``prefill`` (one 2,048-token prompt in one
 step, median of device-event times) with its TFLOP/s and its fraction of the bf16 matrix-core peak;
 ``roofline`` (bytes the decode step has to read: every weight once plus the cache of the live requests,
-over its time, against 8 TB/s); ``points`` with decode at batch 1 and 64.  Beside the published peaks
+over its time, against 8 TB/s); ``points`` with decode at batch 1 and 64; ``points_other`` with the Qwen2.5-7B shape
+(all 28 layers, weights drawn on the GPU): decode at batch 8 with contexts ending at 8,192 tokens and the 2,048-token
+prefill.  What a step reads and computes is asked of the model's parts (``DecoderModel.num_weight_bytes`` /
+``flops``), its sizes for the record of the architecture's registry entry: this program reads no key of any
+architecture's configuration.  Beside the published peaks
 stand measured ones (``measured_peak``): a read stream over 2 GiB and a loop of matrix-core products, by
 this package's own kernels on the same GPU in the same run.
 """
@@ -40,27 +44,32 @@ MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 from pico_vllm_amd.config.presets import preset   # noqa: E402  (needs ROOT on the path)
 
-CONFIG_1P5B = preset("1.5b")       # the default run: the Qwen2.5-1.5B shape
-CONFIG_7B = preset("7b")           # the Qwen2.5-7B shape (measured with fewer layers when asked: --layers)
-SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", CONFIG_1P5B), "7b": ("Qwen2.5-7B shape", CONFIG_7B),
+# name -> (what the record calls it, the configuration as its config.json would hold it); the default run is the
+# Qwen2.5-1.5B shape, the others are measured with fewer layers when asked (--layers)
+SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", preset("1.5b")), "7b": ("Qwen2.5-7B shape", preset("7b")),
           "32b": ("Qwen2.5-32B shape", preset("32b"))}
-CONFIG = CONFIG_1P5B         # the shape being measured (set in main)
+CONFIG = SHAPES["1.5b"][1]   # the shape being measured (set in main)
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
+OTHER_SHAPE, OTHER_CONTEXT = "7b", 8192      # ``points_other``
+
+
+def describe(raw):
+    """(registry entry, typed configuration, model description) of a configuration."""
+    from pico_vllm_amd.config.registry import resolve_architecture
+    arch = resolve_architecture(raw)
+    typed = arch.config_from_dict(raw)
+    return arch, typed, arch.build_spec(typed)
 
 
 def log(msg: str) -> None:
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
-def prefill_flops(cfg, T: int) -> float:
-    """GEMM flops of T prompt tokens, causal attention flops, and the output matrix on one row."""
-    H, L, nq, nkv = cfg["hidden_size"], cfg["num_hidden_layers"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
-    d = cfg.get("head_dim") or H // nq
-    I, V = cfg["intermediate_size"], cfg["vocab_size"]
-    per_token = 2.0 * L * (H * (nq + 2 * nkv) * d + nq * d * H + 2 * H * I + I * H)
-    attn = 4.0 * nq * d * (T * (T + 1) / 2) * L
-    return per_token * T + attn + 2.0 * H * V
+def prefill_flops(model, T: int) -> float:
+    """What a prompt of T tokens alone costs: the matrices for every token, attention over the T (T + 1) / 2 (query,
+    key) pairs of a causal mask, and the output matrix on one row; each part of the model reports its own."""
+    return model.flops(T, T * (T + 1) // 2, 1)
 
 
 def measured_peaks():
@@ -81,12 +90,9 @@ def device_model(cfg, dtype, seed=0):
     folders: matrices and biases N(0, 0.02), norm weights 1 + U(-0.1, 0.1)): for sizes whose file would take
     longer to write and read than the measurement."""
     import torch
-    from pico_vllm_amd.config.registry import resolve_architecture
     from pico_vllm_amd.parts.model import DecoderModel
-    arch = resolve_architecture(cfg)
-    typed = arch.config_from_dict(cfg)
-    model = DecoderModel(arch.build_spec(typed), {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype],
-                         torch.device("cuda:0"))
+    _, typed, spec = describe(cfg)
+    model = DecoderModel(spec, {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype], torch.device("cuda:0"))
     g = torch.Generator(device="cuda:0").manual_seed(seed)
     tensors = {}
     for p in model.param_specs():
@@ -103,26 +109,28 @@ def device_model(cfg, dtype, seed=0):
     return model
 
 
-def make_engine(model_dir, dtype, batch, layers_model=None):
+def make_engine(model_dir, dtype, batch, layers_model=None, context=None):
     from pico_vllm_amd import EngineArgs
     from pico_vllm_amd.engine.llm import LLMEngine
     block = 16
+    context = context or CONTEXT
     args = EngineArgs(model=model_dir, dtype=dtype, block_size=block,
-                      num_gpu_blocks=batch * (CONTEXT // block + 1) + 8, max_seq_len=CONTEXT + 16,
+                      num_gpu_blocks=batch * (context // block + 1) + 8, max_seq_len=context + 16,
                       max_num_seqs=batch, max_num_batched_tokens=max(PREFILL_TOKENS, batch),
                       use_cuda_graph=True, max_batch_size=64, tune_library_gemm=True)
     return LLMEngine(args, model=layers_model)
 
 
-def decode_point(model_dir, model, dtype, batch, steps, warmup):
-    """Fill `batch` requests so that the timed steps end at CONTEXT tokens, then time `steps` decode steps."""
+def decode_point(model_dir, model, dtype, batch, steps, warmup, context=None):
+    """Fill `batch` requests so that the timed steps end at the context length, then time `steps` decode steps."""
     import torch
-    eng = make_engine(model_dir, dtype, batch, model)
-    V = CONFIG["vocab_size"]
+    context = context or CONTEXT
+    eng = make_engine(model_dir, dtype, batch, model, context)
+    V = eng.model.spec.vocab_size
     g = torch.Generator().manual_seed(batch)
     # while later prompts are still being prefilled the earlier requests already decode: leave room for that
-    slack = batch * (-(-CONTEXT // PREFILL_TOKENS)) + 2
-    prompt_len = CONTEXT - (warmup + steps) - 1 - slack
+    slack = batch * (-(-context // PREFILL_TOKENS)) + 2
+    prompt_len = context - (warmup + steps) - 1 - slack
     for i in range(batch):
         ids = torch.randint(0, V, (prompt_len,), generator=g).tolist()
         eng.submit(ids, max_new_tokens=warmup + steps + 1 + slack, temperature=0.0, ignore_eos=True)
@@ -168,12 +176,12 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup):
     return res, model
 
 
-def prefill_point(model_dir, model, dtype, reps=7, tokens=PREFILL_TOKENS):
+def prefill_point(model_dir, model, dtype, reps=7, tokens=PREFILL_TOKENS, context=None):
     import torch
     from pico_vllm_amd.engine.batch import SeqStep
     peak = measured_peaks()[1] if dtype == "bfloat16" else None       # before the timed steps: a profile ends with them
-    eng = make_engine(model_dir, dtype, 1, model)
-    V = CONFIG["vocab_size"]
+    eng = make_engine(model_dir, dtype, 1, model, context)
+    V = eng.model.spec.vocab_size
     ids = torch.randint(0, V, (tokens,), generator=torch.Generator().manual_seed(7)).tolist()
     m = eng.runner.manager
     times = []
@@ -192,7 +200,7 @@ def prefill_point(model_dir, model, dtype, reps=7, tokens=PREFILL_TOKENS):
         m.free_request(rid)
     times = sorted(times[1:])                         # the first run builds, tunes and warms
     dt = times[len(times) // 2]
-    flops = prefill_flops(CONFIG, tokens)
+    flops = prefill_flops(eng.model, tokens)
     out = {"value": tokens / dt, "tokens": tokens, "ms": dt * 1e3, "ms_min": times[0] * 1e3,
            "tflops": flops / dt / 1e12, "frac": flops / dt / MFMA_PEAK[dtype]}
     if peak is not None:
@@ -207,7 +215,7 @@ def sweep_point(model_dir, model, dtype, batch, bin_width=256):
     pico_vllm/profiling/profile_pagedkvcacheTritoncompile.py:43-113, for its successive engines)."""
     import torch
     eng = make_engine(model_dir, dtype, batch, model)
-    V = CONFIG["vocab_size"]
+    V = eng.model.spec.vocab_size
     g = torch.Generator().manual_seed(11)
     new = CONTEXT - 16
     for _ in range(batch):
@@ -237,7 +245,7 @@ def long_prompt_point(model_dir, model, dtype, prompt_len):
     until its first token is sampled."""
     import torch
     eng = make_engine(model_dir, dtype, 1, model)
-    V = CONFIG["vocab_size"]
+    V = eng.model.spec.vocab_size
     g = torch.Generator().manual_seed(3)
     warm = eng.submit(torch.randint(0, V, (prompt_len,), generator=g).tolist(), max_new_tokens=2, ignore_eos=True)
     while not eng.is_done():
@@ -258,11 +266,7 @@ def long_prompt_point(model_dir, model, dtype, prompt_len):
     del eng
     torch.cuda.empty_cache()
     return {"tokens": prompt_len, "portions": steps, "ms": dt * 1e3, "tok_s": prompt_len / dt,
-            "tflops": prefill_flops_long(CONFIG, prompt_len) / dt / 1e12}, model
-
-
-def prefill_flops_long(cfg, T):
-    return prefill_flops(cfg, T)
+            "tflops": prefill_flops(model, prompt_len) / dt / 1e12}, model
 
 
 def serve_point(model_dir, dtype, requests, max_new, model=None):
@@ -282,7 +286,7 @@ def serve_point(model_dir, dtype, requests, max_new, model=None):
     eng = LLMEngine(EngineArgs(model=model_dir, dtype=dtype, block_size=block, num_gpu_blocks=pages, max_seq_len=CONTEXT,
                                max_num_seqs=requests, max_num_batched_tokens=PREFILL_TOKENS, use_cuda_graph=True,
                                max_batch_size=64, tune_library_gemm=True), model=model)
-    V = CONFIG["vocab_size"]
+    V = eng.model.spec.vocab_size
     # a short run first: kernels built and tuned, graphs captured for the batch sizes of the run's tail
     for n in (PREFILL_TOKENS, 300):
         eng.submit(torch.randint(0, V, (n,), generator=g).tolist(), max_new_tokens=4, ignore_eos=True)
@@ -308,8 +312,9 @@ def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20, chunk_len=0):
     with the shape's heads; ``shape``: what FastAttention.prefill_teams would return, 0 = ask it."""
     import torch
     from pico_vllm_amd.ops.attention_fast import FastAttention
-    nq, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
-    d, P, dev = cfg["hidden_size"] // nq, 16, "cuda"
+    mixer = describe(cfg)[2].layers[0].slots["mixer"][1].params          # the constants of the first layer's attention part
+    nq, nkv, d = mixer["num_heads"], mixer["num_kv_heads"], mixer["head_dim"]
+    P, dev = 16, "cuda"
     g = torch.Generator(device=dev).manual_seed(0)
     ctx = new_len + prefix
     per = -(-ctx // P)
@@ -336,7 +341,8 @@ def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20, chunk_len=0):
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) / reps * 1e3
     flops = 4.0 * nq * d * nseq * (new_len * prefix + new_len * (new_len + 1) / 2)
-    return {"us": round(us, 1), "shape": shape, "tflops": round(flops / us / 1e6, 1), "frac": round(flops / (us * 1e-6) / MFMA_PEAK["bfloat16"], 4)}
+    return {"us": round(us, 1), "shape": shape, "tflops": round(flops / us / 1e6, 1), "frac": round(flops / (us * 1e-6) / MFMA_PEAK["bfloat16"], 4),
+            "heads": nq, "kv_heads": nkv}
 
 
 def sampling_point(cfg, rows, top_p, reps=50):
@@ -344,7 +350,7 @@ def sampling_point(cfg, rows, top_p, reps=50):
     and temperature 0.8 with ``top_p``; microseconds a call."""
     import torch
     from pico_vllm_amd.ops import kernels
-    dev, V = "cuda", cfg["vocab_size"]
+    dev, V = "cuda", describe(cfg)[2].vocab_size
     g = torch.Generator(device=dev).manual_seed(0)
     logits = torch.randn(rows, V, device=dev, generator=g) * 3.0
     u = torch.rand(rows, device=dev, generator=g)
@@ -365,7 +371,31 @@ def sampling_point(cfg, rows, top_p, reps=50):
         e1.record()
         torch.cuda.synchronize()
         res[name] = round(e0.elapsed_time(e1) / reps * 1e3, 1)
+    res["vocab"] = V
     return res
+
+
+def other_shape_points(dtype, steps, warmup):
+    """``points_other``: the OTHER_SHAPE shape with all its layers (weights drawn on the GPU), decode at batch 8 with
+    contexts ending at OTHER_CONTEXT tokens and the 2,048-token prefill."""
+    import torch
+    name, raw = SHAPES[OTHER_SHAPE]
+    arch, typed, _ = describe(raw)
+    t0 = time.time()
+    model = device_model(raw, dtype)
+    torch.cuda.synchronize()
+    log(f"{name}: {model.num_weight_bytes() / 1e9:.1f} GB of matrices drawn on the GPU in {time.time() - t0:.0f}s")
+    r, model = decode_point("", model, dtype, 8, steps, warmup, OTHER_CONTEXT)
+    log(f"{name} decode batch 8 at context {OTHER_CONTEXT}: {r['tok_s']:.0f} tok/s, {r['ms_per_step']:.3f} ms/step")
+    pf = prefill_point("", model, dtype, reps=5, context=OTHER_CONTEXT)
+    log(f"{name} prefill: {pf}")
+    del model
+    torch.cuda.empty_cache()
+    return {"model": name, "layers": arch.sizes(typed)["layers"], "context": OTHER_CONTEXT,
+            "decode_b8": round(r["tok_s"], 1), "decode_b8_ms_per_step": round(r["ms_per_step"], 4),
+            "decode_b8_gbytes_per_step": round(r["bytes"] / 1e9, 3), "decode_b8_hbm_frac": round(r["gbps"] * 1e9 / HBM_PEAK, 4),
+            "prefill_tokens": pf["tokens"], "prefill_tok_s": round(pf["value"], 1), "prefill_ms": round(pf["ms"], 4),
+            "prefill_tflops": round(pf["tflops"], 1), "prefill_frac": round(pf["frac"], 4)}
 
 
 def main() -> int:
@@ -375,7 +405,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill (long workload: the decode points)")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill and the other shape (long workload: the decode points)")
+    ap.add_argument("--no-other", action="store_true", help="skip ``points_other`` (the 7B shape)")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --prefill-only: the prompt's length (2 to 2048; the contract's prefill is of 2,048 tokens)")
@@ -401,12 +432,15 @@ def main() -> int:
     a = ap.parse_args()
     global CONFIG, CONTEXT
     shape_name, full = SHAPES[a.shape]
+    arch, typed_full, _ = describe(full)
+    layers_full = arch.sizes(typed_full)["layers"]
     CONFIG = dict(full)
     if a.layers:
-        if not 0 < a.layers <= full["num_hidden_layers"]:
-            print(f"bench.py: --layers must be 1..{full['num_hidden_layers']}")
+        if not 0 < a.layers <= layers_full:
+            print(f"bench.py: --layers must be 1..{layers_full}")
             return 2
-        CONFIG["num_hidden_layers"] = a.layers
+        CONFIG = arch.with_layers(full, a.layers)
+    sizes = arch.sizes(arch.config_from_dict(CONFIG))       # flat: layers, hidden, q_heads, kv_heads, head_dim, intermediate, vocab, tied
     CONTEXT = a.context
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -425,7 +459,7 @@ def main() -> int:
                             chunk_len=nums[4] if len(nums) > 4 else 0)
         print(json.dumps({"metric": "prefill attention kernel", "unit": "us", "value": r["us"], "workgroup_shape": r["shape"],
                           "tflops": r["tflops"], "frac_of_bf16_peak": r["frac"], "sequences": nums[0], "new_tokens": nums[1],
-                          "prefix": nums[2], "heads": CONFIG["num_attention_heads"], "kv_heads": CONFIG["num_key_value_heads"]}))
+                          "prefix": nums[2], "heads": r["heads"], "kv_heads": r["kv_heads"]}))
         return 0
     if a.sampling:
         parts = a.sampling.split(",")
@@ -435,7 +469,7 @@ def main() -> int:
             return 2
         r = sampling_point(CONFIG, rows, top_p)
         print(json.dumps({"metric": "sampling call", "unit": "us", "value": r["top_p"], "greedy": r["greedy"],
-                          "temperature": r["temperature"], "top_p": r["top_p"], "rows": rows, "vocab_size": CONFIG["vocab_size"],
+                          "temperature": r["temperature"], "top_p": r["top_p"], "rows": rows, "vocab_size": r["vocab"],
                           "p": top_p}))
         return 0
     if a.write_model:
@@ -447,7 +481,7 @@ def main() -> int:
     preloaded = None
     if a.device_weights:
         t0 = time.time()
-        log(f"drawing random weights of the {shape_name}, {CONFIG['num_hidden_layers']} layers, on the GPU ...")
+        log(f"drawing random weights of the {shape_name}, {sizes['layers']} layers, on the GPU ...")
         preloaded = device_model(CONFIG, a.dtype)
         torch.cuda.synchronize()
         log(f"... {time.time() - t0:.0f}s, {preloaded.num_weight_bytes() / 1e9:.1f} GB of matrices")
@@ -456,7 +490,7 @@ def main() -> int:
         tmp = tempfile.mkdtemp(prefix="pico_bench_")
         model_dir = tmp
         t0 = time.time()
-        log(f"writing random weights of the {shape_name}, {CONFIG['num_hidden_layers']} layers ...")
+        log(f"writing random weights of the {shape_name}, {sizes['layers']} layers ...")
         write_random_model(model_dir, CONFIG, seed=0)
         log(f"... {time.time() - t0:.0f}s")
     try:
@@ -471,8 +505,8 @@ def main() -> int:
                 "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
                 "data": "synthetic: random weights N(0, 0.02), uniform random token ids, prompt lengths uniform in 128..4096",
                 "config": {"model": shape_name, "requests": a.requests, "new_tokens_each": a.max_new,
-                           "prompt_tokens": r["prompt_tokens"], "layers": full["num_hidden_layers"],
-                           "layers_run": CONFIG["num_hidden_layers"], "hidden": CONFIG["hidden_size"],
+                           "prompt_tokens": r["prompt_tokens"], "layers": layers_full,
+                           "layers_run": sizes["layers"], "hidden": sizes["hidden"],
                            "max_num_batched_tokens": PREFILL_TOKENS, "max_seq_len": CONTEXT, "page_size": 16,
                            "preemptions": r["preemptions"]}}), flush=True)
             return 0
@@ -482,8 +516,8 @@ def main() -> int:
         if a.workload == "sweep":
             rows = sweep_point(model_dir, preloaded, a.dtype, a.batch)
             print(json.dumps({"metric": f"decode ms/step by context, batch {a.batch}, {shape_name.split()[0]} {a.dtype}",
-                              "unit": "ms", "n_gpus": 1, "batch": a.batch, "layers_run": CONFIG["num_hidden_layers"],
-                              "layers": full["num_hidden_layers"], "rows": rows}), flush=True)
+                              "unit": "ms", "n_gpus": 1, "batch": a.batch, "layers_run": sizes["layers"],
+                              "layers": layers_full, "rows": rows}), flush=True)
             return 0
         if a.workload == "long":
             if a.prompt + 8 > CONTEXT:
@@ -504,10 +538,10 @@ def main() -> int:
                 "ms_per_step": pts["decode_b8"]["ms_per_step"] if pts else None, "higher_is_better": True,
                 "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
                 "data": "synthetic: random weights N(0, 0.02)" + (" drawn on the GPU" if a.device_weights else "") + ", uniform random token ids",
-                "config": {"model": shape_name, "layers": full["num_hidden_layers"], "layers_run": CONFIG["num_hidden_layers"],
-                           "hidden": CONFIG["hidden_size"], "q_heads": CONFIG["num_attention_heads"],
-                           "kv_heads": CONFIG["num_key_value_heads"], "intermediate": CONFIG["intermediate_size"],
-                           "vocab": CONFIG["vocab_size"], "seq_len": CONTEXT, "prompt": a.prompt, "portion": PREFILL_TOKENS,
+                "config": {"model": shape_name, "layers": layers_full, "layers_run": sizes["layers"],
+                           "hidden": sizes["hidden"], "q_heads": sizes["q_heads"],
+                           "kv_heads": sizes["kv_heads"], "intermediate": sizes["intermediate"],
+                           "vocab": sizes["vocab"], "seq_len": CONTEXT, "prompt": a.prompt, "portion": PREFILL_TOKENS,
                            "page_size": 16, "weight_gbytes": round(model.num_weight_bytes() / 1e9, 1)},
                 "long_prompt": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in lp.items()},
                 "points": pts}), flush=True)
@@ -522,12 +556,12 @@ def main() -> int:
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
             "config": {"model": shape_name, "global_batch": a.batch, "seq_len": CONTEXT,
-                       "parallelism": "single GPU", "layers": full["num_hidden_layers"],
-                       "layers_run": CONFIG["num_hidden_layers"], "hidden": CONFIG["hidden_size"],
-                       "q_heads": CONFIG["num_attention_heads"], "kv_heads": CONFIG["num_key_value_heads"],
-                       "head_dim": CONFIG["hidden_size"] // CONFIG["num_attention_heads"],
-                       "intermediate": CONFIG["intermediate_size"], "vocab": CONFIG["vocab_size"],
-                       "tied": CONFIG["tie_word_embeddings"],
+                       "parallelism": "single GPU", "layers": layers_full,
+                       "layers_run": sizes["layers"], "hidden": sizes["hidden"],
+                       "q_heads": sizes["q_heads"], "kv_heads": sizes["kv_heads"],
+                       "head_dim": sizes["head_dim"],
+                       "intermediate": sizes["intermediate"], "vocab": sizes["vocab"],
+                       "tied": sizes["tied"],
                        "page_size": 16, "prompt_len": int(main_res["prompt_len"]),
                        "context_in_timed_steps": round(main_res["context"], 1)},
             "roofline": {"bound": "hbm", "achieved": round(main_res["gbps"], 1), "peak": HBM_PEAK / 1e9,
@@ -554,6 +588,11 @@ def main() -> int:
                 # (README.md:9,43-45 of the reference); other hardware, so a context, not a baseline
                 pts["decode_b1_vs_reference_published"] = round(pts["decode_b1"] / 97.0, 2)
             out["points"] = pts
+            if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16" and not a.no_other:
+                # a second shape, driver-visible: the larger the matrices, the nearer a step comes to what the memory allows
+                del model
+                torch.cuda.empty_cache()
+                out["points_other"] = other_shape_points(a.dtype, min(a.steps, 50), min(a.warmup, 5))
         print(json.dumps(out), flush=True)
     finally:
         if tmp:

@@ -1,16 +1,14 @@
-"""Device tensors of the cache: pages of keys and values per layer, and the
+"""Device tensors of the cache: per layer the page tensors that its mixer's ``CacheSpec`` names, and the
 per-request state of mixers that keep one.
 
-Layout of one layer (one allocation each for K and V):
-  K [pages, kv heads, page size, head size]     a token's key is contiguous
-  V [pages, kv heads, head size, page size]     a head-dimension's values of a page are contiguous
-The reference keeps one tensor [2, L, pages, kv heads, page, d] for all layers
-(pico_vllm/blockmanager.py:39-42) with V laid out like K; V is transposed here
-because the matrix-core kernels contract over keys.
+A paged layer gets one allocation per tensor of its spec, [pages, *shape of one page] in the engine's dtype
+(or the tensor's own); what the tensors hold and how a page is laid out is the mixer's business.  The
+attention of this package asks for ``k`` and ``v`` (``parts.attention.kv_page_tensors``); the reference keeps
+one tensor [2, L, pages, kv heads, page, d] for all layers (pico_vllm/blockmanager.py:39-42).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Dict
 
 import torch
@@ -21,17 +19,36 @@ from .manager import CacheManager
 
 @dataclass
 class PagedKVLayer:
-    k: torch.Tensor
-    v: torch.Tensor
+    """The page tensors of one layer by name (also as attributes: ``layer.k``)."""
+    tensors: Dict[str, torch.Tensor]
     group: int
     page_size: int
     read_only: bool = False    # True for a run that reads another run's cache: it attends over it and stores nothing
+
+    def __getattr__(self, name: str) -> torch.Tensor:
+        try:
+            return self.__dict__["tensors"][name]
+        except KeyError:
+            raise AttributeError(f"this layer's cache has no tensor {name!r}; it holds {sorted(self.__dict__.get('tensors', {}))}") from None
 
 
 @dataclass
 class StateLayer:
     state: torch.Tensor        # [slots + 1, *state_shape]; the last slot belongs to padding rows
     group: int = -1
+
+
+def bytes_per_page(layer_specs: Dict[int, CacheSpec], page_size: int, dtype: torch.dtype) -> int:
+    """Device bytes that one more page in every group's pool costs, over all paged layers."""
+    total = 0
+    for spec in layer_specs.values():
+        if spec.kind == "paged_kv":
+            for t in spec.page_tensors:
+                n = 1
+                for s in t.resolved(page_size):
+                    n *= s
+                total += n * torch.empty(0, dtype=getattr(torch, t.dtype) if t.dtype else dtype).element_size()
+    return total
 
 
 class CacheStorage:
@@ -44,9 +61,9 @@ class CacheStorage:
             if spec.kind == "paged_kv":
                 gi = manager.layer_group[layer]
                 n = manager.groups[gi].pool.num_pages
-                k = torch.zeros(n, spec.num_kv_heads, P, spec.head_dim, dtype=dtype, device=device)
-                v = torch.zeros(n, spec.num_kv_heads, spec.head_dim, P, dtype=dtype, device=device)
-                self._layers[layer] = PagedKVLayer(k, v, gi, P)
+                self._layers[layer] = PagedKVLayer(
+                    {t.name: torch.zeros(n, *t.resolved(P), dtype=getattr(torch, t.dtype) if t.dtype else dtype, device=device)
+                     for t in spec.page_tensors}, gi, P)
             elif spec.kind == "state":
                 sdt = getattr(torch, spec.state_dtype)
                 # one slot more than requests can hold: the padding rows of a recorded decode batch write there
@@ -59,7 +76,7 @@ class CacheStorage:
         """The cache of run entry ``index``; ``read_only`` for a run that was given another run's cache."""
         entry = self._layers.get(index)
         if read_only and isinstance(entry, PagedKVLayer):
-            return PagedKVLayer(entry.k, entry.v, entry.group, entry.page_size, read_only=True)
+            return PagedKVLayer(entry.tensors, entry.group, entry.page_size, read_only=True)
         return entry
 
     def save_state(self):
@@ -85,7 +102,7 @@ class CacheStorage:
         total = 0
         for l in self._layers.values():
             if isinstance(l, PagedKVLayer):
-                total += l.k.numel() * l.k.element_size() * 2
+                total += sum(t.numel() * t.element_size() for t in l.tensors.values())
             elif isinstance(l, StateLayer):
                 total += l.state.numel() * l.state.element_size()
         return total
@@ -95,5 +112,5 @@ class CacheStorage:
         total = 0
         for l in self._layers.values():
             if isinstance(l, PagedKVLayer):
-                total += 2 * l.k.shape[1] * l.k.shape[3] * l.k.element_size()
+                total += sum(t[0].numel() * t.element_size() for t in l.tensors.values()) // l.page_size
         return total

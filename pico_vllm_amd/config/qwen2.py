@@ -48,4 +48,16 @@ def qwen2_spec(cfg: Qwen2Config) -> ModelSpec:
     )
 
 
-register_architecture("Qwen2ForCausalLM", Qwen2Config.from_dict, qwen2_spec)
+def qwen2_sizes(cfg: Qwen2Config) -> dict:
+    """The sizes of a configuration as a flat record (for a benchmark's report)."""
+    return {"layers": cfg.num_hidden_layers, "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size,
+            "vocab": cfg.vocab_size, "tied": cfg.tie_word_embeddings}
+
+
+def qwen2_with_layers(raw: dict, layers: int) -> dict:
+    """The same layer sizes with ``layers`` layers (a measurement that memory or time limits to fewer)."""
+    return dict(raw, num_hidden_layers=layers)
+
+
+register_architecture("Qwen2ForCausalLM", Qwen2Config.from_dict, qwen2_spec, qwen2_sizes, qwen2_with_layers)

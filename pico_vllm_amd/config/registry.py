@@ -7,7 +7,7 @@ directly (pico_vllm/run_single.py:2,10-11).
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict
+from typing import Any, Callable, Dict, Optional
 
 from .model_config import ConfigError, read_config_json
 
@@ -17,13 +17,16 @@ class Architecture:
     name: str
     config_from_dict: Callable[[Dict[str, Any]], Any]   # raw config.json -> typed config
     build_spec: Callable[[Any], Any]                     # typed config -> parts.spec.ModelSpec
+    # for reports and measurements, so that the programs that make them read no architecture's keys:
+    sizes: Optional[Callable[[Any], Dict[str, Any]]] = None          # typed config -> flat {name: number} of its sizes
+    with_layers: Optional[Callable[[Dict[str, Any], int], Dict[str, Any]]] = None   # raw config, n -> the same layer sizes, n layers
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_from_dict, build_spec) -> Architecture:
-    arch = Architecture(name, config_from_dict, build_spec)
+def register_architecture(name: str, config_from_dict, build_spec, sizes=None, with_layers=None) -> Architecture:
+    arch = Architecture(name, config_from_dict, build_spec, sizes, with_layers)
     _ARCHITECTURES[name] = arch
     return arch
 

@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 
+from ..cache.storage import bytes_per_page
 from ..config.engine_args import EngineArgs
 from ..ops import linear
 from ..parts.model import DecoderModel, load_model
@@ -56,14 +57,15 @@ class LLMEngine:
             # second engine does not change what the first one runs
             linear.set_library_tuning(True)
         num_pages = args.num_gpu_blocks
+        self.pool_sizing = {"pages": num_pages, "from": "num_gpu_blocks"}
         if num_pages is None:
-            num_pages = args.max_num_seqs * (-(-args.max_seq_len // args.block_size))
+            num_pages, self.pool_sizing = self._pages_from_memory(args)
         self.runner = ModelRunner(self.model, args.block_size, num_pages, args.max_num_seqs,
                                   args.max_num_batched_tokens, args.max_seq_len,
                                   use_graph=args.use_cuda_graph, max_graph_batch=args.max_batch_size,
                                   graph_prompts=args.graph_prompts)
         self.scheduler = Scheduler(self.runner.manager, args.max_num_seqs, args.max_num_batched_tokens,
-                                   args.max_seq_len)
+                                   args.max_seq_len, args.prefill_chunk)
         self.sampler = Sampler(self.model.device, args.max_num_seqs)
         self.eos_token_id = self.model.spec.eos_token_id
         if self.eos_token_id is None and tokenizer is not None:     # the reference's source for it, pico_vllm/engine.py:48
@@ -75,6 +77,24 @@ class LLMEngine:
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
         self.timers = PhaseTimers(args.profile_phases)
         self._inflight: Optional[_Inflight] = None      # a launched step whose tokens have not been read
+
+    def _pages_from_memory(self, args: EngineArgs):
+        """Pages per group when ``num_gpu_blocks`` is not given: as many as ``max_num_seqs`` requests of ``max_seq_len``
+        can use at once (more would never be touched), or fewer if ``kv_memory_fraction`` of the GPU memory that is free
+        now, with the weights loaded, does not hold that many.  (The reference fixes 500 blocks in its script,
+        pico_vllm/run_single.py:17-22.)  Returns (pages, how they were found, for ``report()``)."""
+        want = args.max_num_seqs * (-(-args.max_seq_len // args.block_size))
+        per_page = bytes_per_page(self.model.cache_specs(), args.block_size, self.model.dtype)
+        free, total = torch.cuda.mem_get_info(self.model.device)
+        fit = int(free * args.kv_memory_fraction) // per_page if per_page else want
+        pages = max(1, min(want, fit))
+        sizing = {"pages": pages, "from": "memory" if fit < want else "max_num_seqs * max_seq_len", "wanted": want,
+                  "fit": fit, "bytes_per_page": per_page, "free_bytes": int(free), "kv_memory_fraction": args.kv_memory_fraction}
+        if pages * args.block_size < args.max_seq_len:
+            raise ValueError(f"the GPU has {free / 2**30:.1f} GiB free, of which {args.kv_memory_fraction:.0%} hold {fit} cache pages "
+                             f"of {args.block_size} tokens ({per_page} bytes each over all layers): not one request of "
+                             f"max_seq_len = {args.max_seq_len}; lower max_seq_len or give num_gpu_blocks")
+        return pages, sizing
 
     # ---- the reference's trio -------------------------------------------
     def submit(self, prompt: Union[str, Sequence[int]], max_new_tokens: int = 16, temperature: float = 0.0,
@@ -220,6 +240,7 @@ class LLMEngine:
         out: Dict[str, object] = dict(self.stats)
         out["pages"] = [{"window": g.window, "layers": len(g.layers), "total": g.pool.num_pages, "in_use": g.pool.num_used,
                          "peak": g.pool.peak_used, "reused": g.pool.reuse_count} for g in m.groups]
+        out["pool_sizing"] = dict(self.pool_sizing)      # how the number of pages was found (given, or from the free memory)
         out["graphs"] = sorted(self.runner._graphs)
         out["prompt_graphs"] = sorted((key[0], key[1]) for key in self.runner._prompt_graphs)   # (single tokens, portion)
         if self.timers.enabled:

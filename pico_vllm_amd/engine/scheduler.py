@@ -3,7 +3,7 @@
 First come, first served, as in the reference (pico_vllm/scheduler.py:174-178:
 ``waiting.pop(0)`` while fewer than ``max_num_seqs`` are in progress).  What
 the reference does not have: a token budget per step with prompts cut into
-portions (it prefills whole prompts, engine.py:305-306), admission that looks
+portions of at most ``prefill_chunk`` tokens (it prefills whole prompts, engine.py:305-306), admission that looks
 at free pages (its ``can_allocate_gpu`` is unused, blockmanager.py:173-176),
 and a decision for the moment pages run out (there the allocation raises from
 inside the step, blockmanager.py:77-78).
@@ -18,7 +18,7 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, List
+from typing import Deque, List, Optional
 
 from ..cache.manager import CacheManager
 from .request import Request, RequestStatus
@@ -47,12 +47,16 @@ class SchedulerOutput:
 
 class Scheduler:
     def __init__(self, manager: CacheManager, max_num_seqs: int = 4, max_num_batched_tokens: int = 2048,
-                 max_seq_len: int = 4096):
+                 max_seq_len: int = 4096, prefill_chunk: Optional[int] = None):
         if max_num_batched_tokens < max_num_seqs:
             raise ValueError("max_num_batched_tokens must be at least max_num_seqs, or decoding requests starve")
+        if prefill_chunk is not None and prefill_chunk < 1:
+            raise ValueError("prefill_chunk must be positive")
         self.manager = manager
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens
+        # the longest portion of one prompt in a step (beside the budget, which all sequences of a step share)
+        self.prefill_chunk = min(prefill_chunk or max_num_batched_tokens, max_num_batched_tokens)
         self.max_seq_len = max_seq_len
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []          # in order of admission
@@ -72,7 +76,7 @@ class Scheduler:
             if g.window > 0:
                 # a group with a window holds the window and the step's own tokens, whatever the length: pages that
                 # the window has passed went back before the step
-                pages = min(pages, -(-(g.window + self.max_num_batched_tokens) // P) + 1)
+                pages = min(pages, -(-(g.window + self.prefill_chunk) // P) + 1)
             if pages > g.pool.num_pages:
                 raise ValueError(f"request {req.request_id} needs {pages} pages at its longest; the pool has "
                                  f"{g.pool.num_pages}, so it could never finish")
@@ -91,7 +95,7 @@ class Scheduler:
         for req in order:
             if req.status is not RequestStatus.RUNNING or budget <= 0:
                 continue
-            n = min(req.num_uncomputed, budget)
+            n = min(req.num_uncomputed, budget, self.prefill_chunk)
             while not self.manager.grow(req.request_id, req.num_computed + n):
                 victim = self.running[-1]
                 self._preempt(victim, out)
@@ -106,7 +110,7 @@ class Scheduler:
         # 2. admit waiting requests in order while everything they need is there
         while self.waiting and len(self.running) < self.max_num_seqs and budget > 0 and not out.preempted:
             req = self.waiting[0]
-            n = min(req.num_uncomputed, budget)
+            n = min(req.num_uncomputed, budget, self.prefill_chunk)
             if not self.manager.add_request(req.request_id):
                 break
             if not self.manager.grow(req.request_id, n):

@@ -11,7 +11,15 @@ from ..ops import kernels
 from ..ops.linear import Linear
 from .base import DeferredNorm, Mixer, StepContext
 from .registry import build_part, register_part
-from .spec import CacheSpec, ParamSpec, PartSpec
+from .spec import CacheSpec, PageTensor, ParamSpec, PartSpec
+
+
+def kv_page_tensors(num_kv_heads: int, head_dim: int):
+    """The layout of a page that this package's attention and store kernels read and write: in ``k`` a token's key
+    is contiguous ([kv heads, page, head size]); in ``v`` a head dimension's values of the page's tokens are
+    ([kv heads, head size, page]: the matrix-core kernels contract over keys).  The reference keeps V like K
+    (pico_vllm/blockmanager.py:39-42)."""
+    return (PageTensor("k", (num_kv_heads, "page", head_dim)), PageTensor("v", (num_kv_heads, head_dim, "page")))
 
 
 @register_part("mixer", "gqa_attention")
@@ -50,7 +58,11 @@ class GQAAttention(Mixer):
         self.fast = None                                # matrix-core kernels, chosen at load
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec("paged_kv", num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
+        return CacheSpec("paged_kv", window=self.window, page_tensors=kv_page_tensors(self.nkv, self.d))
+
+    def flops(self, tokens: int, pairs: int) -> float:
+        # the projections, and q.k and p.v for every (query, key) pair of every head
+        return super().flops(tokens, pairs) + 4.0 * self.nq * self.d * pairs
 
     def param_specs(self) -> List[ParamSpec]:
         H, nq, nkv, d = self.hidden_size, self.nq, self.nkv, self.d

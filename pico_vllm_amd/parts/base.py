@@ -13,6 +13,7 @@ Interfaces:
   Mixer.cache_spec() -> CacheSpec;  Mixer.forward(x, ctx, cache) -> y
   FeedForward.forward(x, ctx) -> y
   Block.forward(resid, pending, ctx, cache) -> (resid, pending)
+  StreamPart.forward(resid, ctx) -> resid
 """
 from __future__ import annotations
 
@@ -93,6 +94,41 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor], device: torch.device, dtype: torch.dtype) -> None:
         pass
 
+    # ---- sizes for reports (the benchmark's roofline) ---------------------
+    def _members(self):
+        """Sub-parts and matrices this part holds: its attributes, and what lists, tuples and dicts among
+        them hold (experts in a list, say)."""
+        from ..ops.linear import Linear
+
+        def walk(v, depth=0):
+            if isinstance(v, (Part, Linear)):
+                yield v
+            elif depth < 3 and isinstance(v, (list, tuple)):
+                for x in v:
+                    yield from walk(x, depth + 1)
+            elif depth < 3 and isinstance(v, dict):
+                for x in v.values():
+                    yield from walk(x, depth + 1)
+        for v in vars(self).values():
+            yield from walk(v)
+
+    def weight_bytes(self) -> int:
+        """Bytes of the matrices a step streams through this part: its ``Linear``s and its sub-parts',
+        wherever they are kept.  A part that reads only some of them per step (experts that no token of the
+        step was routed to) still counts all: the figure is what a full batch reads."""
+        from ..ops.linear import Linear
+        return sum(m.weight.numel() * m.weight.element_size() if isinstance(m, Linear) else m.weight_bytes()
+                   for m in self._members())
+
+    def flops(self, tokens: int, pairs: int) -> float:
+        """Floating-point operations of a step with ``tokens`` new tokens and ``pairs`` (query, key) pairs that
+        attention looks at (a prompt of T tokens alone: T (T + 1) / 2): two per weight and token for the matrices
+        of this part and its sub-parts; a part with other work (attention's scores) adds its own.  A part that
+        runs only some of its matrices per token (routing) overrides this."""
+        from ..ops.linear import Linear
+        return sum(2.0 * tokens * m.weight.numel() if isinstance(m, Linear) else m.flops(tokens, pairs)
+                   for m in self._members())
+
 
 class DeferredNorm:
     """A norm whose operands are known but which has not run: ``resid_in + delta`` normed.  A block hands
@@ -125,6 +161,15 @@ class Norm(Part):
         with ``rows`` only those rows are produced and resid is left unchanged.  delta is
         [T, H] in the activation dtype or float32, or a float32 stack [S, T, H] of partial
         sums (what ``ops.linear.Linear.partial`` returns), all of which are added."""
+        raise NotImplementedError
+
+
+class StreamPart(Part):
+    """A part that works on the residual stream outside the layers (``ModelSpec.before_layers`` /
+    ``after_layers``): learned absolute positions added to the embeddings, a norm of the embeddings."""
+
+    def forward(self, resid: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
+        """resid: float32 [T, H], the residual stream (with nothing pending); returns it (changed in place or anew)."""
         raise NotImplementedError
 
 

@@ -46,6 +46,9 @@ def model_param_specs(spec: ModelSpec) -> List[ParamSpec]:
     for lspec in spec.layers:
         blk, sub = _build_layer(lspec, torch.float32)
         out += [p for _, _, p in _layer_params(lspec, blk, sub)]
+    for prefix, pspec in tuple(spec.before_layers) + tuple(spec.after_layers):
+        part = build_part("stream", pspec, act_dtype=torch.float32)
+        out += [ParamSpec(f"{prefix}.{p.name}" if prefix else p.name, p.shape, p.role, p.std) for p in part.param_specs()]
     fn = build_part("norm", spec.final_norm, act_dtype=torch.float32)
     out += [ParamSpec(f"{spec.final_norm_name}.{p.name}", p.shape, p.role, p.std) for p in fn.param_specs()]
     if spec.head_name:
@@ -56,7 +59,7 @@ def model_param_specs(spec: ModelSpec) -> List[ParamSpec]:
 
 
 class DecoderModel:
-    """embedding (times ``spec.embed_scale``) -> layers in ``run_order`` -> final norm on the wanted rows ->
+    """embedding (times ``spec.embed_scale``) -> ``spec.before_layers`` -> layers in ``run_order`` -> ``spec.after_layers`` -> final norm on the wanted rows ->
     output matrix (+ ``spec.head_bias_name``, soft cap ``spec.logit_softcap``) (pico_vllm/model.py:427-445; the
     reference's model has no multiplier, bias or cap: 1, none and 0 here).  Logits are float32 and exist
     only for the wanted rows (the reference computes all rows and keeps the
@@ -72,6 +75,9 @@ class DecoderModel:
             self.layers.append(blk)
             self._sub.append(sub)
         self.final_norm = build_part("norm", spec.final_norm, act_dtype=dtype)
+        # what stands around the layers on the residual stream: (prefix, part)
+        self.before = [(pre, build_part("stream", ps, act_dtype=dtype)) for pre, ps in spec.before_layers]
+        self.after = [(pre, build_part("stream", ps, act_dtype=dtype)) for pre, ps in spec.after_layers]
         self.embed: Optional[torch.Tensor] = None
         self.head: Optional[Linear] = None
         for i, e in enumerate(spec.run_order):
@@ -98,6 +104,9 @@ class DecoderModel:
             for slot, part in blk.parts.items():
                 pre = f"{lspec.prefix}.{sub[slot]}."
                 part.load({p.name: tensors[pre + p.name] for p in part.param_specs()}, dev, self.dtype)
+        for prefix, part in self.before + self.after:
+            pre = prefix + "." if prefix else ""
+            part.load({p.name: tensors[pre + p.name] for p in part.param_specs()}, dev, self.dtype)
         pre = spec.final_norm_name + "."
         self.final_norm.load({p.name: tensors[pre + p.name] for p in self.final_norm.param_specs()}, dev, self.dtype)
         self.head = Linear(tensors[spec.head_name].to(dev) if spec.head_name else self.embed,
@@ -106,7 +115,10 @@ class DecoderModel:
     def is_graph_safe(self, prompts: bool = False) -> bool:
         """Whether a decode step (``prompts``: a padded prompt step) of this model may be recorded into a HIP
         graph: every part says so."""
-        return all(blk.is_graph_safe(prompts) for blk in self.layers) and self.final_norm.is_graph_safe(prompts)
+        return all(p.is_graph_safe(prompts) for p in self._all_parts())
+
+    def _all_parts(self):
+        return self.layers + [self.final_norm] + [p for _, p in self.before + self.after]
 
     def graph_variant(self, ctx) -> tuple:
         """The host-side choices of all parts for this step, each distinct one once (layers of one kind choose
@@ -119,15 +131,18 @@ class DecoderModel:
         return tuple(seen)
 
     def num_weight_bytes(self) -> int:
-        """Bytes a decode step streams: every matrix once (the embedding table only as the
-        output matrix when tied)."""
+        """Bytes of matrices a decode step streams: what every part reports (``Part.weight_bytes``), a layer as often
+        as the run order names it, and the output matrix (the embedding table only as that, when tied)."""
         total = self.head.weight.numel() * self.head.weight.element_size()
-        for blk in self.layers:
-            for part in blk.parts.values():
-                for v in vars(part).values():
-                    if isinstance(v, Linear):
-                        total += v.weight.numel() * v.weight.element_size()
-        return total
+        total += sum(self.layers[e.layer].weight_bytes() for e in self.spec.run_order)
+        return total + sum(p.weight_bytes() for _, p in self.before + self.after) + self.final_norm.weight_bytes()
+
+    def flops(self, tokens: int, pairs: int, wanted_rows: int) -> float:
+        """Floating-point operations of a step of ``tokens`` new tokens whose attention looks at ``pairs`` (query,
+        key) pairs, with logits at ``wanted_rows`` rows: the sum of what the parts report (``Part.flops``)."""
+        total = 2.0 * wanted_rows * self.head.weight.numel()
+        total += sum(self.layers[e.layer].flops(tokens, pairs) for e in self.spec.run_order)
+        return total + sum(p.flops(tokens, pairs) for _, p in self.before + self.after)
 
     def forward(self, ctx: StepContext, storage) -> torch.Tensor:
         """Logits float32 [R, V] at ctx.want_rows."""
@@ -137,6 +152,8 @@ class DecoderModel:
     def _forward(self, ctx: StepContext, storage) -> torch.Tensor:
         ctx.shared.clear()      # what layers share belongs to this pass (a context may be run again, as at graph capture)
         resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens], scale=self.spec.embed_scale)
+        for _, part in self.before:
+            resid = part.forward(resid, ctx)
         pending = None
         for i, e in enumerate(self.spec.run_order):
             # a run that names another run's cache reads it and stores nothing of its own
@@ -144,6 +161,13 @@ class DecoderModel:
                                                           storage.layer(self.spec.cache_id(i), read_only=e.cache_of is not None))
         if ctx.want_rows.numel() == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+        if self.after:
+            if pending is not None:            # these parts see the whole stream: the last layer's delta joins it first
+                for delta in (pending if pending.dim() == 3 else (pending,)):       # a stack of partial sums: each in turn
+                    kernels.residual_add(resid, delta)
+                pending = None
+            for _, part in self.after:
+                resid = part.forward(resid, ctx)
         h = self.final_norm.add_norm(resid, pending, rows=ctx.want_rows)
         logits = self.head(h, out_dtype=torch.float32)
         if self.spec.logit_softcap > 0:

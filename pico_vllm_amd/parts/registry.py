@@ -1,6 +1,6 @@
 """Registries: a part kind (a string in a ``PartSpec``) to the class that
 builds it, one registry per category.  A new mixer, feed-forward, norm,
-position encoding or block arrangement is added by registering a class; the
+position encoding, block arrangement or part around the layers ("stream") is added by registering a class; the
 model builder, the cache manager and the step function only see the
 interfaces in ``parts.base``.
 """
@@ -8,7 +8,7 @@ from __future__ import annotations
 
 from typing import Callable, Dict
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "stream")
 _REGISTRY: Dict[str, Dict[str, Callable]] = {c: {} for c in CATEGORIES}
 
 

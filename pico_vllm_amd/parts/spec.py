@@ -8,7 +8,7 @@ from it through the part registries in ``parts.registry``.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, List, Optional, Tuple, Union
 
 
 @dataclass(frozen=True)
@@ -35,21 +35,49 @@ class ParamSpec:
 
 
 @dataclass(frozen=True)
+class PageTensor:
+    """One tensor that a paged cache keeps for every page.  ``shape`` is that of ONE page; the string
+    "page" in it stands for the number of tokens a page holds (an engine option, not the part's).
+    ``dtype``: a torch dtype by name, or None for the engine's."""
+    name: str
+    shape: Tuple[Union[int, str], ...]
+    dtype: Optional[str] = None
+
+    def resolved(self, page_size: int) -> Tuple[int, ...]:
+        out = []
+        for s in self.shape:
+            if s == "page":
+                out.append(page_size)
+            elif isinstance(s, int) and s > 0:
+                out.append(s)
+            else:
+                raise ValueError(f"page tensor {self.name!r}: a dimension is a positive int or 'page', got {s!r}")
+        return tuple(out)
+
+
+@dataclass(frozen=True)
 class CacheSpec:
     """What a mixer keeps per request between steps.
 
-    kind "paged_kv": keys and values of ``num_kv_heads`` x ``head_dim`` per
-    token in pages; ``window`` > 0 means only the last ``window`` positions
-    are ever read again, so older pages can be given back early.
+    kind "paged_kv": what ``page_tensors`` lists, per page of tokens (the mixer names the tensors
+    and their layout inside a page; the cache only allocates them, one allocation a tensor and
+    layer, and hands them to the mixer by name); ``window`` > 0 means only the last ``window``
+    positions are ever read again, so older pages can be given back early.
     kind "state": a fixed-size tensor of ``state_shape`` per request.
     kind "none": nothing.
+    Layers with equal specs share a pool of page ids and a block table per request.
     """
     kind: str = "none"
-    num_kv_heads: int = 0
-    head_dim: int = 0
     window: int = 0
+    page_tensors: Tuple[PageTensor, ...] = ()
     state_shape: Tuple[int, ...] = ()
     state_dtype: str = "float32"
+
+    def __post_init__(self):
+        if self.kind == "paged_kv":
+            names = [t.name for t in self.page_tensors]
+            if not names or len(set(names)) != len(names):
+                raise ValueError("a paged cache needs page tensors with distinct names")
 
 
 @dataclass(frozen=True)
@@ -88,6 +116,10 @@ class ModelSpec:
     # names (shell patterns allowed) of tensors a checkpoint may hold that the model does not use: a tied model's
     # stored output matrix, buffers that another implementation keeps in its files
     ignored_tensors: Tuple[str, ...] = ()
+    # parts that run on the residual stream before the first and after the last layer (category "stream":
+    # learned absolute positions, a norm of the embeddings): (prefix of the part's tensors, the part)
+    before_layers: Tuple[Tuple[str, PartSpec], ...] = ()
+    after_layers: Tuple[Tuple[str, PartSpec], ...] = ()
     embed_scale: float = 1.0          # the embedding rows are multiplied by this (1: as they are)
     logit_softcap: float = 0.0        # > 0: logits = cap * tanh(logits / cap)
     head_bias_name: Optional[str] = None   # a bias [vocab] added to the logits

@@ -30,7 +30,11 @@ def main(argv=None) -> int:
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--block-size", type=int, default=16)
-    ap.add_argument("--num-gpu-blocks", type=int, default=500)
+    ap.add_argument("--num-gpu-blocks", type=lambda v: None if v == "auto" else int(v), default=500,
+                    help="cache pages per group of layers (the reference's 500), or 'auto': what --max-num-seqs requests of "
+                         "--max-seq-len can use, within --kv-memory-fraction of the free GPU memory")
+    ap.add_argument("--kv-memory-fraction", type=float, default=0.9)
+    ap.add_argument("--prefill-chunk", type=int, default=None, help="longest portion of one prompt in a step (default: the step's budget)")
     ap.add_argument("--max-seq-len", type=int, default=4096)
     ap.add_argument("--max-num-seqs", type=int, default=4)
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
@@ -96,6 +100,7 @@ def _generate(ap, args) -> int:
     ea = EngineArgs(model=args.model, dtype=args.dtype, block_size=args.block_size,
                     num_gpu_blocks=args.num_gpu_blocks, max_seq_len=args.max_seq_len,
                     max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
+                    prefill_chunk=args.prefill_chunk, kv_memory_fraction=args.kv_memory_fraction,
                     use_cuda_graph=args.use_cuda_graph, max_batch_size=args.max_batch_size,
                     manual_seed=args.manual_seed, pipeline_decode=args.pipeline_decode, profile_phases=args.profile_phases)
     llm = LLM(tokenizer=tokenizer, engine_args=ea)

@@ -5,10 +5,11 @@ import torch
 
 from pico_vllm_amd.cache.manager import CacheManager
 from pico_vllm_amd.engine.batch import BatchBuffers, BatchError, SeqStep, build_context
+from pico_vllm_amd.parts.attention import kv_page_tensors
 from pico_vllm_amd.parts.spec import CacheSpec
 
-FULL = CacheSpec("paged_kv", num_kv_heads=1, head_dim=16)
-WIN = CacheSpec("paged_kv", num_kv_heads=1, head_dim=16, window=12)
+FULL = CacheSpec("paged_kv", page_tensors=kv_page_tensors(1, 16))
+WIN = CacheSpec("paged_kv", window=12, page_tensors=kv_page_tensors(1, 16))
 P, VOCAB = 8, 100
 
 

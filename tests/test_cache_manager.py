@@ -5,10 +5,11 @@ import pytest
 
 from pico_vllm_amd.cache.manager import CacheManager
 from pico_vllm_amd.cache.page_pool import PagePool, PagePoolError, StateSlots
+from pico_vllm_amd.parts.attention import kv_page_tensors
 from pico_vllm_amd.parts.spec import CacheSpec
 
-FULL = CacheSpec("paged_kv", num_kv_heads=2, head_dim=16)
-WIN = CacheSpec("paged_kv", num_kv_heads=2, head_dim=16, window=20)
+FULL = CacheSpec("paged_kv", page_tensors=kv_page_tensors(2, 16))
+WIN = CacheSpec("paged_kv", window=20, page_tensors=kv_page_tensors(2, 16))
 STATE = CacheSpec("state", state_shape=(4,))
 
 

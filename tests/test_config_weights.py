@@ -94,6 +94,10 @@ def test_engine_args_validate():
         EngineArgs(dtype="float16").validate()
     with pytest.raises(ValueError):
         EngineArgs(block_size=12).validate()
+    for bad in (dict(prefill_chunk=0), dict(num_gpu_blocks=0), dict(kv_memory_fraction=0.0), dict(kv_memory_fraction=1.5)):
+        with pytest.raises(ValueError, match=next(iter(bad))):
+            EngineArgs(**bad).validate()
+    EngineArgs(prefill_chunk=512, num_gpu_blocks=10, kv_memory_fraction=1.0).validate()
 
 
 # ---- safetensors -----------------------------------------------------------
@@ -312,7 +316,7 @@ def test_parts_are_found_by_category_and_kind_and_unknown_ones_are_named():
         register_part("router", "top2")
     with pytest.raises(KeyError, match="no router part"):
         part_class("router", "top2")
-    assert set(CATEGORIES) == {"mixer", "feed_forward", "norm", "position", "block"}
+    assert set(CATEGORIES) == {"mixer", "feed_forward", "norm", "position", "block", "stream"}
 
 
 def test_parts_refuse_sizes_that_make_no_sense_when_they_are_built():

@@ -347,6 +347,28 @@ def test_what_generate_and_the_step_refuse_and_the_defaults_they_fall_back_to():
     eng = LLM(model=model_dir("A"), dtype="float32", block_size=16, max_seq_len=100, max_num_seqs=3, max_num_batched_tokens=64,
               use_cuda_graph=False)
     assert eng.engine.runner.manager.groups[0].pool.num_pages == 3 * 7
+    sizing = eng.engine.report()["pool_sizing"]
+    assert sizing["pages"] == 21 == sizing["wanted"] and sizing["from"] == "max_num_seqs * max_seq_len" and sizing["fit"] > 21
+    # 2 layers x (k and v) x 1 kv head x 16 x 16 tokens x 4 bytes
+    assert sizing["bytes_per_page"] == 2 * 2 * 16 * 16 * 4
+    # ... or as many as a share of the free memory holds, when that is fewer; none for a whole request is refused
+    free = torch.cuda.mem_get_info()[0]
+    share = 40.5 * sizing["bytes_per_page"] / free
+    small = LLM(model=model_dir("A"), dtype="float32", block_size=16, max_seq_len=100, max_num_seqs=30, max_num_batched_tokens=64,
+                use_cuda_graph=False, kv_memory_fraction=share)
+    sizing = small.engine.report()["pool_sizing"]
+    assert sizing["from"] == "memory" and sizing["wanted"] == 210 and 30 <= sizing["pages"] <= 41
+    assert small.engine.runner.manager.groups[0].pool.num_pages == sizing["pages"]
+    with pytest.raises(ValueError, match="not one request of max_seq_len"):
+        LLM(model=model_dir("A"), dtype="float32", block_size=16, max_seq_len=100, max_num_seqs=30, max_num_batched_tokens=64,
+            use_cuda_graph=False, kv_memory_fraction=3.5 * sizing["bytes_per_page"] / free)
+    # portions of a prompt capped beside the budget
+    capped = LLM(model=model_dir("A"), dtype="float32", block_size=16, max_seq_len=100, max_num_seqs=3, max_num_batched_tokens=64,
+                 use_cuda_graph=False, prefill_chunk=7)
+    prompts = prompts_for("A", [30, 9], seed=2)
+    outs = capped.generate(prompts, SamplingParams(max_new_tokens=5, ignore_eos=True))
+    assert capped.engine.stats["steps"] >= 5 + 4                       # 30 tokens in portions of at most 7
+    check_greedy("A", "float32", prompts, outs)
     prompts = prompts_for("A", [5, 9], seed=2)
     outs = eng.generate(prompts)                                       # no options given: greedy, 16 tokens at most
     assert all(1 <= len(o.token_ids) <= 16 for o in outs)

@@ -460,6 +460,7 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(dtype):
     from pico_vllm_amd.engine.batch import SeqStep
     from pico_vllm_amd.engine.step import ModelRunner
     from pico_vllm_amd.ops import kernels
+    from pico_vllm_amd.ops.linear import Linear
     from pico_vllm_amd.parts.base import FeedForward, PositionEncoding
     from pico_vllm_amd.parts.model import load_model
     from pico_vllm_amd.parts.registry import register_part
@@ -496,8 +497,16 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(dtype):
 
         def load(self, tensors, device, dtype):
             self.router = tensors["router.weight"].to(device).float()
-            self.w_in = [tensors[f"experts.{e}.in.weight"].to(device) for e in range(self.E)]
-            self.w_out = [tensors[f"experts.{e}.out.weight"].to(device) for e in range(self.E)]
+            # the experts' matrices in lists: what the part reports as streamed bytes finds them there
+            self.w_in = [Linear(tensors[f"experts.{e}.in.weight"].to(device)) for e in range(self.E)]
+            self.w_out = [Linear(tensors[f"experts.{e}.out.weight"].to(device)) for e in range(self.E)]
+
+        def weight_bytes(self):
+            return super().weight_bytes() + self.router.numel() * self.router.element_size()
+
+        def flops(self, tokens, pairs):
+            # the router for every token, and the one expert it chose: not what the default counts (every matrix)
+            return 2.0 * tokens * (self.E * self.H + 2 * self.I * self.H)
 
         def forward(self, x, ctx):
             choice = (x.float() @ self.router.T).argmax(-1)            # router logits in float32
@@ -505,8 +514,8 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(dtype):
             for e in range(self.E):
                 rows = (choice == e).nonzero().flatten()
                 if rows.numel():
-                    h = torch.relu(x[rows] @ self.w_in[e].T)
-                    out[rows] = h @ self.w_out[e].T
+                    h = torch.relu(x[rows] @ self.w_in[e].weight.T)
+                    out[rows] = h @ self.w_out[e].weight.T
             return out
 
     def toy_spec(cfg):
@@ -528,6 +537,15 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(dtype):
         model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
         r = ModelRunner(model, 8, 16, 3, 64, 64)
         toks = torch.randint(0, V, (43,), generator=torch.Generator().manual_seed(1)).tolist()
+        # what a step streams and computes is asked of the parts: all three experts' matrices and the router, the dense
+        # feed-forward of the other layer, both attentions, the tied output matrix
+        size = 4 if dtype == torch.float32 else 2
+        attn_w = (NQ + 2 * NKV) * D * H + H * NQ * D
+        assert model.num_weight_bytes() == size * (2 * attn_w + E * 2 * I * H + 3 * I * H + V * H) + 4 * E * H
+        assert r.decode_bytes([10, 5]) == model.num_weight_bytes() + 15 * 2 * (2 * NKV * D * size)
+        T, pairs = 7, 7 * 8 // 2
+        assert model.flops(T, pairs, 2) == 2.0 * T * (2 * attn_w + (E * H + 2 * I * H) + 3 * I * H) \
+            + 2 * 4.0 * NQ * D * pairs + 2.0 * 2 * V * H
 
         # the plain computation, whole sequence, no cache
         def plain(rnd):
@@ -1007,3 +1025,113 @@ def test_a_toy_norm_and_a_toy_arrangement_of_the_parts(dtype):
             outs.append([o.token_ids for o in llm.generate([toks[:9], toks[5:20]], SamplingParams(max_new_tokens=6, temperature=0.0))])
             del llm
         assert outs[0] == outs[1]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_parts_around_the_layers_learned_positions_in_front_and_a_gain_behind(dtype):
+    """``ModelSpec.before_layers`` / ``after_layers``: parts of the category "stream" that work on the residual stream
+    outside the layers, defined and registered here: learned absolute positions added to the embeddings (a table of the
+    checkpoint, looked up by ``ctx.positions``) and a gain per channel behind the last layer.  The attention layers carry
+    no position encoding, so positions reach the logits through the table alone.  Portions, single tokens (recorded
+    steps too) and the whole prompt against the plain computation."""
+    import dataclasses
+    import tempfile
+    from pico_vllm_amd.config.model_config import Qwen2Config
+    from pico_vllm_amd.config.qwen2 import qwen2_spec
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.base import StreamPart
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import LayerSpec, ParamSpec, PartSpec
+    from pico_vllm_amd.weights.random_init import write_random_model
+    from tiny_configs import TINY_A, strong
+
+    @register_part("stream", "toy_learned_positions")
+    class LearnedPositions(StreamPart):
+        graph_safe_prompts = True
+
+        def __init__(self, size, most, act_dtype=torch.bfloat16):
+            self.size, self.most = size, most
+
+        def param_specs(self):
+            return [ParamSpec("weight", (self.most, self.size), std=0.5)]
+
+        def load(self, tensors, device, dtype):
+            self.table = tensors["weight"].to(device).float()
+
+        def forward(self, resid, ctx):
+            T = resid.shape[0]
+            resid += self.table.index_select(0, ctx.positions[:T].long())       # device work only: may be recorded
+            return resid
+
+    @register_part("stream", "toy_gain")
+    class Gain(StreamPart):
+        graph_safe_prompts = True
+
+        def __init__(self, size, act_dtype=torch.bfloat16):
+            self.size = size
+
+        def param_specs(self):
+            return [ParamSpec("weight", (self.size,), role="norm")]
+
+        def load(self, tensors, device, dtype):
+            self.gain = tensors["weight"].to(device).float()
+
+        def forward(self, resid, ctx):
+            return resid * self.gain
+
+    MOST = 96
+
+    def spec_with_parts_around(cfg):
+        spec = qwen2_spec(cfg)
+        layers = []
+        for l in spec.layers:
+            name, attn = l.slots["mixer"]
+            layers.append(LayerSpec(l.prefix, l.block, {**l.slots, "mixer": (name, PartSpec(attn.kind, dict(attn.params, position=PartSpec("none", {}))))}))
+        return dataclasses.replace(spec, layers=layers,
+                                   before_layers=(("model.wpe", PartSpec("toy_learned_positions", {"size": cfg.hidden_size, "most": MOST})),),
+                                   after_layers=(("model.out_gain", PartSpec("toy_gain", {"size": cfg.hidden_size})),))
+    register_architecture("ToyLearnedPositionsLM", Qwen2Config.from_dict, spec_with_parts_around)
+    cfg = dict(TINY_A, architectures=["ToyLearnedPositionsLM"])
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=21, std_overrides=strong(cfg))
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        plain = P.PlainModel(d)
+        w, c = plain.w, plain.cfg
+        assert w["model.wpe.weight"].shape == (MOST, c.hidden_size) and w["model.out_gain.weight"].shape == (c.hidden_size,)
+
+        def want(toks, rnd, first=0):
+            nq, nkv, hd = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+            x = w["model.embed_tokens.weight"][toks].float() + w["model.wpe.weight"][first:first + len(toks)]
+            for i in range(c.num_hidden_layers):
+                p = f"model.layers.{i}"
+                h = rnd(P.rms_norm(x, w[f"{p}.input_layernorm.weight"], c.rms_norm_eps))
+                Wm = torch.cat([w[f"{p}.self_attn.{n}_proj.weight"] for n in "qkv"])
+                b = torch.cat([w[f"{p}.self_attn.{n}_proj.bias"] for n in "qkv"])
+                q, k, v = P.split_qkv(rnd(h @ Wm.T + b), nq, nkv, hd)
+                o = rnd(P.causal_attention(q, k, v, rnd_p=None if rnd is P._same else rnd))
+                x = x + rnd(o.reshape(len(toks), nq * hd) @ w[f"{p}.self_attn.o_proj.weight"].T)
+                x = x + P.mlp_layer(rnd(P.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], c.rms_norm_eps)), w, p, rnd)
+            x = x * w["model.out_gain.weight"]
+            return rnd(P.rms_norm(x, w["model.norm.weight"], c.rms_norm_eps)) @ w["model.embed_tokens.weight"].T
+        toks = torch.randint(0, 255, (70,), generator=torch.Generator().manual_seed(6)).tolist()
+        exact = want(toks, P._same)
+        # positions do reach the logits, and through the table: the same tokens from another first position differ
+        assert float((want(toks, P._same, first=9) - exact).abs().max()) > 0.05 * float(exact.std())
+        for graphs in (False, True):
+            r = ModelRunner(model, 16, 12, 2, 64, 96, use_graph=graphs, max_graph_batch=2)
+            assert r.use_graph == graphs and r.graph_prompts == graphs
+            r.manager.add_request("a")
+            got, fed = [], 0
+            for n in [23, 2, 17] + [1] * 28:
+                assert r.manager.grow("a", fed + n)
+                seqs = [SeqStep("a", toks[fed:fed + n], [n - 1] if graphs else list(range(n)))]
+                got.append(r.step(seqs).clone())
+                r.advance(seqs)
+                fed += n
+            rows = [22, 24, 41] + list(range(42, 70)) if graphs else list(range(70))
+            close_to_plain(torch.cat(got), exact[rows], want(toks, P.to_bf16)[rows], dtype)
+            if graphs:
+                assert r._graphs and r._prompt_graphs

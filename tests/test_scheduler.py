@@ -6,11 +6,12 @@ import pytest
 from pico_vllm_amd.cache.manager import CacheManager
 from pico_vllm_amd.engine.request import Request, RequestStatus
 from pico_vllm_amd.engine.scheduler import Scheduler
+from pico_vllm_amd.parts.attention import kv_page_tensors
 from pico_vllm_amd.parts.spec import CacheSpec
 from pico_vllm_amd.sampling.params import SamplingParams
 from pico_vllm_amd.sampling.sampler import uniform
 
-SPEC = {0: CacheSpec("paged_kv", num_kv_heads=1, head_dim=16)}
+SPEC = {0: CacheSpec("paged_kv", page_tensors=kv_page_tensors(1, 16))}
 
 
 def make(num_pages=64, page=16, max_seqs=4, budget=32, max_len=512):
@@ -45,6 +46,24 @@ def drive(s: Scheduler, requests, max_steps=10000, log=None):
                     order.append(r.request_id)
         s.manager.check()
     raise AssertionError("did not finish")
+
+
+def test_a_prompt_portion_is_capped_beside_the_budget():
+    # prefill_chunk: the longest portion of ONE prompt in a step; the budget is what all sequences of a step share
+    m = CacheManager(SPEC, 16, 64, 4)
+    s = Scheduler(m, 4, 32, 512, prefill_chunk=12)
+    for i, n in enumerate([30, 10, 29]):
+        s.add_request(req(i, n, 2))
+    log = []
+    drive(s, None, log=log)
+    assert log[0] == [(0, 0, 12), (1, 0, 10), (2, 0, 10)]                  # 12 of request 0, then the budget's rest
+    assert log[1] == [(0, 12, 12), (1, 10, 1), (2, 10, 12)] or log[1] == [(1, 10, 1), (0, 12, 12), (2, 10, 12)]
+    assert all(n <= 12 for step in log for _, _, n in step)
+    assert all(sum(n for _, _, n in step) <= 32 for step in log)
+    # the cap never exceeds the budget, and nonsense is refused
+    assert Scheduler(m, 4, 32, 512, prefill_chunk=100).prefill_chunk == 32 and Scheduler(m, 4, 32, 512).prefill_chunk == 32
+    with pytest.raises(ValueError, match="prefill_chunk"):
+        Scheduler(m, 4, 32, 512, prefill_chunk=0)
 
 
 def test_fcfs_admission_and_token_budget_cut_prompts_into_portions():
@@ -181,7 +200,7 @@ def test_a_preempted_request_can_finish_while_it_waits():
 def test_a_windowed_group_is_sized_by_its_window_not_by_the_length():
     # layers that read only the last 40 keys hold 40 + a step's tokens, whatever the length of the request: a pool
     # of 8 pages (128 tokens) serves a request of 400 tokens, which a group without a window would refuse
-    win = {0: CacheSpec("paged_kv", num_kv_heads=1, head_dim=16, window=40)}
+    win = {0: CacheSpec("paged_kv", window=40, page_tensors=kv_page_tensors(1, 16))}
     m = CacheManager(win, 16, 8, 2)
     s = Scheduler(m, 2, 32, 512)
     s.add_request(req(0, 300, 100))
