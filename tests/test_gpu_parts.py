@@ -1135,3 +1135,156 @@ def test_toy_parts_around_the_layers_learned_positions_in_front_and_a_gain_behin
             close_to_plain(torch.cat(got), exact[rows], want(toks, P.to_bf16)[rows], dtype)
             if graphs:
                 assert r._graphs and r._prompt_graphs
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_toy_mixer_whose_pages_hold_what_it_says(dtype):
+    """The tensors of a cache page are the mixer's to name (``CacheSpec.page_tensors``): this toy mixer keeps ONE latent
+    vector of 12 numbers per token, in float32 whatever the engine's dtype, in pages [page, 12], beside a second
+    tensor [3, page] of the positions' powers that it never needs again but stores to show two tensors of different
+    shapes; it mixes by the causal mean of the cached latents (y_t = Wu mean_{s <= t} Wd x_s).  Layer 0 has it, layer 1
+    the framework's attention: two groups of pages with one block table each.  Whole against a plain computation,
+    portions and mixed steps against whole, pages given back and used again, and generation through the scheduler."""
+    import tempfile
+    from pico_vllm_amd.config.registry import register_architecture
+    from pico_vllm_amd.engine.batch import SeqStep
+    from pico_vllm_amd.engine.step import ModelRunner
+    from pico_vllm_amd.parts.base import Mixer
+    from pico_vllm_amd.parts.model import load_model
+    from pico_vllm_amd.parts.registry import register_part
+    from pico_vllm_amd.parts.spec import CacheSpec, LayerSpec, ModelSpec, PageTensor, ParamSpec, PartSpec, RunEntry
+    from pico_vllm_amd.weights.random_init import write_random_model
+
+    H, V, R, NQ, NKV, D = 40, 90, 12, 2, 1, 16
+
+    @register_part("mixer", "toy_latent_mean")
+    class LatentMean(Mixer):
+        graph_safe = False                   # it sizes a gather by the longest context of the step, on the host
+
+        def __init__(self, hidden_size, latent, act_dtype=torch.bfloat16):
+            self.H, self.R = hidden_size, latent
+
+        def cache_spec(self):
+            return CacheSpec("paged_kv", page_tensors=(PageTensor("latent", ("page", self.R), "float32"),
+                                                       PageTensor("powers", (3, "page"), "float32")))
+
+        def param_specs(self):
+            return [ParamSpec("down.weight", (self.R, self.H), std=0.4), ParamSpec("up.weight", (self.H, self.R), std=0.4)]
+
+        def load(self, tensors, device, dtype):
+            self.wd, self.wu = tensors["down.weight"].to(device).float(), tensors["up.weight"].to(device).float()
+
+        def forward(self, x, ctx, cache):
+            T, P = x.shape[0], cache.page_size
+            assert cache.latent.shape[1:] == (P, self.R) and cache.powers.shape[1:] == (3, P) and cache.latent.dtype == torch.float32
+            seq, pos = ctx.token_seq[:T].long(), ctx.positions[:T].long()
+            slots = ctx.slot_mapping[cache.group][:T].long()                 # page * P + place in the page
+            flat = cache.latent.view(-1, self.R)
+            flat.index_copy_(0, slots, x.float() @ self.wd.T)
+            pw = cache.powers.permute(0, 2, 1).reshape(-1, 3)                # a copy: written back below
+            pw[slots] = torch.stack([pos.float(), pos.float() ** 2, pos.float() ** 3], 1)
+            cache.powers.copy_(pw.view(-1, P, 3).permute(0, 2, 1))
+            # every token's mean over the latents of its request up to its own position, from the pages
+            longest = int(ctx.host["context_lens"][:ctx.num_seqs].max())
+            keys = torch.arange(longest, device=x.device)
+            pages = ctx.block_tables[cache.group][seq][:, keys // P].long()     # [T, longest]; -1 beyond a request's pages
+            seen = keys[None, :] <= pos[:, None]
+            lat = flat[(pages * P + keys % P).clamp(min=0)] * seen[..., None]
+            mean = lat.sum(1) / (pos + 1).float()[:, None]
+            return (mean @ self.wu.T).to(x.dtype)
+
+    def toy_spec(cfg):
+        norm = PartSpec("rms_norm", {"size": H, "eps": 1e-5})
+        attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": D, "qkv_bias": True,
+                                          "window": 0, "position": PartSpec("rotary_half", {"rotary_dim": D, "theta": 1e4})})
+        mixers = [("lat", PartSpec("toy_latent_mean", {"hidden_size": H, "latent": R})), ("attn", attn)]
+        ff = PartSpec("swiglu_mlp", {"hidden_size": H, "intermediate_size": 56})
+        layers = [LayerSpec(f"toy.layers.{i}", "prenorm", {"norm1": ("ln1", norm), "mixer": mixers[i], "norm2": ("ln2", norm),
+                                                          "ff": ("ff", ff)}) for i in range(2)]
+        return ModelSpec(H, V, "toy.embed.weight", layers, [RunEntry(0), RunEntry(1)], norm, "toy.norm", None)
+
+    register_architecture("ToyLatentPagesLM", lambda raw: raw, toy_spec)
+    cfg = {"architectures": ["ToyLatentPagesLM"]}
+    rnd = P._same if dtype == torch.float32 else P.to_bf16
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(d, cfg, seed=8, std_overrides={"attn": 0.3, "embed": 0.5, "ff": 0.2})
+        w = {k: v.float() for k, v in P.read_weights(d).items()}
+        model = load_model(d, "float32" if dtype == torch.float32 else "bfloat16", DEV)
+        r = ModelRunner(model, 8, 14, 3, 64, 64)
+        assert len(r.manager.groups) == 2 and not r.use_graph
+        lat_layer = r.storage.layer(0)
+        assert set(lat_layer.tensors) == {"latent", "powers"} and lat_layer.latent.shape == (14, 8, R)
+        assert r.storage.bytes_per_token() == 4 * (R + 3) + 2 * NKV * D * (4 if dtype == torch.float32 else 2)
+
+        def plain(toks, rnd):
+            n = len(toks)
+            pos = torch.arange(n)
+            x = w["toy.embed.weight"][toks]
+            p = "toy.layers.0"
+            h = rnd(P.rms_norm(x, w[f"{p}.ln1.weight"], 1e-5))
+            lat = h @ w[f"{p}.lat.down.weight"].T
+            mean = torch.cumsum(lat, 0) / (pos + 1).float()[:, None]
+            x = x + rnd(mean @ w[f"{p}.lat.up.weight"].T)
+            x = x + P.mlp_layer(rnd(P.rms_norm(x, w[f"{p}.ln2.weight"], 1e-5)), {k.replace(".ff.", ".mlp."): v for k, v in w.items()}, p, rnd)
+            p = "toy.layers.1"
+            h = rnd(P.rms_norm(x, w[f"{p}.ln1.weight"], 1e-5))
+            Wm = torch.cat([w[f"{p}.attn.{n}_proj.weight"] for n in "qkv"])
+            b = torch.cat([w[f"{p}.attn.{n}_proj.bias"] for n in "qkv"])
+            q, k, v = P.split_qkv(rnd(h @ Wm.T + b), NQ, NKV, D)
+            cos, sin = P.rope_tables(pos, D, 1e4)
+            o = rnd(P.causal_attention(rnd(P.apply_rope(q, cos, sin)), rnd(P.apply_rope(k, cos, sin)), v, rnd_p=None if rnd is P._same else rnd))
+            x = x + rnd(o.reshape(n, NQ * D) @ w[f"{p}.attn.o_proj.weight"].T)
+            x = x + P.mlp_layer(rnd(P.rms_norm(x, w[f"{p}.ln2.weight"], 1e-5)), {k.replace(".ff.", ".mlp."): v for k, v in w.items()}, p, rnd)
+            return rnd(P.rms_norm(x, w["toy.norm.weight"], 1e-5)) @ w["toy.embed.weight"].T
+
+        g = torch.Generator().manual_seed(2)
+        reqs = {rid: torch.randint(0, V, (n,), generator=g).tolist() for rid, n in (("a", 43), ("b", 21), ("c", 30))}
+        whole = {}
+        for rid, toks in reqs.items():
+            r.manager.add_request(rid)
+            assert r.manager.grow(rid, len(toks))
+            whole[rid] = r.step([SeqStep(rid, toks, list(range(len(toks))))])
+            r.manager.free_request(rid)
+            close_to_plain(whole[rid], plain(toks, P._same), plain(toks, rnd), dtype)
+        # a and b in portions beside each other; b ends, c takes its pages (14 pages of 8 do not hold all three)
+        got = {rid: [] for rid in reqs}
+        fed = {rid: 0 for rid in reqs}
+        plan = [(("a", 9), ("b", 2)), (("b", 1), ("a", 1)), (("a", 2), ("b", 18)), (("a", 24),), (("c", 13), ("a", 1)), (("a", 6), ("c", 17))]
+        r.manager.add_request("a"); r.manager.add_request("b")
+        for step in plan:
+            if step[0][0] == "c" and "c" not in r.manager.requests:
+                r.manager.free_request("b")
+                r.manager.add_request("c")
+            seqs = []
+            for rid, n in step:
+                assert r.manager.grow(rid, fed[rid] + n), (rid, fed[rid], n)
+                seqs.append(SeqStep(rid, reqs[rid][fed[rid]:fed[rid] + n], list(range(n))))
+            out = r.step(seqs)
+            r.advance(seqs)
+            at = 0
+            for rid, n in step:
+                got[rid].append(out[at:at + n])
+                at += n
+                fed[rid] += n
+            r.manager.check()
+        for rid in reqs:
+            assert fed[rid] == len(reqs[rid])
+            close(torch.cat(got[rid]), whole[rid], dtype, scale=float(whole[rid].std()) * 3)
+        assert all(g.pool.reuse_count > 0 for g in r.manager.groups)
+        del r, model
+        # through the scheduler: generation with a pool so small that requests wait for pages
+        from pico_vllm_amd import LLM, SamplingParams
+        kind = "float32" if dtype == torch.float32 else "bfloat16"
+        prompts = [reqs["a"][:20], reqs["b"][:9], reqs["c"][:15]]
+        sp = SamplingParams(max_new_tokens=10, temperature=0.0, ignore_eos=True)
+        llm = LLM(model=d, dtype=kind, block_size=8, num_gpu_blocks=9, max_seq_len=64, max_num_seqs=3, max_num_batched_tokens=16)
+        assert not llm.engine.runner.use_graph
+        outs = llm.generate(prompts, sp)
+        for prompt, o in zip(prompts, outs):
+            toks = list(prompt)
+            for t in o.token_ids:
+                logits = plain(toks, P._same)[-1]
+                assert float(logits[t]) >= float(logits.max()) - (1e-4 if dtype == torch.float32 else 0.05 * float(logits.std()))
+                toks.append(t)
+        llm.engine.runner.manager.check()
+        assert all(g.pool.num_free == 9 for g in llm.engine.runner.manager.groups)
