@@ -469,7 +469,7 @@ def main() -> int:
             return 2
         r = sampling_point(CONFIG, rows, top_p)
         print(json.dumps({"metric": "sampling call", "unit": "us", "value": r["top_p"], "greedy": r["greedy"],
-                          "temperature": r["temperature"], "top_p": r["top_p"], "rows": rows, "vocab_size": r["vocab"],
+                          "temperature": r["temperature"], "top_p": r["top_p"], "rows": rows, "vocab": r["vocab"],
                           "p": top_p}))
         return 0
     if a.write_model:
