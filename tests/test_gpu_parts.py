@@ -100,11 +100,12 @@ def test_attention_and_mlp_and_block_parts(name, dtype):
     close_to_plain(resid2 + whole(pending), wantb, P.block(x, plain.w, 0, cfg, pos, rnd=P.to_bf16), dtype)
 
 
-@pytest.mark.parametrize("d", [16, 64])
+@pytest.mark.parametrize("d", [16, 64, 24, 40])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_part_with_a_window(dtype, d):
     """The same mixer class with window = 24: its cache group gives pages back, and the result is
-    the plain windowed attention (head size 16: the 32-query matrix-core kernels in bfloat16, 64: the 16-query ones)."""
+    the plain windowed attention (head size 16: the 32-query matrix-core kernels in bfloat16, 64: the 16-query ones,
+    24 and 40: no multiple of 16, the plain kernel in both precisions)."""
     from pico_vllm_amd.cache.manager import CacheManager
     from pico_vllm_amd.cache.storage import CacheStorage
     from pico_vllm_amd.engine.batch import BatchBuffers, SeqStep, build_context
