@@ -412,7 +412,8 @@ def main() -> int:
                     help="with --prefill-only: the prompt's length (2 to 2048; the contract's prefill is of 2,048 tokens)")
     ap.add_argument("--write-model", metavar="DIR", default=None,
                     help="only write the random-weights model folder to DIR (to reuse with --model) and exit")
-    ap.add_argument("--model", default=None, help="reuse a model folder instead of writing random weights")
+    ap.add_argument("--model", default=None, help="measure this model folder (config.json + model.safetensors, any registered "
+                    "architecture) instead of writing random weights of --shape")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes (default: the 1.5B shape)")
     ap.add_argument("--layers", type=int, default=0, help="run only this many layers of the shape (0: all)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
@@ -432,6 +433,20 @@ def main() -> int:
     a = ap.parse_args()
     global CONFIG, CONTEXT
     shape_name, full = SHAPES[a.shape]
+    if a.model:
+        # a model folder says itself what it is (any registered architecture); it keeps the shape's name if it has the shape's sizes
+        from pico_vllm_amd.config.model_config import read_config_json
+        own = read_config_json(a.model)
+        if a.layers:
+            print("bench.py: --layers cuts a named shape; a model folder has the layers it has")
+            return 2
+        arch_own = describe(own)[0]
+        if arch_own.sizes is None:
+            print(f"bench.py: the architecture of {a.model} registers no sizes for the record")
+            return 2
+        if arch_own.sizes(arch_own.config_from_dict(own)) != describe(full)[0].sizes(describe(full)[1]):
+            shape_name = f"{arch_own.name} in {os.path.basename(os.path.normpath(a.model))}"
+        full = own
     arch, typed_full, _ = describe(full)
     layers_full = arch.sizes(typed_full)["layers"]
     CONFIG = dict(full)
@@ -583,12 +598,12 @@ def main() -> int:
                 pts[f"decode_b{b}"] = round(r["tok_s"], 1)
                 pts[f"decode_b{b}_hbm_frac"] = round(r["gbps"] * 1e9 / HBM_PEAK, 4)
                 log(f"decode batch {b}: {r['tok_s']:.0f} tok/s, {r['ms_per_step']:.3f} ms/step")
-            if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16":
+            if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16" and shape_name == SHAPES["1.5b"][0]:
                 # the one figure the reference publishes for this model: 97 tok/s at batch 1 on its authors' card
                 # (README.md:9,43-45 of the reference); other hardware, so a context, not a baseline
                 pts["decode_b1_vs_reference_published"] = round(pts["decode_b1"] / 97.0, 2)
             out["points"] = pts
-            if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16" and not a.no_other:
+            if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16" and not a.no_other and not a.model:
                 # a second shape, driver-visible: the larger the matrices, the nearer a step comes to what the memory allows
                 del model
                 torch.cuda.empty_cache()
