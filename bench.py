@@ -328,8 +328,10 @@ def attention_point(cfg, nseq, new_len, prefix, shape=0, reps=20, chunk_len=0):
     fa = FastAttention(nq, nkv, d)
     shape = shape or fa.prefill_teams([new_len] * nseq, [ctx] * nseq)
     out = torch.empty(nseq * new_len, nq * d, dtype=torch.bfloat16, device=dev)
-    run = lambda: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, out=out, teams=shape, chunk_len=chunk_len,
-                             max_chunks=-(-ctx // chunk_len) if chunk_len else 0)
+    order = fa.order_list(nseq * new_len, nseq, dev) if nseq > 1 else None      # the tiles of all sequences, longest first
+    run = lambda build=False: fa.prefill(q, kc, vc, bt, cu, cl, nseq, d ** -0.5, out=out, teams=shape, chunk_len=chunk_len,
+                                         max_chunks=-(-ctx // chunk_len) if chunk_len else 0, order=order, order_build=build)
+    run(True)          # the list is written once a step, by the first layer
     for _ in range(5):
         run()
     torch.cuda.synchronize()

@@ -694,7 +694,7 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, int num_seqs, bf16_t* __restrict__ out, int nq, int nkv, int P, int num_pages,
-    float scale, int reach, int chunk_len, int max_chunks, float* __restrict__ part) {
+    float scale, int reach, int chunk_len, int max_chunks, float* __restrict__ part, const int* __restrict__ order) {
   static_assert(NQB == 1 || KT <= 2, "two query blocks a wave: one or two teams (three would leave a wave 170 registers)");
   constexpr int PF_TK = 64 * KT, PF_VROW = PF_TK + 8;
   constexpr int BMQ = PF_BM * NQB;            // queries per workgroup
@@ -704,13 +704,20 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
   __shared__ alignas(16) char lds[LDS_BYTES];
   PfTiles<KT>& tiles = *reinterpret_cast<PfTiles<KT>*>(lds);
   int b = 0, tile = (int)blockIdx.y, ntiles = 0;
-  for (; b < num_seqs; b++) {
-    ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + BMQ - 1) / BMQ;
-    if (tile < ntiles) break;
-    tile -= ntiles;
+  if (order != nullptr) {       // the tiles of all sequences, longest first (pf_order_kernel): (sequence << 16) | tile, -1 behind the last
+    const int e = order[blockIdx.y];
+    if (e < 0) return;
+    b = e >> 16;
+    tile = e & 0xffff;
+  } else {                      // sequence by sequence, each from its last (longest) tile down
+    for (; b < num_seqs; b++) {
+      ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + BMQ - 1) / BMQ;
+      if (tile < ntiles) break;
+      tile -= ntiles;
+    }
+    if (b >= num_seqs) return;
+    tile = ntiles - 1 - tile;
   }
-  if (b >= num_seqs) return;
-  tile = ntiles - 1 - tile;
   const int head = blockIdx.x, g = head / (nq / nkv);
   const int tok0 = cu_seqlens[b], new_len = cu_seqlens[b + 1] - tok0;
   const int ctx = context_lens[b], prefix = ctx - new_len;
@@ -890,6 +897,45 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
       *reinterpret_cast<uint2*>(orow + 16 * tt) = v;
     }
   }
+}
+
+// The order in which the workgroups of prefill16_kernel take the query tiles of a step with several sequences: all
+// tiles of all sequences by the number of keys they read, most first.  Workgroups start in the order of the grid, and a
+// compute unit takes the next one when it has finished one; sequence by sequence, the long tiles of the last sequence
+// would start when the others are nearly through and the launch would end on them (eight prompts of 2,048 tokens: the
+// compute units finished between 117 and 176 us).  One workgroup; every thread ranks its entries against all others in
+// LDS, which is quadratic and therefore offered only up to PF_ORDER_MAX entries.
+// order[r] = (sequence << 16) | tile for rank r, -1 from the number of tiles on (capacity entries in all).
+constexpr int PF_ORDER_MAX = 512;
+__global__ __launch_bounds__(256) void pf_order_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+                                                       int num_seqs, int bmq, int* __restrict__ order, int capacity) {
+  __shared__ int keys[PF_ORDER_MAX], ids[PF_ORDER_MAX], first[PF_ORDER_MAX + 1];
+  if (threadIdx.x == 0) {
+    int n = 0;
+    for (int b = 0; b < num_seqs; b++) {
+      first[b] = n;
+      n += (cu_seqlens[b + 1] - cu_seqlens[b] + bmq - 1) / bmq;
+    }
+    first[num_seqs] = n;
+  }
+  __syncthreads();
+  const int n = min(first[num_seqs], PF_ORDER_MAX);          // the host has checked that it holds all of them
+  for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) {
+    const int new_len = cu_seqlens[b + 1] - cu_seqlens[b], ctx = context_lens[b], prefix = ctx - new_len;
+    for (int e = first[b]; e < min(first[b + 1], PF_ORDER_MAX); e++) {
+      const int tile = e - first[b];
+      keys[e] = min(ctx, prefix + min(new_len, (tile + 1) * bmq));
+      ids[e] = (b << 16) | tile;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n; e += blockDim.x) {
+    const int key = keys[e];
+    int rank = 0;
+    for (int o = 0; o < n; o++) rank += (keys[o] > key || (keys[o] == key && o < e)) ? 1 : 0;
+    order[rank] = ids[e];
+  }
+  for (int e = n + threadIdx.x; e < capacity; e += blockDim.x) order[e] = -1;
 }
 
 // Joins the chunks of the tiles that prefill16_kernel cut (chunk_len > 0): out[token, head, :] =
@@ -1286,11 +1332,14 @@ extern "C" int pico_attn_head_dim() { return D; }
 // value gives the same result up to rounding.  chunk_len > 0 (a multiple of 128, no window, not three teams, head sizes in steps of 32): the keys of every tile are cut
 // into chunks of that many, each a workgroup of its own, and a second launch joins the chunks of a tile; part is
 // their workspace, float32 [num_tokens, nq, max_chunks, D + 4], and max_chunks at least ceil(longest context / chunk_len).
+// order (may be null): room for order_capacity >= num_tokens / 64 + num_seqs integers; with several sequences their query
+// tiles are taken longest first from the list that pf_order_kernel writes there, when order_build is set (the first
+// layer of a step) or has written there (the others: same sequences, same `teams`).
 extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int* block_table, int max_pages, const int* cu_seqlens,
                                  const int* context_lens, int num_seqs, int num_tokens, void* out, int nq, int nkv,
                                  int d, int P, int num_pages, float scale, int teams, int window, int chunk_len,
-                                 int max_chunks, float* part, hipStream_t stream) {
+                                 int max_chunks, float* part, int* order, int order_capacity, int order_build, hipStream_t stream) {
   if (check_common("pico_attn_prefill", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
   PICO_REQUIRE(window >= 0 && window < NO_WINDOW, "pico_attn_prefill: bad window %d", window);
   const int reach = window > 0 ? window : NO_WINDOW;
@@ -1312,18 +1361,29 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
                    "(got %d), 1 to 64 chunks (got %d) and an aligned workspace", chunk_len, max_chunks);
       grid.z = max_chunks;
     }
-    int bmq = PF_BM;
+    // 4 and 6: 128 queries a workgroup (two blocks of 16 a wave), in one team or two
+    const bool wide = (teams == 4 || teams == 6) && PF_KT_MAX == 2;
+    const int bmq = wide ? 2 * PF_BM : PF_BM;
+    if (wide) grid.y = num_tokens / (2 * PF_BM) + num_seqs;
+    // several sequences: their tiles longest first, from the caller's list (built here when the caller says so: once a
+    // step, the layers of a step share it); a step of more tiles than the ordering kernel takes goes sequence by sequence
+    const int* ord = nullptr;
+    if (order != nullptr && num_seqs >= 2 && num_seqs <= PF_ORDER_MAX && (int)grid.y <= PF_ORDER_MAX) {
+      PICO_REQUIRE(order_capacity >= (int)grid.y, "pico_attn_prefill: the list of tiles holds %d entries, the step may have %d",
+                   order_capacity, (int)grid.y);
+      if (order_build) {
+        pf_order_kernel<<<1, 256, 0, stream>>>(cu_seqlens, context_lens, num_seqs, bmq, order, (int)grid.y);
+        PICO_LAUNCH_CHECK();
+      }
+      ord = order;
+    }
 #define PF_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, \
-                cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach, chunk_len, max_chunks, part
-    if (teams == 6 && PF_KT_MAX == 2) {      // 128 queries a workgroup and two key teams
-      grid.y = num_tokens / (2 * PF_BM) + num_seqs;
-      bmq = 2 * PF_BM;
+                cu_seqlens, context_lens, num_seqs, (bf16_t*)out, nq, nkv, P, num_pages, scale, reach, chunk_len, max_chunks, part, ord
+    if (teams == 6 && PF_KT_MAX == 2)             // 128 queries a workgroup and two key teams
       prefill16_kernel<PF_KT_MAX == 2 ? 2 : 1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 512, 0, stream>>>(PF_ARGS);
-    } else if (teams == 4 && PF_KT_MAX == 2) {      // 128 queries a workgroup, two blocks of 16 a wave
-      grid.y = num_tokens / (2 * PF_BM) + num_seqs;
-      bmq = 2 * PF_BM;
+    else if (teams == 4 && PF_KT_MAX == 2)        // 128 queries a workgroup, two blocks of 16 a wave
       prefill16_kernel<1, PF_KT_MAX == 2 ? 2 : 1><<<grid, 256, 0, stream>>>(PF_ARGS);
-    } else if (teams == 1 || PF_KT_MAX == 1)
+    else if (teams == 1 || PF_KT_MAX == 1)
       prefill16_kernel<1><<<grid, 256, 0, stream>>>(PF_ARGS);
     else if (teams == 3 && PF_KT_MAX == 2)
       prefill16_kernel<PF_KT_MAX == 2 ? 3 : 1><<<grid, 768, 0, stream>>>(PF_ARGS);

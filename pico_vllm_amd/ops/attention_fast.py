@@ -124,11 +124,13 @@ class FastAttention:
 
     def prefill(self, q: torch.Tensor, k_cache, v_cache, block_table, cu_seqlens, context_lens, num_seqs: int,
                 scale: float, out: Optional[torch.Tensor] = None, teams: int = 0, chunk_len: int = 0,
-                max_chunks: int = 0) -> torch.Tensor:
+                max_chunks: int = 0, order: Optional[torch.Tensor] = None, order_build: bool = True) -> torch.Tensor:
         """q [T, >= nq*d] bfloat16 (row stride free); any mixture of portions; returns [T, nq*d].
         teams: 0 lets the kernel choose, else the result of ``prefill_teams``.  chunk_len > 0: the keys of every
         query tile are cut into chunks of that many, each a workgroup of its own (``max_chunks`` of them cover the
-        longest context), and a second launch joins them."""
+        longest context), and a second launch joins them.  order: ``order_list(T, num_seqs)``, where the kernel
+        writes (``order_build``) or finds (the other layers of a step) the query tiles of all sequences longest
+        first; without it the sequences are taken one after the other."""
         nq, nkv, d = self.nq, self.nkv, self.d
         T = q.shape[0]
         pages, P = _check_cache(k_cache, v_cache, nkv, d)
@@ -146,8 +148,14 @@ class FastAttention:
         _check(self.lib, self.lib.pico_attn_prefill(
             _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens), _ptr(context_lens), num_seqs, T, _ptr(out), nq, nkv, d, P, pages, c_float(scale),
-            teams, self.window, chunk_len, max_chunks, _ptr(part), _stream()))
+            teams, self.window, chunk_len, max_chunks, _ptr(part), _ptr(order), 0 if order is None else order.numel(),
+            1 if order_build else 0, _stream()))
         return out
+
+    @staticmethod
+    def order_list(num_tokens: int, num_seqs: int, device) -> torch.Tensor:
+        """Room for the list of a step's query tiles (``prefill(order=...)``): one entry a tile of 64 queries at most."""
+        return torch.empty(num_tokens // 64 + num_seqs, dtype=torch.int32, device=device)
 
     def decode(self, q: torch.Tensor, k_cache, v_cache, block_table, context_lens, num_seqs: int, scale: float,
                nsplit: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -215,9 +223,18 @@ class FastAttention:
             return self.decode(qkv, cache.k, cache.v, block_table, ctx.context_lens, B, scale,
                                self.num_splits(B, ctx.max_context))
         teams, lead, chunk_len, max_chunks = self.plan(ctx)
-        if lead == 0 or not grouped:
+        if not grouped:
+            lead = 0
+        # several portions: the list of their query tiles, longest first, written by the first layer of the step
+        order, build = None, False
+        if B - lead >= 2:
+            key = ("fast_attention_order", teams in (4, 6), lead)
+            order, build = ctx.shared.get(key), key not in ctx.shared
+            if build:
+                order = ctx.shared[key] = self.order_list(qkv.shape[0], B - lead, qkv.device)
+        if lead == 0:
             return self.prefill(qkv, cache.k, cache.v, block_table, ctx.cu_seqlens, ctx.context_lens, B, scale, teams=teams,
-                                chunk_len=chunk_len, max_chunks=max_chunks)
+                                chunk_len=chunk_len, max_chunks=max_chunks, order=order, order_build=build)
         # A mixed step: the scheduler puts the decoding requests first.  Their tokens (one row each, rows
         # 0 .. lead - 1) go through the decode kernel, which reads keys and values once for all query heads of
         # a group; the prompt portions behind them through the prefill kernel, whose offsets are absolute.
@@ -226,7 +243,8 @@ class FastAttention:
                     self.num_splits(lead, ctx.max_context), out=out[:lead])
         if lead < B:
             self.prefill(qkv, cache.k, cache.v, block_table[lead:], ctx.cu_seqlens[lead:], ctx.context_lens[lead:],
-                         B - lead, scale, out=out, teams=teams, chunk_len=chunk_len, max_chunks=max_chunks)
+                         B - lead, scale, out=out, teams=teams, chunk_len=chunk_len, max_chunks=max_chunks, order=order,
+                         order_build=build)
         return out
 
 

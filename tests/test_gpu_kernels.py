@@ -485,7 +485,7 @@ def test_sampling_top_p(K):
 
 # ---- matrix-core attention (bfloat16) ----------------------------------------------------------
 def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0, as_step=False,
-               window=0, chunk_len=0, max_chunks=0):
+               window=0, chunk_len=0, max_chunks=0, order=None):
     from pico_vllm_amd.ops.attention_fast import FastAttention
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(seed)
@@ -514,8 +514,11 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
     elif decode:
         out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
     else:
+        if order is not None:           # a list to fill: the query tiles of all sequences longest first
+            order.append(fa.order_list(T, B, DEV))
         out = fa.prefill(wide, kc, vc, bt, cu, ctxl, B, scale, teams=teams, chunk_len=chunk_len,
-                         max_chunks=max_chunks or (-(-max(totals) // chunk_len) if chunk_len else 0))
+                         max_chunks=max_chunks or (-(-max(totals) // chunk_len) if chunk_len else 0),
+                         order=order[0] if order is not None else None)
     want = torch.cat([P.causal_attention(qb, kb, vb, q_positions=torch.arange(p, p + n), window=window)
                       for qb, kb, vb, n, p in zip(qs, ks, vs, new_lens, prefix_lens)], 0)
     return out.reshape(-1, nq, d), want
@@ -591,6 +594,28 @@ def test_fast_prefill_with_every_shape_of_workgroup(K, nq, nkv, d, Pg, teams):
     out, want = _fast_case([63, 1, 65, 130, 2, 200, 193, 127, 257], [0, 127, 1, 62, 191, 129, 383, 1, 64], nq, nkv, d, Pg, seed=5,
                            teams=teams)
     close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("teams,chunk_len", [(1, 0), (2, 0), (3, 0), (4, 0), (6, 0), (1, 256), (4, 128)])
+@pytest.mark.parametrize("nq,nkv,d,Pg", [(12, 2, 128, 16), (6, 3, 32, 8), (4, 1, 96, 32), (2, 1, 160, 8)])
+def test_fast_prefill_takes_the_tiles_of_several_sequences_longest_first(K, nq, nkv, d, Pg, teams, chunk_len):
+    # with a list to fill, the workgroups take the query tiles of all sequences by the keys they read, most first: the
+    # list is a permutation of the tiles in that order, and the attention is the same bits as sequence by sequence
+    new_lens, prefix_lens = [63, 1, 65, 130, 2, 200, 193, 127, 257], [0, 127, 1, 62, 191, 129, 383, 1, 64]
+    plain, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=5, teams=teams, chunk_len=chunk_len)
+    order = []
+    out, _ = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=5, teams=teams, chunk_len=chunk_len, order=order)
+    close(out, want, torch.bfloat16)
+    assert torch.equal(out, plain)
+    bmq = 128 if teams in (4, 6) and d <= 128 else 64
+    tiles = [(b, t) for b, n in enumerate(new_lens) for t in range(-(-n // bmq))]
+    grid = sum(new_lens) // bmq + len(new_lens)                 # tiles the launch has room for; the list may be longer
+    got = order[0].cpu().tolist()[:grid]
+    assert got[len(tiles):] == [-1] * (grid - len(tiles)) and order[0].numel() >= grid
+    listed = [(e >> 16, e & 0xffff) for e in got[:len(tiles)]]
+    assert sorted(listed) == tiles
+    keys = [min(prefix_lens[b] + new_lens[b], prefix_lens[b] + (t + 1) * bmq) for b, t in listed]
+    assert keys == sorted(keys, reverse=True)
 
 
 @pytest.mark.parametrize("Pg", [8, 16, 32])
