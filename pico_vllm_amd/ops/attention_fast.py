@@ -228,7 +228,7 @@ class FastAttention:
         # several portions: the list of their query tiles, longest first, written by the first layer of the step
         order, build = None, False
         if B - lead >= 2:
-            key = ("fast_attention_order", teams in (4, 6), lead)
+            key = ("fast_attention_order", self.d, teams, lead)        # the tiles' size goes with the head size and the shape
             order, build = ctx.shared.get(key), key not in ctx.shared
             if build:
                 order = ctx.shared[key] = self.order_list(qkv.shape[0], B - lead, qkv.device)
