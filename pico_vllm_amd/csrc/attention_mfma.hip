@@ -989,17 +989,30 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(c
                                                      const int* __restrict__ block_table, int max_pages,
                                                      const int* __restrict__ context_lens,
                                                      float* __restrict__ part, int nsplit, int nq, int nkv, int P,
-                                                     int num_pages, float scale, int reach) {
+                                                     int num_pages, float scale, int reach, const int4* __restrict__ plan) {
   __shared__ Tiles tiles;
-  const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  const int g = blockIdx.y;
   const int G = nq / nkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
-  const int ctx = context_lens[b];
+  int b, ctx, k_begin, k_end;
+  size_t part_slot;                 // this workgroup's place among the partial results, counted in (query heads) rows
+  if (plan != nullptr) {            // splits of equal length over all sequences (decode_plan_kernel): grid x is the split
+    const int4 mine = plan[blockIdx.x];
+    if (mine.x < 0) return;
+    b = mine.x, k_begin = mine.y, k_end = mine.z, ctx = mine.w;
+    part_slot = (size_t)blockIdx.x * nq;
+  } else {                          // every sequence in nsplit splits of its own
+    b = blockIdx.x;
+    ctx = context_lens[b];
+    const int lo_tile = max(0, ctx - reach) / BN * BN;
+    // this split's keys: a whole number of LDS tiles
+    const int per = ((ctx - lo_tile + nsplit - 1) / nsplit + BN - 1) / BN * BN;
+    k_begin = lo_tile + (int)blockIdx.z * per, k_end = min(ctx, k_begin + per);
+    part_slot = (size_t)b * nq * nsplit + blockIdx.z;
+  }
+  const size_t part_stride = plan != nullptr ? 1 : nsplit;      // rows of the partial results between two heads
   // the query sits at position ctx - 1 and sees keys lo .. ctx - 1; the splits share them from the tile that holds lo on
-  const int lo = max(0, ctx - reach), lo_tile = lo / BN * BN;
-  // this split's keys: a whole number of LDS tiles
-  const int per = ((ctx - lo_tile + nsplit - 1) / nsplit + BN - 1) / BN * BN;
-  const int k_begin = lo_tile + split * per, k_end = min(ctx, k_begin + per);
+  const int lo = max(0, ctx - reach);
   const int* bt = block_table + (size_t)b * max_pages;
   const bool col_ok = col < G;
   const int head = g * G + (col_ok ? col : 0);
@@ -1044,7 +1057,7 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(c
   const float m_use = (m == -INFINITY) ? 0.f : m;
   const float a0 = __expf(st.m - m_use), a1 = __expf(m1 - m_use);
   const float l = st.l * a0 + l1 * a1;
-  float* po = part + (((size_t)b * nq + head) * nsplit + split) * (D + 2);
+  float* po = part + (part_slot + (size_t)head * part_stride) * (D + 2);
 #pragma unroll
   for (int tt = 0; tt < DT; tt++)
 #pragma unroll
@@ -1081,17 +1094,30 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
                                                           const int* __restrict__ block_table, int max_pages,
                                                           const int* __restrict__ context_lens,
                                                           float* __restrict__ part, int nsplit, int nq, int nkv, int P,
-                                                          int num_pages, float scale, int reach) {
+                                                          int num_pages, float scale, int reach, const int4* __restrict__ plan) {
   __shared__ float xo[3][D][16];     // outputs of waves 1..3 for the final merge
   __shared__ float xml[3][2][16];
-  const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  const int g = blockIdx.y;
   const int G = nq / nkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
-  const int ctx = context_lens[b];
+  int b, ctx, k_begin, k_end;
+  size_t part_slot;                 // this workgroup's place among the partial results, counted in (query heads) rows
+  if (plan != nullptr) {            // splits of equal length over all sequences (decode_plan_kernel): grid x is the split
+    const int4 mine = plan[blockIdx.x];
+    if (mine.x < 0) return;
+    b = mine.x, k_begin = mine.y, k_end = mine.z, ctx = mine.w;
+    part_slot = (size_t)blockIdx.x * nq;
+  } else {                          // every sequence in nsplit splits of its own
+    b = blockIdx.x;
+    ctx = context_lens[b];
+    const int lo_block = max(0, ctx - reach) & ~31;
+    const int per = ((ctx - lo_block + nsplit - 1) / nsplit + 31) / 32 * 32;
+    k_begin = lo_block + (int)blockIdx.z * per, k_end = min(ctx, k_begin + per);
+    part_slot = (size_t)b * nq * nsplit + blockIdx.z;
+  }
+  const size_t part_stride = plan != nullptr ? 1 : nsplit;      // rows of the partial results between two heads
   // the query sits at position ctx - 1 and sees keys lo .. ctx - 1; the splits share them from the block that holds lo on
-  const int lo = max(0, ctx - reach), lo_block = lo & ~31;
-  const int per = ((ctx - lo_block + nsplit - 1) / nsplit + 31) / 32 * 32;
-  const int k_begin = lo_block + split * per, k_end = min(ctx, k_begin + per);
+  const int lo = max(0, ctx - reach);
   const int* bt = block_table + (size_t)b * max_pages;
   const bool col_ok = col < G;
   const int head = g * G + (col_ok ? col : 0);
@@ -1227,7 +1253,7 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
     aw[w] = __expf(xml[w][0][col] - m_use);
     L += xml[w][1][col] * aw[w];
   }
-  float* po = part + (((size_t)b * nq + head) * nsplit + split) * (D + 2);
+  float* po = part + (part_slot + (size_t)head * part_stride) * (D + 2);
 #pragma unroll
   for (int tt = 0; tt < DT16; tt++)
 #pragma unroll
@@ -1247,20 +1273,29 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 // quarter of each 64 splits for all head dimensions, the loads of a quarter issued together; wave 0
 // adds the four quarters.
 constexpr int MERGE_MAX_SPLITS = 256;
+// rows (with splits of equal length over all sequences): (first split, number of splits) of every sequence; the partial
+// results of a split's heads then lie together, nq rows apart from split to split.
 __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
-                                                           bf16_t* __restrict__ out, int nq) {
+                                                           bf16_t* __restrict__ out, int nq, const int2* __restrict__ rows) {
   constexpr int DPL = (D + 63) / 64;                        // head dimensions per lane
   constexpr int CH = MERGE_MAX_SPLITS / 64;
   __shared__ float quarter[3][DPL * 64];
   const int b = blockIdx.x, head = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float* p = part + ((size_t)b * nq + head) * nsplit * (D + 2);
+  size_t step = D + 2;                                      // floats from one split of this head to the next
+  if (rows != nullptr) {
+    const int2 mine = rows[b];
+    nsplit = mine.y;
+    p = part + ((size_t)mine.x * nq + head) * (D + 2);
+    step = (size_t)nq * (D + 2);
+  }
   float m[CH], l[CH], wt[CH];
   float mx = -INFINITY;
 #pragma unroll
   for (int c = 0; c < CH; c++) {
     const bool mine = 64 * c + lane < nsplit;
-    m[c] = mine ? p[(64 * c + lane) * (D + 2) + D] : -INFINITY;
-    l[c] = mine ? p[(64 * c + lane) * (D + 2) + D + 1] : 0.f;
+    m[c] = mine ? p[(64 * c + lane) * step + D] : -INFINITY;
+    l[c] = mine ? p[(64 * c + lane) * step + D + 1] : 0.f;
     mx = fmaxf(mx, m[c]);
   }
   const float M = wave_max(mx);
@@ -1291,7 +1326,7 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restri
 #pragma unroll
       for (int i = 0; i < DPL; i++) {
         const int dim = lane + 64 * i;
-        v[j][i] = dim < D ? p[s * (D + 2) + dim] : 0.f;
+        v[j][i] = dim < D ? p[s * step + dim] : 0.f;
       }
     }
 #pragma unroll
@@ -1314,6 +1349,73 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restri
     if (dim < D)
       o[dim] = f32_to_bf16((acc[i] + quarter[0][dim] + quarter[1][dim] + quarter[2][dim]) * inv);
   }
+}
+
+// Splits of equal length over all sequences of a decode step.  With the same number of splits for every sequence a
+// step of unequal contexts ends on the workgroups of its longest sequences (64 sequences of 128 to 4,224 tokens: 35 us a
+// layer where equal contexts of the same total take 27).  Here all sequences are cut into pieces of one length T, the
+// smallest whole number of `unit` keys for which the pieces of all sequences fit the `slots` workgroups of the launch
+// (and no sequence has more than the merging kernel takes); with equal contexts that is the cut they had before.  T
+// depends on the contexts of the step alone (rows without a context, the padding of a recorded step, count for
+// nothing), so a sequence is cut alike whether the step is recorded and padded or not.
+// plan[slot] = (sequence, first key, end, context) or (-1, ..) for a slot that stays empty; rows[b] = (first slot, slots).
+// One workgroup; at most PLAN_MAX_ROWS sequences.
+constexpr int PLAN_MAX_ROWS = 1024;
+__global__ __launch_bounds__(256) void decode_plan_kernel(const int* __restrict__ context_lens, int num_seqs, int slots,
+                                                          int reach, int unit, int4* __restrict__ plan, int2* __restrict__ rows) {
+  __shared__ int len[PLAN_MAX_ROWS], low[PLAN_MAX_ROWS], first[PLAN_MAX_ROWS + 1];
+  __shared__ int red[256];
+  __shared__ int piece;
+  auto block_reduce = [&](int v, bool take_max) {
+    red[threadIdx.x] = v;
+    __syncthreads();
+    for (int w = 128; w >= 1; w >>= 1) {
+      if ((int)threadIdx.x < w) red[threadIdx.x] = take_max ? max(red[threadIdx.x], red[threadIdx.x + w]) : red[threadIdx.x] + red[threadIdx.x + w];
+      __syncthreads();
+    }
+    const int r = red[0];
+    __syncthreads();
+    return r;
+  };
+  int my_sum = 0, my_max = 0;
+  for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) {
+    const int ctx = context_lens[b];
+    const int lo = max(0, ctx - reach) / unit * unit;        // the splits share the keys from the unit that holds the first visible one on
+    low[b] = lo;
+    len[b] = ctx > 0 ? ctx - lo : 0;
+    my_sum += (len[b] + unit - 1) / unit;                    // counted in units, so the sums stay small
+    my_max = max(my_max, len[b]);
+  }
+  const int total_units = block_reduce(my_sum, false), longest = block_reduce(my_max, true);
+  // the smallest T = t units with sum over b of ceil(len_b / T) <= slots: t lies between what fills every slot exactly and
+  // one piece a sequence (which fits: the launch has a slot for every sequence)
+  int t_lo = max(1, max((total_units + slots - 1) / slots, ((longest + MERGE_MAX_SPLITS - 1) / MERGE_MAX_SPLITS + unit - 1) / unit));
+  int t_hi = max(t_lo, (longest + unit - 1) / unit);
+  while (t_lo < t_hi) {                                       // the same for all threads
+    const int mid = (t_lo + t_hi) / 2, T = mid * unit;
+    int mine = 0;
+    for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) mine += (len[b] + T - 1) / T;
+    if (block_reduce(mine, false) <= slots) t_hi = mid;
+    else t_lo = mid + 1;
+  }
+  if (threadIdx.x == 0) {
+    const int T = t_lo * unit;
+    piece = T;
+    int n = 0;
+    for (int b = 0; b < num_seqs; b++) {
+      first[b] = n;
+      n += (len[b] + T - 1) / T;
+    }
+    first[num_seqs] = n;
+  }
+  __syncthreads();
+  const int T = piece;
+  for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) {
+    const int count = first[b + 1] - first[b], ctx = low[b] + len[b];
+    rows[b] = make_int2(first[b], count);
+    for (int i = 0; i < count; i++) plan[first[b] + i] = make_int4(b, low[b] + i * T, min(ctx, low[b] + (i + 1) * T), ctx);
+  }
+  for (int e = first[num_seqs] + threadIdx.x; e < slots; e += blockDim.x) plan[e] = make_int4(-1, 0, 0, 0);
 }
 
 static int check_common(const char* who, int nq, int nkv, int d, int P, int max_pages, int num_pages, int q_stride) {
@@ -1412,10 +1514,13 @@ extern "C" int pico_attn_prefill(const void* q, int q_stride, const void* k_cach
 }
 
 // part: float32 workspace of num_seqs * nq * nsplit * (D + 2) entries
+// plan (may be null): 4 * plan_slots + 2 * num_seqs integers; the contexts of all sequences are then cut into pieces of
+// one length, at most plan_slots >= num_seqs of them in all (pico_attn_decode_plan writes the cut when plan_build is
+// set, the first layer of a step; the other layers find it there), and part holds plan_slots * nq * (D + 2) floats.
 extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                 const int* block_table, int max_pages, const int* context_lens, int num_seqs,
                                 void* out, float* part, int nsplit, int nq, int nkv, int d, int P, int num_pages,
-                                float scale, int window, hipStream_t stream) {
+                                float scale, int window, int* plan, int plan_slots, int plan_build, hipStream_t stream) {
   if (check_common("pico_attn_decode", nq, nkv, d, P, max_pages, num_pages, q_stride)) return -1;
   PICO_REQUIRE(window >= 0 && window < NO_WINDOW, "pico_attn_decode: bad window %d", window);
   const int reach = window > 0 ? window : NO_WINDOW;
@@ -1426,18 +1531,35 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
   bool direct = false;
 #if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
   direct = nq / nkv <= 16;
+#endif
+  const int4* cut = nullptr;
+  const int2* rows = nullptr;
+  if (plan != nullptr) {
+    PICO_REQUIRE(plan_slots >= num_seqs && num_seqs <= PLAN_MAX_ROWS && (uintptr_t)plan % 16 == 0,
+                 "pico_attn_decode: a cut of %d sequences into %d pieces (at most %d sequences, a piece each at least, 16-byte aligned)",
+                 num_seqs, plan_slots, PLAN_MAX_ROWS);
+    cut = reinterpret_cast<const int4*>(plan);
+    rows = reinterpret_cast<const int2*>(plan + 4 * (size_t)plan_slots);
+    if (plan_build) {
+      decode_plan_kernel<<<1, 256, 0, stream>>>(context_lens, num_seqs, plan_slots, reach, direct ? 32 : BN,
+                                                reinterpret_cast<int4*>(plan), reinterpret_cast<int2*>(plan + 4 * (size_t)plan_slots));
+      PICO_LAUNCH_CHECK();
+    }
+    grid = dim3(plan_slots, nkv, 1);
+  }
+#if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
   if (direct)
     decode16_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                              (const bf16_t*)v_cache, block_table, max_pages, context_lens, part,
-                                             nsplit, nq, nkv, P, num_pages, scale, reach);
+                                             nsplit, nq, nkv, P, num_pages, scale, reach, cut);
 #endif
   if (!direct)
     decode_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                            block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
-                                           scale, reach);
+                                           scale, reach, cut);
   PICO_LAUNCH_CHECK();
   dim3 mgrid(num_seqs, nq);
-  decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq);
+  decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq, rows);
   PICO_LAUNCH_CHECK();
   return 0;
 }

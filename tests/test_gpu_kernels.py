@@ -485,7 +485,7 @@ def test_sampling_top_p(K):
 
 # ---- matrix-core attention (bfloat16) ----------------------------------------------------------
 def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode=False, nsplit=1, teams=0, as_step=False,
-               window=0, chunk_len=0, max_chunks=0, order=None):
+               window=0, chunk_len=0, max_chunks=0, order=None, cut=None):
     from pico_vllm_amd.ops.attention_fast import FastAttention
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(seed)
@@ -512,7 +512,9 @@ def _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=0, boost=None, decode
                                context_lens=ctxl, host={"cu_seqlens": cu.cpu().numpy(), "context_lens": ctxl.cpu().numpy()}, shared={})
         out = fa(wide, SimpleNamespace(k=kc, v=vc), bt, step, scale)
     elif decode:
-        out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit)
+        if cut is not None:             # a cut to fill: the contexts of all sequences in pieces of one length
+            cut.append(fa.decode_cut(B, nsplit, DEV))
+        out = fa.decode(wide, kc, vc, bt, ctxl, B, scale, nsplit, cut=cut[0] if cut is not None else None)
     else:
         if order is not None:           # a list to fill: the query tiles of all sequences longest first
             order.append(fa.order_list(T, B, DEV))
@@ -634,6 +636,64 @@ def test_fast_prefill_whole_key_tiles_at_every_head_size_and_page_size(K, d, Pg)
     for nsplit in (1, 5):
         out, want = _fast_case([1, 1], [330, 65], 2, 1, d, Pg, seed=d + Pg, boost=boost, decode=True, nsplit=nsplit)
         close(out, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("nq,nkv,d,Pg,nsplit", [(12, 2, 128, 16, 8), (6, 3, 32, 8, 2), (5, 5, 48, 16, 3), (4, 1, 256, 32, 4), (8, 2, 96, 16, 16)])
+def test_fast_decode_with_the_contexts_cut_into_pieces_of_one_length(K, nq, nkv, d, Pg, nsplit, window):
+    # from 16 sequences on the contexts of a decode step are cut into pieces of one length over all sequences (the pieces of
+    # a long context are as long as a short context's): the cut covers every sequence's keys once, in order, in whole units
+    # of 32 keys (of an LDS tile where the kernel stages tiles), in no more pieces than nsplit splits of 16 sequences
+    # would be and with the smallest length that allows that; the attention is the plain one; and sequences without a context
+    # behind the others (the padding of a recorded step) change no bit of the others
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    def boost(qs, ks, vs):
+        for q in qs:
+            q *= 2.0
+    prefix_lens = [3000, 17, 0, 1000, 64, 129, 2047, 5, 700, 31, 32, 33, 1500]
+    new_lens = [1] * len(prefix_lens)
+    cut = []
+    out, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=nsplit + window, boost=boost, decode=True, nsplit=nsplit,
+                           window=window, cut=cut)
+    close(out, want, torch.bfloat16)
+    plan, slots = cut[0]
+    B = len(prefix_lens)
+    assert slots == 16 * nsplit
+    pieces = plan[:4 * slots].reshape(slots, 4).cpu().tolist()
+    rows = plan[4 * slots:4 * slots + 2 * B].reshape(B, 2).cpu().tolist()
+    unit = 32 if (d % 32 == 0 and d <= 128 and nq // nkv <= 16) else (64 if d <= 128 else 32)
+    used = sum(n for _, n in rows)
+    assert used <= slots and all(p[0] == -1 for p in pieces[used:])
+    lengths = set()
+    for b, (first, n) in enumerate(rows):
+        ctx = prefix_lens[b] + 1
+        low = max(0, ctx - window) // unit * unit if window else 0
+        mine = pieces[first:first + n]
+        assert [p[0] for p in mine] == [b] * n and all(p[3] == ctx for p in mine) and 1 <= n <= 256
+        assert mine[0][1] == low and mine[-1][2] == ctx and all(x[2] == y[1] for x, y in zip(mine, mine[1:]))
+        lengths |= {p[2] - p[1] for p in mine[:-1]}
+        T = mine[0][2] - mine[0][1] if n > 1 else None
+        assert all(p[2] - p[1] == T for p in mine[:-1])
+    assert len(lengths) <= 1 and all(t % unit == 0 for t in lengths)
+    if lengths:                                            # a unit shorter, the pieces would not fit the launch
+        T = lengths.pop()
+        spans = [prefix_lens[b] + 1 - (max(0, prefix_lens[b] + 1 - window) // unit * unit if window else 0) for b in range(B)]
+        assert all(-(-x // T) == n for x, (_, n) in zip(spans, rows))
+        assert T == unit or sum(-(-x // (T - unit)) for x in spans) > slots or -(-max(spans) // (T - unit)) > 256
+    # the same sequences with three rows without a context behind them: the same bits
+    fa = FastAttention(nq, nkv, d, window)
+    g = torch.Generator().manual_seed(7)
+    totals = [p + 1 for p in prefix_lens]
+    ks = [torch.randn(N, nkv, d, generator=g).bfloat16().float() for N in totals]
+    vs = [torch.randn(N, nkv, d, generator=g).bfloat16().float() for N in totals]
+    kc, vc, bt = paged_cache(ks, vs, Pg, sum(-(-N // Pg) for N in totals) + 3, torch.bfloat16, 1)
+    q = torch.randn(B + 3, (nq + 2 * nkv) * d, generator=g).bfloat16().to(DEV)
+    ctxl = torch.tensor(totals + [0, 0, 0], dtype=torch.int32, device=DEV)
+    bt16 = torch.full((B + 3, bt.shape[1]), -1, dtype=torch.int32, device=DEV)
+    bt16[:B] = bt
+    real = fa.decode(q[:B], kc, vc, bt, ctxl[:B], B, d ** -0.5, nsplit, cut=fa.decode_cut(B, nsplit, DEV))
+    padded = fa.decode(q, kc, vc, bt16, ctxl, B + 3, d ** -0.5, nsplit, cut=fa.decode_cut(B + 3, nsplit, DEV))
+    assert torch.equal(real, padded[:B]) and not padded[B:].float().abs().sum().item()
 
 
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(12, 2, 128, 16), (6, 3, 32, 8), (5, 5, 48, 16), (4, 1, 16, 16)])
