@@ -983,22 +983,27 @@ __global__ __launch_bounds__(256) void pf_merge_kernel(const float* __restrict__
 // decode: one query token per sequence, the G heads of a kv group as the 32 columns
 // ---------------------------------------------------------------------------
 // partial results per (sequence, query head, split): o [D] unnormalised, then m and l
+// CUT: the workgroup's keys come from the step's cut into pieces of one length (plan), not from a split of its own sequence
+template <bool CUT>
 __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(const bf16_t* __restrict__ q, int q_stride,
                                                      const bf16_t* __restrict__ k_cache,
                                                      const bf16_t* __restrict__ v_cache,
                                                      const int* __restrict__ block_table, int max_pages,
                                                      const int* __restrict__ context_lens,
                                                      float* __restrict__ part, int nsplit, int nq, int nkv, int P,
-                                                     int num_pages, float scale, int reach, const int4* __restrict__ plan) {
+                                                     int num_pages, float scale, int reach, const int4* __restrict__ plan,
+                                                     int num_seqs) {
   __shared__ Tiles tiles;
   const int g = blockIdx.y;
   const int G = nq / nkv;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   int b, ctx, k_begin, k_end;
   size_t part_slot;                 // this workgroup's place among the partial results, counted in (query heads) rows
-  if (plan != nullptr) {            // splits of equal length over all sequences (decode_plan_kernel): grid x is the split
+  if (CUT) {                        // pieces of one length over all sequences (decode_plan_kernel): grid x is the piece
     const int4 mine = plan[blockIdx.x];
-    if (mine.x < 0) return;
+    // an empty slot; or not a piece of a sequence of this step (a cut that was never written): nothing is read through it
+    if (mine.x < 0 || mine.x >= num_seqs || mine.y < 0 || mine.y >= mine.z || mine.z > mine.w ||
+        mine.w > (long long)max_pages * P) return;
     b = mine.x, k_begin = mine.y, k_end = mine.z, ctx = mine.w;
     part_slot = (size_t)blockIdx.x * nq;
   } else {                          // every sequence in nsplit splits of its own
@@ -1010,7 +1015,7 @@ __global__ __launch_bounds__(256, PICO_ATTN_WAVES_PER_SIMD) void decode_kernel(c
     k_begin = lo_tile + (int)blockIdx.z * per, k_end = min(ctx, k_begin + per);
     part_slot = (size_t)b * nq * nsplit + blockIdx.z;
   }
-  const size_t part_stride = plan != nullptr ? 1 : nsplit;      // rows of the partial results between two heads
+  const size_t part_stride = CUT ? 1 : nsplit;                  // rows of the partial results between two heads
   // the query sits at position ctx - 1 and sees keys lo .. ctx - 1; the splits share them from the tile that holds lo on
   const int lo = max(0, ctx - reach);
   const int* bt = block_table + (size_t)b * max_pages;
@@ -1088,13 +1093,15 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int KS16 = D / 32;   // contraction steps of a 16-key tile
 constexpr int DT16 = D / 16;   // 16-wide tiles of the output's head dimension
 
+template <bool CUT>
 __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restrict__ q, int q_stride,
                                                           const bf16_t* __restrict__ k_cache,
                                                           const bf16_t* __restrict__ v_cache,
                                                           const int* __restrict__ block_table, int max_pages,
                                                           const int* __restrict__ context_lens,
                                                           float* __restrict__ part, int nsplit, int nq, int nkv, int P,
-                                                          int num_pages, float scale, int reach, const int4* __restrict__ plan) {
+                                                          int num_pages, float scale, int reach, const int4* __restrict__ plan,
+                                                          int num_seqs) {
   __shared__ float xo[3][D][16];     // outputs of waves 1..3 for the final merge
   __shared__ float xml[3][2][16];
   const int g = blockIdx.y;
@@ -1102,9 +1109,11 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 15, kq = lane >> 4;
   int b, ctx, k_begin, k_end;
   size_t part_slot;                 // this workgroup's place among the partial results, counted in (query heads) rows
-  if (plan != nullptr) {            // splits of equal length over all sequences (decode_plan_kernel): grid x is the split
+  if (CUT) {                        // pieces of one length over all sequences (decode_plan_kernel): grid x is the piece
     const int4 mine = plan[blockIdx.x];
-    if (mine.x < 0) return;
+    // an empty slot; or not a piece of a sequence of this step (a cut that was never written): nothing is read through it
+    if (mine.x < 0 || mine.x >= num_seqs || mine.y < 0 || mine.y >= mine.z || mine.z > mine.w ||
+        mine.w > (long long)max_pages * P) return;
     b = mine.x, k_begin = mine.y, k_end = mine.z, ctx = mine.w;
     part_slot = (size_t)blockIdx.x * nq;
   } else {                          // every sequence in nsplit splits of its own
@@ -1115,7 +1124,7 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
     k_begin = lo_block + (int)blockIdx.z * per, k_end = min(ctx, k_begin + per);
     part_slot = (size_t)b * nq * nsplit + blockIdx.z;
   }
-  const size_t part_stride = plan != nullptr ? 1 : nsplit;      // rows of the partial results between two heads
+  const size_t part_stride = CUT ? 1 : nsplit;                  // rows of the partial results between two heads
   // the query sits at position ctx - 1 and sees keys lo .. ctx - 1; the splits share them from the block that holds lo on
   const int lo = max(0, ctx - reach);
   const int* bt = block_table + (size_t)b * max_pages;
@@ -1275,19 +1284,21 @@ __global__ __launch_bounds__(256, 2) void decode16_kernel(const bf16_t* __restri
 constexpr int MERGE_MAX_SPLITS = 256;
 // rows (with splits of equal length over all sequences): (first split, number of splits) of every sequence; the partial
 // results of a split's heads then lie together, nq rows apart from split to split.
+template <bool CUT>
 __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restrict__ part, int nsplit,
-                                                           bf16_t* __restrict__ out, int nq, const int2* __restrict__ rows) {
+                                                           bf16_t* __restrict__ out, int nq, const int2* __restrict__ rows,
+                                                           int slots) {
   constexpr int DPL = (D + 63) / 64;                        // head dimensions per lane
   constexpr int CH = MERGE_MAX_SPLITS / 64;
   __shared__ float quarter[3][DPL * 64];
   const int b = blockIdx.x, head = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float* p = part + ((size_t)b * nq + head) * nsplit * (D + 2);
-  size_t step = D + 2;                                      // floats from one split of this head to the next
-  if (rows != nullptr) {
-    const int2 mine = rows[b];
+  const size_t step = CUT ? (size_t)nq * (D + 2) : D + 2;   // floats from one split of this head to the next
+  if (CUT) {
+    int2 mine = rows[b];
+    if (mine.x < 0 || mine.y < 0 || mine.y > MERGE_MAX_SPLITS || mine.x + mine.y > slots) mine = make_int2(0, 0);   // never written
     nsplit = mine.y;
     p = part + ((size_t)mine.x * nq + head) * (D + 2);
-    step = (size_t)nq * (D + 2);
   }
   float m[CH], l[CH], wt[CH];
   float mx = -INFINITY;
@@ -1359,26 +1370,25 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float* __restri
 // depends on the contexts of the step alone (rows without a context, the padding of a recorded step, count for
 // nothing), so a sequence is cut alike whether the step is recorded and padded or not.
 // plan[slot] = (sequence, first key, end, context) or (-1, ..) for a slot that stays empty; rows[b] = (first slot, slots).
-// One workgroup; at most PLAN_MAX_ROWS sequences.
+// At most PLAN_MAX_ROWS sequences.
 constexpr int PLAN_MAX_ROWS = 1024;
-__global__ __launch_bounds__(256) void decode_plan_kernel(const int* __restrict__ context_lens, int num_seqs, int slots,
-                                                          int reach, int unit, int4* __restrict__ plan, int2* __restrict__ rows) {
+__device__ __forceinline__ int plan_wave_sum(int v) {
+#pragma unroll
+  for (int w = 32; w >= 1; w >>= 1) v += __shfl_xor(v, w, 64);
+  return v;
+}
+__device__ __forceinline__ int plan_wave_max(int v) {
+#pragma unroll
+  for (int w = 32; w >= 1; w >>= 1) v = max(v, __shfl_xor(v, w, 64));
+  return v;
+}
+// One wave: its sums and maxima need no barrier, and the search below is a dozen of them.
+__global__ __launch_bounds__(64) void decode_plan_kernel(const int* __restrict__ context_lens, int num_seqs, int slots,
+                                                         int reach, int unit, int4* __restrict__ plan, int2* __restrict__ rows) {
   __shared__ int len[PLAN_MAX_ROWS], low[PLAN_MAX_ROWS], first[PLAN_MAX_ROWS + 1];
-  __shared__ int red[256];
-  __shared__ int piece;
-  auto block_reduce = [&](int v, bool take_max) {
-    red[threadIdx.x] = v;
-    __syncthreads();
-    for (int w = 128; w >= 1; w >>= 1) {
-      if ((int)threadIdx.x < w) red[threadIdx.x] = take_max ? max(red[threadIdx.x], red[threadIdx.x + w]) : red[threadIdx.x] + red[threadIdx.x + w];
-      __syncthreads();
-    }
-    const int r = red[0];
-    __syncthreads();
-    return r;
-  };
+  const int lane = threadIdx.x;
   int my_sum = 0, my_max = 0;
-  for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) {
+  for (int b = lane; b < num_seqs; b += 64) {
     const int ctx = context_lens[b];
     const int lo = max(0, ctx - reach) / unit * unit;        // the splits share the keys from the unit that holds the first visible one on
     low[b] = lo;
@@ -1386,36 +1396,41 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(const int* __restrict_
     my_sum += (len[b] + unit - 1) / unit;                    // counted in units, so the sums stay small
     my_max = max(my_max, len[b]);
   }
-  const int total_units = block_reduce(my_sum, false), longest = block_reduce(my_max, true);
+  const int total_units = plan_wave_sum(my_sum), longest = plan_wave_max(my_max);
   // the smallest T = t units with sum over b of ceil(len_b / T) <= slots: t lies between what fills every slot exactly and
   // one piece a sequence (which fits: the launch has a slot for every sequence)
   int t_lo = max(1, max((total_units + slots - 1) / slots, ((longest + MERGE_MAX_SPLITS - 1) / MERGE_MAX_SPLITS + unit - 1) / unit));
   int t_hi = max(t_lo, (longest + unit - 1) / unit);
-  while (t_lo < t_hi) {                                       // the same for all threads
+  while (t_lo < t_hi) {                                       // the same for all lanes
     const int mid = (t_lo + t_hi) / 2, T = mid * unit;
     int mine = 0;
-    for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) mine += (len[b] + T - 1) / T;
-    if (block_reduce(mine, false) <= slots) t_hi = mid;
+    for (int b = lane; b < num_seqs; b += 64) mine += (len[b] + T - 1) / T;
+    if (plan_wave_sum(mine) <= slots) t_hi = mid;
     else t_lo = mid + 1;
   }
-  if (threadIdx.x == 0) {
-    const int T = t_lo * unit;
-    piece = T;
-    int n = 0;
-    for (int b = 0; b < num_seqs; b++) {
-      first[b] = n;
-      n += (len[b] + T - 1) / T;
+  const int T = t_lo * unit;
+  // first[b]: the pieces of the sequences before b; 64 sequences a turn, a prefix sum over the lanes
+  int base = 0;
+  for (int b0 = 0; b0 < num_seqs; b0 += 64) {
+    const int b = b0 + lane;
+    const int count = b < num_seqs ? (len[b] + T - 1) / T : 0;
+    int incl = count;
+#pragma unroll
+    for (int w = 1; w < 64; w <<= 1) {
+      const int up = __shfl_up(incl, w, 64);
+      if (lane >= w) incl += up;
     }
-    first[num_seqs] = n;
+    if (b < num_seqs) first[b] = base + incl - count;
+    base += __shfl(incl, 63, 64);
   }
+  if (lane == 0) first[num_seqs] = base;
   __syncthreads();
-  const int T = piece;
-  for (int b = threadIdx.x; b < num_seqs; b += blockDim.x) {
+  for (int b = lane; b < num_seqs; b += 64) {
     const int count = first[b + 1] - first[b], ctx = low[b] + len[b];
     rows[b] = make_int2(first[b], count);
     for (int i = 0; i < count; i++) plan[first[b] + i] = make_int4(b, low[b] + i * T, min(ctx, low[b] + (i + 1) * T), ctx);
   }
-  for (int e = first[num_seqs] + threadIdx.x; e < slots; e += blockDim.x) plan[e] = make_int4(-1, 0, 0, 0);
+  for (int e = first[num_seqs] + lane; e < slots; e += 64) plan[e] = make_int4(-1, 0, 0, 0);
 }
 
 static int check_common(const char* who, int nq, int nkv, int d, int P, int max_pages, int num_pages, int q_stride) {
@@ -1541,25 +1556,29 @@ extern "C" int pico_attn_decode(const void* q, int q_stride, const void* k_cache
     cut = reinterpret_cast<const int4*>(plan);
     rows = reinterpret_cast<const int2*>(plan + 4 * (size_t)plan_slots);
     if (plan_build) {
-      decode_plan_kernel<<<1, 256, 0, stream>>>(context_lens, num_seqs, plan_slots, reach, direct ? 32 : BN,
+      decode_plan_kernel<<<1, 64, 0, stream>>>(context_lens, num_seqs, plan_slots, reach, direct ? 32 : BN,
                                                 reinterpret_cast<int4*>(plan), reinterpret_cast<int2*>(plan + 4 * (size_t)plan_slots));
       PICO_LAUNCH_CHECK();
     }
     grid = dim3(plan_slots, nkv, 1);
   }
+#define DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, context_lens, \
+                    part, nsplit, nq, nkv, P, num_pages, scale, reach, cut, num_seqs
 #if PICO_HEAD_DIM % 32 == 0 && PICO_HEAD_DIM <= 128
-  if (direct)
-    decode16_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-                                             (const bf16_t*)v_cache, block_table, max_pages, context_lens, part,
-                                             nsplit, nq, nkv, P, num_pages, scale, reach, cut);
+  if (direct) {
+    if (cut != nullptr) decode16_kernel<true><<<grid, 256, 0, stream>>>(DECODE_ARGS);
+    else decode16_kernel<false><<<grid, 256, 0, stream>>>(DECODE_ARGS);
+  }
 #endif
-  if (!direct)
-    decode_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
-                                           block_table, max_pages, context_lens, part, nsplit, nq, nkv, P, num_pages,
-                                           scale, reach, cut);
+  if (!direct) {
+    if (cut != nullptr) decode_kernel<true><<<grid, 256, 0, stream>>>(DECODE_ARGS);
+    else decode_kernel<false><<<grid, 256, 0, stream>>>(DECODE_ARGS);
+  }
+#undef DECODE_ARGS
   PICO_LAUNCH_CHECK();
   dim3 mgrid(num_seqs, nq);
-  decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq, rows);
+  if (rows != nullptr) decode_merge_kernel<true><<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq, rows, plan_slots);
+  else decode_merge_kernel<false><<<mgrid, 256, 0, stream>>>(part, nsplit, (bf16_t*)out, nq, rows, plan_slots);
   PICO_LAUNCH_CHECK();
   return 0;
 }

@@ -694,6 +694,12 @@ def test_fast_decode_with_the_contexts_cut_into_pieces_of_one_length(K, nq, nkv,
     real = fa.decode(q[:B], kc, vc, bt, ctxl[:B], B, d ** -0.5, nsplit, cut=fa.decode_cut(B, nsplit, DEV))
     padded = fa.decode(q, kc, vc, bt16, ctxl, B + 3, d ** -0.5, nsplit, cut=fa.decode_cut(B + 3, nsplit, DEV))
     assert torch.equal(real, padded[:B]) and not padded[B:].float().abs().sum().item()
+    # a cut that was never written names no piece of this step: nothing is read through it, every row comes out empty
+    plan, slots = fa.decode_cut(B, nsplit, DEV)
+    for junk in (1 << 30, -7):
+        plan.fill_(junk)
+        out = fa.decode(q[:B], kc, vc, bt, ctxl[:B], B, d ** -0.5, nsplit, cut=(plan, slots), cut_build=False)
+        assert not out.float().abs().sum().item()
 
 
 @pytest.mark.parametrize("nq,nkv,d,Pg", [(12, 2, 128, 16), (6, 3, 32, 8), (5, 5, 48, 16), (4, 1, 16, 16)])
