@@ -709,6 +709,8 @@ __global__ __launch_bounds__(256 * KT, (KT == 2 || NQB == 2) ? 2 : 3) void prefi
     if (e < 0) return;
     b = e >> 16;
     tile = e & 0xffff;
+    // not a tile of a sequence of this step (a list that was never written): nothing is read through it
+    if (b >= num_seqs || tile * BMQ >= cu_seqlens[b + 1] - cu_seqlens[b]) return;
   } else {                      // sequence by sequence, each from its last (longest) tile down
     for (; b < num_seqs; b++) {
       ntiles = (cu_seqlens[b + 1] - cu_seqlens[b] + BMQ - 1) / BMQ;
