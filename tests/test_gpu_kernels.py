@@ -656,16 +656,16 @@ def test_fast_prefill_whole_key_tiles_at_every_head_size_and_page_size(K, d, Pg)
 @pytest.mark.parametrize("window", [0, 100])
 @pytest.mark.parametrize("nq,nkv,d,Pg,nsplit", [(12, 2, 128, 16, 8), (6, 3, 32, 8, 2), (5, 5, 48, 16, 3), (4, 1, 256, 32, 4), (8, 2, 96, 16, 16)])
 def test_fast_decode_with_the_contexts_cut_into_pieces_of_one_length(K, nq, nkv, d, Pg, nsplit, window):
-    # from 16 sequences on the contexts of a decode step are cut into pieces of one length over all sequences (the pieces of
+    # from 17 sequences on (32, counted as a recorded step is padded) the contexts of a decode step are cut into pieces of one length over all sequences (the pieces of
     # a long context are as long as a short context's): the cut covers every sequence's keys once, in order, in whole units
-    # of 32 keys (of an LDS tile where the kernel stages tiles), in no more pieces than nsplit splits of 16 sequences
+    # of 32 keys (of an LDS tile where the kernel stages tiles), in no more pieces than nsplit splits of 32 sequences
     # would be and with the smallest length that allows that; the attention is the plain one; and sequences without a context
     # behind the others (the padding of a recorded step) change no bit of the others
     from pico_vllm_amd.ops.attention_fast import FastAttention
     def boost(qs, ks, vs):
         for q in qs:
             q *= 2.0
-    prefix_lens = [3000, 17, 0, 1000, 64, 129, 2047, 5, 700, 31, 32, 33, 1500]
+    prefix_lens = [3000, 17, 0, 1000, 64, 129, 2047, 5, 700, 31, 32, 33, 1500, 95, 96, 2, 260, 511, 4100, 1]
     new_lens = [1] * len(prefix_lens)
     cut = []
     out, want = _fast_case(new_lens, prefix_lens, nq, nkv, d, Pg, seed=nsplit + window, boost=boost, decode=True, nsplit=nsplit,
@@ -673,7 +673,7 @@ def test_fast_decode_with_the_contexts_cut_into_pieces_of_one_length(K, nq, nkv,
     close(out, want, torch.bfloat16)
     plan, slots = cut[0]
     B = len(prefix_lens)
-    assert slots == 16 * nsplit
+    assert slots == 32 * nsplit
     pieces = plan[:4 * slots].reshape(slots, 4).cpu().tolist()
     rows = plan[4 * slots:4 * slots + 2 * B].reshape(B, 2).cpu().tolist()
     unit = 32 if (d % 32 == 0 and d <= 128 and nq // nkv <= 16) else (64 if d <= 128 else 32)
