@@ -61,10 +61,10 @@ class FastAttention:
 
     def decode_cut(self, num_seqs: int, nsplit: int, device) -> Optional[tuple]:
         """Room for the cut of a decode step's contexts into pieces of one length over all sequences (``decode(cut=...)``),
-        or None where every sequence keeps ``nsplit`` splits of its own: few sequences (unequal contexts cost nothing
-        there: 15.3 against 14.9 us at 8 sequences, 16.1 against 16.1 at 16, but 22.6 against 18.2 at 32 and 35 against 27 at 64,
-        while the cut's indirection costs a layer about 1 us) or a single split.  The pieces fill the
-        workgroups that ``nsplit`` splits of the padded number of sequences would."""
+        or None where every sequence keeps ``nsplit`` splits of its own: few sequences (unequal contexts cost
+        nothing there: 15.3 against 14.9 us at 8 sequences, 16.1 against 16.1 at 16, but 22.6 against 18.2 at 32 and
+        35 against 27 at 64, while the cut's indirection costs a layer about 1 us) or a single split.  The pieces
+        fill the workgroups that ``nsplit`` splits of the padded number of sequences would."""
         padded = self.padded(num_seqs)
         if nsplit < 2 or padded < self.CUT_FROM or num_seqs > 1024:
             return None
