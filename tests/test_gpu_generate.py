@@ -115,6 +115,28 @@ def test_decode_steps_replayed_from_a_graph_give_the_same_tokens(dtype):
     check_greedy("A", dtype, prompts[:2], more)
 
 
+def test_decode_steps_of_many_unequal_requests_cut_their_contexts_alike_recorded_or_not(monkeypatch):
+    # 21 requests (a recorded step of them is padded to 32) with prompts of 3 to 120 tokens: their decode steps cut the
+    # contexts of all sequences into pieces of one length; recorded and padded or not, the same tokens in bfloat16
+    # (that the logits of such steps are the plain implementation's within rounding: test_gpu_replay.py)
+    from pico_vllm_amd import SamplingParams
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    cuts = []
+    real = FastAttention.decode_cut
+    monkeypatch.setattr(FastAttention, "decode_cut", lambda self, n, ns, dev: cuts.append((n, ns, real(self, n, ns, dev))) or cuts[-1][2])
+    lengths = [3, 120, 17, 64, 5, 99, 33, 2, 80, 47, 111, 9, 65, 28, 1, 73, 16, 104, 55, 12, 90]
+    prompts = prompts_for("B", lengths, seed=21)
+    sp = SamplingParams(max_new_tokens=25, temperature=0.0, ignore_eos=True)
+    kw = dict(num_gpu_blocks=21 * 20 + 8, max_num_seqs=21, max_num_batched_tokens=512, max_seq_len=192)
+    eager = llm("B", "bfloat16", **kw).generate(prompts, sp)
+    assert any(c is not None and n == 21 for n, _, c in cuts), "no decode step cut its contexts over all sequences"
+    cuts.clear()
+    graph_llm = llm("B", "bfloat16", use_cuda_graph=True, max_batch_size=32, **kw)
+    graphed = graph_llm.generate(prompts, sp)
+    assert 32 in graph_llm.engine.runner._graphs and any(c is not None and n == 32 for n, _, c in cuts)
+    assert [o.token_ids for o in graphed] == [o.token_ids for o in eager]
+
+
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
 def test_steps_of_decoding_requests_and_a_prompt_portion_replayed_from_graphs_give_the_same_tokens(name, dtype):
     # a small token budget: while prompts are still coming in, most steps are a few decoding requests and one portion of a

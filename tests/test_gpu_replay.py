@@ -343,6 +343,36 @@ def test_a_context_of_thousands_of_tokens_in_portions_of_2048(monkeypatch):
         del _plain_cache[key]
 
 
+@pytest.mark.parametrize("name", ["B", "C", "E"])
+def test_twenty_requests_decoding_at_once(name, monkeypatch):
+    # 20 requests of 33 to 200 tokens live at once, their last 32 tokens one by one in steps of 20 single tokens: from 17
+    # sequences on a decode step cuts the contexts of all of them into pieces of one length (head sizes 32 and 96: the
+    # kernel that reads the pages directly; 48: the one that stages tiles); the logits are the plain implementation's
+    # within rounding, as with four live requests
+    from pico_vllm_amd.engine.replay import TraceReplayer
+    from pico_vllm_amd.ops.attention_fast import FastAttention
+    cuts = []
+    real = FastAttention.decode_cut
+    monkeypatch.setattr(FastAttention, "decode_cut", lambda self, n, ns, dev: cuts.append(real(self, n, ns, dev)) or cuts[-1])
+    lengths = [40, 150, 65, 97, 33, 180, 70, 129, 45, 200, 64, 90, 36, 160, 110, 50, 77, 140, 34, 100]
+    reqs = make_requests(name, lengths, seed=9)
+    tail = 32
+    t = Trace()
+    t.add([(rid, toks[:len(toks) - tail], range(len(toks) - tail)) for rid, toks in reqs.items()])
+    for i in range(tail):
+        t.add([(rid, toks[len(toks) - tail + i:len(toks) - tail + i + 1], [0]) for rid, toks in reqs.items()],
+              end=list(reqs) if i == tail - 1 else [])
+    rp = TraceReplayer(model_dir(name), "bfloat16", t.live_peak, PAGE_SIZE[name], max_live=24)
+    got = {}
+    for step in t.steps:
+        out = rp.run_step(step)
+        for row, key in zip(out, t.rows[step["step"]]):
+            got[key] = row
+    rp.runner.manager.check()
+    assert sum(c is not None for c in cuts) >= tail, "the decode steps did not cut their contexts over all sequences"
+    compare(name, "bfloat16", reqs, got, "twenty at once")
+
+
 def test_forty_more_drawn_configurations_in_every_way_of_cutting():
     # a sweep over sizes nobody looked at, in both precisions, whole, with the tail token by token and mixed in a
     # small pool; it stops at the first configuration that fails and names it
